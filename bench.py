@@ -1,0 +1,214 @@
+#!/usr/bin/env python3
+"""Benchmark of the causal linear-attention product on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg2|cfg3|cfg5|cfg4op]
+
+A step is one forward + backward of ``causal_dot_product`` over one batch of synthetic input,
+called through the C ABI with outputs and workspace pre-allocated and every input already in
+HBM.  The default workload is the configuration the metric is quoted on:
+N=10, H=8, L=1000, E=M=64, fp32.  Steps rotate over several input sets (> 512 MB in total) so
+that the 256 MB Infinity Cache cannot serve a step from the previous one.
+
+Prints ONE JSON line.  ``value`` is N*L / t(fwd+bwd) in Mtokens/s.  ``roofline`` covers the
+backward launch sequence (the dominant part of a step) against HBM: algorithmic bytes are
+4*(4E+3M) per (n,h,l) position for fp32 (read Q,K,V,G, write dQ,dK,dV), timed with events on
+the stream the kernels are launched on.  ``cpu_baseline`` times the reference's own CPU
+extension (or, when it is not built, its C restatement) on this box's host cores over a
+bounded number of calls of the same workload.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for p in (ROOT, os.path.join(ROOT, "fast-transformers_amd")):
+    if p not in sys.path:
+        sys.path.insert(0, p)
+
+HBM_PEAK_GBPS = 8000.0          # MI355X HBM3E, published
+MFMA_FP32_PEAK_TFLOPS = 157.3   # MI355X dense fp32 matrix, published
+
+WORKLOADS = {
+    # name: (N, H, L, E, M, dtype, seed)
+    "cfg2": (10, 8, 1000, 64, 64, "f32", 2),
+    "cfg3": (1, 16, 65536, 64, 64, "f32", 3),
+    "cfg4op": (10, 8, 4096, 64, 64, "f32", 4),
+    "cfg5": (4, 32, 16384, 32, 128, "bf16", 5),
+}
+
+
+def alg_bytes_per_position(E, M, dtype):
+    """(forward, backward) algorithmic bytes per (n,h,l) position."""
+    if dtype == "f32":
+        return 4 * (2 * E + 2 * M), 4 * (4 * E + 3 * M)
+    # bf16 Q,K,V and their gradients; product and upstream gradient fp32
+    return 2 * (2 * E + M) + 4 * M, 2 * (2 * E + M) + 4 * M + 2 * (2 * E + M)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--workload", default="cfg2", choices=sorted(WORKLOADS))
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--sets", type=int, default=0, help="input sets to rotate over (0 = auto)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on ONE GPU (the path shards over N*H with no "
+              "communication; no multi-GPU figure is produced). Use --gpus 1.", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from fast_transformers_amd import _native
+    from fast_transformers_amd.causal_product import causal_dot_product_hip, \
+        causal_dot_backward_hip
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    _native.load()
+    torch.cuda.set_device(0)
+    dev = torch.device("cuda:0")
+
+    N, H, L, E, M, dtype, seed = WORKLOADS[args.workload]
+    tdtype = torch.float32 if dtype == "f32" else torch.bfloat16
+    esz = 4 if dtype == "f32" else 2
+    set_bytes = N * H * L * ((2 * E + M) * esz * 2 + 2 * M * 4)
+    nsets = args.sets or max(1, min(8, -(-(768 << 20) // set_bytes)))
+
+    gen = torch.Generator(device="cpu").manual_seed(seed)
+    sets = []
+    for s in range(nsets):
+        if s == 0:
+            import torch.nn.functional as F
+            Q = F.elu(torch.randn(N, H, L, E, generator=gen)) + 1
+            K = F.elu(torch.randn(N, H, L, E, generator=gen)) + 1
+            V = torch.randn(N, H, L, M, generator=gen)
+            G = torch.randn(N, H, L, M, generator=gen)
+            base = [Q.to(tdtype).to(dev), K.to(tdtype).to(dev), V.to(tdtype).to(dev), G.to(dev)]
+            ins = base
+        else:
+            # further sets: same distribution, decorrelated by a roll along L (device-side)
+            ins = [torch.roll(t, shifts=17 * s, dims=2).contiguous() for t in base]
+        outs = [torch.empty(N, H, L, M, device=dev, dtype=torch.float32),
+                torch.empty(N, H, L, E, device=dev, dtype=tdtype),
+                torch.empty(N, H, L, E, device=dev, dtype=tdtype),
+                torch.empty(N, H, L, M, device=dev, dtype=tdtype)]
+        sets.append((ins, outs))
+
+    def step(i):
+        (q, k, v, g), (o, dq, dk, dv) = sets[i % nsets]
+        causal_dot_product_hip(q, k, v, o)
+        causal_dot_backward_hip(q, k, v, g, dq, dk, dv)
+
+    for i in range(args.warmup):
+        step(i)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        step(i)
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    ms_per_step = (t1 - t0) * 1e3 / args.steps
+
+    # per-direction device time with events on the launch stream
+    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(args.steps)]
+    for i in range(args.steps):
+        (q, k, v, g), (o, dq, dk, dv) = sets[i % nsets]
+        ev[i][0].record()
+        causal_dot_product_hip(q, k, v, o)
+        ev[i][1].record()
+        causal_dot_backward_hip(q, k, v, g, dq, dk, dv)
+        ev[i][2].record()
+    torch.cuda.synchronize()
+    fwd_ms = sorted(e[0].elapsed_time(e[1]) for e in ev)
+    bwd_ms = sorted(e[1].elapsed_time(e[2]) for e in ev)
+    fwd_avg, bwd_avg = sum(fwd_ms) / len(fwd_ms), sum(bwd_ms) / len(bwd_ms)
+
+    TH = N * H * L
+    fb, bb = alg_bytes_per_position(E, M, dtype)
+    bwd_gbps = bb * TH / (bwd_avg * 1e-3) / 1e9
+    fwd_gbps = fb * TH / (fwd_avg * 1e-3) / 1e9
+    value = N * L / (ms_per_step * 1e-3) / 1e6
+
+    result = {
+        "metric": "causal_dot_product fwd+bwd Mtokens/s (H=8,E=M=64); % of HBM/MFMA roofline",
+        "value": round(value, 3),
+        "unit": "Mtokens/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 5),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32" if dtype == "f32" else "bf16 in / f32 accumulate",
+        "data": "synthetic",
+        "config": {"workload": "%s: causal_dot_product fwd+bwd N=%d H=%d L=%d E=%d M=%d %s"
+                               % (args.workload, N, H, L, E, M, dtype),
+                   "input_sets_rotated": nsets,
+                   "token_heads_per_s": round(TH / (ms_per_step * 1e-3), 1),
+                   "fwd_ms_avg": round(fwd_avg, 5), "fwd_ms_min": round(fwd_ms[0], 5),
+                   "bwd_ms_avg": round(bwd_avg, 5), "bwd_ms_min": round(bwd_ms[0], 5),
+                   "fwd_alg_GBps": round(fwd_gbps, 1),
+                   "fwdbwd_alg_GBps": round((fb + bb) * TH / (ms_per_step * 1e-3) / 1e9, 1),
+                   "fwdbwd_alg_TFLOPs": round(14 * E * M * TH / (ms_per_step * 1e-3) / 1e12, 2),
+                   "fwdbwd_frac_of_hbm_roofline":
+                       round((fb + bb) * TH / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)},
+        "roofline": {"bound": "hbm", "kernel": "backward launch sequence",
+                     "achieved": round(bwd_gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": round(bwd_gbps / HBM_PEAK_GBPS, 4), "traffic": None},
+    }
+
+    if not args.no_cpu:
+        result["cpu_baseline"] = cpu_baseline(N, H, L, E, M, seed, args.workload)
+    print(json.dumps(result))
+
+
+def cpu_baseline(N, H, L, E, M, seed, workload):
+    """The reference's CPU extension (oracle/_ref) or its restatement, fwd+bwd, fp32, timed
+    the way the reference's benchmark does (warm-up calls, then timed calls, wall clock;
+    tests/causal_product/test_causal_product_cpu.py:87-99)."""
+    import torch
+    import oracle
+    Q, K, V, G = oracle.make_inputs(N, H, L, E, M, seed)
+    out = torch.empty(N, H, L, M)
+    gq, gk, gv = torch.empty_like(Q), torch.empty_like(K), torch.empty_like(V)
+    if oracle.reference_extension_available():
+        ref = oracle.load_reference_extension()
+        fwd, bwd, kind = ref.causal_dot_product, ref.causal_dot_backward, "reference"
+    else:
+        fwd, bwd, kind = oracle.causal_dot_product, oracle.causal_dot_backward, "port"
+
+    def call():
+        fwd(Q, K, V, out)
+        bwd(Q, K, V, G, gq, gk, gv)
+
+    t = time.perf_counter()
+    call()
+    one = time.perf_counter() - t
+    warm = 10 if one < 0.5 else 1
+    timed = 10 if one < 0.5 else (3 if one < 5 else 1)
+    for _ in range(warm):
+        call()
+    t = time.perf_counter()
+    for _ in range(timed):
+        call()
+    dt = (time.perf_counter() - t) / timed
+    threads = torch.get_num_threads()
+    try:
+        threads = int(os.environ.get("OMP_NUM_THREADS", "")) or threads
+    except ValueError:
+        pass
+    return {"value": round(N * L / dt / 1e6, 4), "unit": "Mtokens/s",
+            "cores": min(threads, N * H), "kind": kind,
+            "sample": "%s fwd+bwd fp32, %d warm-up + %d timed calls, %.1f ms per call; "
+                      "OpenMP over N*H=%d chains, host cpu_count=%d"
+                      % (workload, warm, timed, dt * 1e3, N * H, os.cpu_count())}
+
+
+if __name__ == "__main__":
+    main()

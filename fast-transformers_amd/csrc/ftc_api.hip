@@ -1,0 +1,162 @@
+// C ABI entry points (include/ftc_causal_product.h): argument checking and dispatch.
+//
+// The four result tensors are all instances of one scan primitive under a change of
+// operand roles (the reference's CUDA path uses the same identity,
+// causal_product_cuda.cu:1119-1187):
+//
+//   product = scan_fwd(a=Q, b=K, v=V)      state E x M
+//   dQ      = scan_fwd(a=G, b=V, v=K)      state M x E
+//   dK      = scan_rev(a=V, b=G, v=Q)      state M x E
+//   dV      = scan_rev(a=K, b=Q, v=G)      state E x M
+#include <stdarg.h>
+#include <stdio.h>
+
+#include <algorithm>
+
+#include "ftc_common.h"
+
+namespace ftc {
+
+static thread_local char g_error[512] = "";
+
+int fail(int code, const char *fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_error, sizeof(g_error), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+namespace {
+
+struct Dims {
+    int64_t N, H, L, E, M;
+};
+
+int check_tensor(const ftc_tensor4 *t, const char *name, int64_t N, int64_t H, int64_t L,
+                 int64_t X, int dtype_a, int dtype_b) {
+    if (!t) return fail(FTC_ERR_INVALID, "%s is null", name);
+    if (t->dtype != dtype_a && t->dtype != dtype_b)
+        return fail(FTC_ERR_INVALID, "%s has dtype code %d, which this argument does not accept",
+                    name, (int)t->dtype);
+    if (t->size[0] != N || t->size[1] != H || t->size[2] != L || t->size[3] != X)
+        return fail(FTC_ERR_INVALID, "%s has shape (%lld,%lld,%lld,%lld), expected (%lld,%lld,%lld,%lld)",
+                    name, (long long)t->size[0], (long long)t->size[1], (long long)t->size[2],
+                    (long long)t->size[3], (long long)N, (long long)H, (long long)L, (long long)X);
+    if (N * H * L * X > 0) {
+        if (!t->ptr) return fail(FTC_ERR_INVALID, "%s has a null data pointer", name);
+        if (X > 1 && t->stride[3] != 1)
+            return fail(FTC_ERR_INVALID, "%s must be contiguous in its last dimension (stride %lld)",
+                        name, (long long)t->stride[3]);
+    }
+    return FTC_OK;
+}
+
+int read_dims(const ftc_tensor4 *q, const ftc_tensor4 *v, Dims *d) {
+    if (!q || !v) return fail(FTC_ERR_INVALID, "queries or values is null");
+    d->N = q->size[0];
+    d->H = q->size[1];
+    d->L = q->size[2];
+    d->E = q->size[3];
+    d->M = v->size[3];
+    if (d->N < 0 || d->H < 0 || d->L < 0 || d->E < 0 || d->M < 0)
+        return fail(FTC_ERR_INVALID, "negative size");
+    if (q->dtype != FTC_F32 && q->dtype != FTC_BF16)
+        return fail(FTC_ERR_INVALID, "queries dtype code %d is neither FTC_F32 nor FTC_BF16",
+                    (int)q->dtype);
+    if (d->L > 0x7fffffffLL || d->N * d->H > 0x7fffffffLL)
+        return fail(FTC_ERR_UNSUPPORTED, "L and N*H must fit in 31 bits");
+    return FTC_OK;
+}
+
+}  // namespace
+}  // namespace ftc
+
+using namespace ftc;
+
+extern "C" {
+
+int ftc_version(void) { return 1000; }
+
+const char *ftc_last_error(void) { return g_error; }
+
+int64_t ftc_causal_dot_product_workspace_bytes(int64_t N, int64_t H, int64_t L, int64_t E,
+                                               int64_t M, int32_t dtype) {
+    if (N < 0 || H < 0 || L < 0 || E < 0 || M < 0) return fail(FTC_ERR_INVALID, "negative size");
+    if (dtype != FTC_F32 && dtype != FTC_BF16) return fail(FTC_ERR_INVALID, "unknown dtype");
+    if (N * H * L == 0 || M == 0 || E == 0) return 0;
+    if (E > kGenericMaxDim || M > kGenericMaxDim)
+        return fail(FTC_ERR_UNSUPPORTED, "E and M must be at most %d", kGenericMaxDim);
+    return generic_scan_workspace_bytes(N, H, L, E, M);
+}
+
+int ftc_causal_dot_product(const ftc_tensor4 *queries, const ftc_tensor4 *keys,
+                           const ftc_tensor4 *values, const ftc_tensor4 *product,
+                           void *workspace, size_t workspace_bytes, void *stream) {
+    Dims d;
+    int rc = read_dims(queries, values, &d);
+    if (rc) return rc;
+    const int dt = queries->dtype;
+    if ((rc = check_tensor(queries, "queries", d.N, d.H, d.L, d.E, dt, dt))) return rc;
+    if ((rc = check_tensor(keys, "keys", d.N, d.H, d.L, d.E, dt, dt))) return rc;
+    if ((rc = check_tensor(values, "values", d.N, d.H, d.L, d.M, dt, dt))) return rc;
+    if ((rc = check_tensor(product, "product", d.N, d.H, d.L, d.M, FTC_F32, FTC_F32))) return rc;
+    if (d.N * d.H * d.L * d.M == 0) return FTC_OK;
+    hipStream_t s = (hipStream_t)stream;
+    if (d.E == 0)  // an empty contraction: every product row is zero
+        return zero_rows(as_operand_out(product), d.N, d.H, d.L, s);
+    return generic_scan(as_operand(queries), as_operand(keys), as_operand(values),
+                        as_operand_out(product), d.N, d.H, d.L, false, workspace, workspace_bytes,
+                        s);
+}
+
+int64_t ftc_causal_dot_backward_workspace_bytes(int64_t N, int64_t H, int64_t L, int64_t E,
+                                                int64_t M, int32_t dtype) {
+    if (N < 0 || H < 0 || L < 0 || E < 0 || M < 0) return fail(FTC_ERR_INVALID, "negative size");
+    if (dtype != FTC_F32 && dtype != FTC_BF16) return fail(FTC_ERR_INVALID, "unknown dtype");
+    if (N * H * L == 0 || M == 0 || E == 0) return 0;
+    if (E > kGenericMaxDim || M > kGenericMaxDim)
+        return fail(FTC_ERR_UNSUPPORTED, "E and M must be at most %d", kGenericMaxDim);
+    return std::max(generic_scan_workspace_bytes(N, H, L, E, M),
+                    generic_scan_workspace_bytes(N, H, L, M, E));
+}
+
+int ftc_causal_dot_backward(const ftc_tensor4 *queries, const ftc_tensor4 *keys,
+                            const ftc_tensor4 *values, const ftc_tensor4 *grad_out,
+                            const ftc_tensor4 *grad_queries, const ftc_tensor4 *grad_keys,
+                            const ftc_tensor4 *grad_values, void *workspace,
+                            size_t workspace_bytes, void *stream) {
+    Dims d;
+    int rc = read_dims(queries, values, &d);
+    if (rc) return rc;
+    const int dt = queries->dtype;
+    if ((rc = check_tensor(queries, "queries", d.N, d.H, d.L, d.E, dt, dt))) return rc;
+    if ((rc = check_tensor(keys, "keys", d.N, d.H, d.L, d.E, dt, dt))) return rc;
+    if ((rc = check_tensor(values, "values", d.N, d.H, d.L, d.M, dt, dt))) return rc;
+    if ((rc = check_tensor(grad_out, "grad_out", d.N, d.H, d.L, d.M, FTC_F32, FTC_F32))) return rc;
+    if ((rc = check_tensor(grad_queries, "grad_queries", d.N, d.H, d.L, d.E, dt, dt))) return rc;
+    if ((rc = check_tensor(grad_keys, "grad_keys", d.N, d.H, d.L, d.E, dt, dt))) return rc;
+    if ((rc = check_tensor(grad_values, "grad_values", d.N, d.H, d.L, d.M, dt, dt))) return rc;
+    if (d.N * d.H * d.L == 0 || d.E == 0 || d.M == 0) {
+        // A zero row width: whichever gradient is non-empty is a sum over an empty index set.
+        const ftc_tensor4 *outs[3] = {grad_queries, grad_keys, grad_values};
+        for (const ftc_tensor4 *t : outs) {
+            if (t->size[0] * t->size[1] * t->size[2] * t->size[3] == 0) continue;
+            if ((rc = zero_rows(as_operand_out(t), d.N, d.H, d.L, (hipStream_t)stream))) return rc;
+        }
+        return FTC_OK;
+    }
+    hipStream_t s = (hipStream_t)stream;
+    const Operand Q = as_operand(queries), K = as_operand(keys), V = as_operand(values),
+                  G = as_operand(grad_out);
+    if ((rc = generic_scan(G, V, K, as_operand_out(grad_queries), d.N, d.H, d.L, false, workspace,
+                           workspace_bytes, s)))
+        return rc;
+    if ((rc = generic_scan(V, G, Q, as_operand_out(grad_keys), d.N, d.H, d.L, true, workspace,
+                           workspace_bytes, s)))
+        return rc;
+    return generic_scan(K, Q, G, as_operand_out(grad_values), d.N, d.H, d.L, true, workspace,
+                        workspace_bytes, s);
+}
+
+}  // extern "C"

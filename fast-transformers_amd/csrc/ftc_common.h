@@ -1,0 +1,79 @@
+// Shared declarations of the gfx950 causal-product library (internal; the public
+// surface is include/ftc_causal_product.h).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "ftc_causal_product.h"
+
+namespace ftc {
+
+// One operand of a scan: rows of `width` contiguous elements addressed by
+// (chain = n*H + h, position l).  Strides in elements.
+struct Operand {
+    const void *ptr;
+    int64_t stride_n, stride_h, stride_l;
+    int32_t dtype;  // ftc_dtype
+    int32_t width;  // elements per row
+};
+
+struct OperandOut {
+    void *ptr;
+    int64_t stride_n, stride_h, stride_l;
+    int32_t dtype;
+    int32_t width;
+};
+
+inline Operand as_operand(const ftc_tensor4 *t) {
+    return Operand{t->ptr, t->stride[0], t->stride[1], t->stride[2], t->dtype, (int32_t)t->size[3]};
+}
+inline OperandOut as_operand_out(const ftc_tensor4 *t) {
+    return OperandOut{t->ptr, t->stride[0], t->stride[1], t->stride[2], t->dtype,
+                      (int32_t)t->size[3]};
+}
+
+// Records the message returned by ftc_last_error() and returns `code`.
+int fail(int code, const char *fmt, ...);
+
+// bf16 <-> fp32 with round-to-nearest-even (finite inputs; NaN stays NaN).
+__device__ __forceinline__ float bf16_to_f32(uint16_t b) {
+    return __uint_as_float(((uint32_t)b) << 16);
+}
+__device__ __forceinline__ uint16_t f32_to_bf16(float f) {
+    uint32_t u = __float_as_uint(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40u);
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return (uint16_t)(u >> 16);
+}
+
+__device__ __forceinline__ float load_as_f32(const void *base, int32_t dtype, int64_t idx) {
+    return dtype == FTC_F32 ? ((const float *)base)[idx]
+                            : bf16_to_f32(((const uint16_t *)base)[idx]);
+}
+__device__ __forceinline__ void store_from_f32(void *base, int32_t dtype, int64_t idx, float x) {
+    if (dtype == FTC_F32)
+        ((float *)base)[idx] = x;
+    else
+        ((uint16_t *)base)[idx] = f32_to_bf16(x);
+}
+
+// ---------------------------------------------------------------------------
+// Generic scan (any D, F <= 512, any L): ftc_generic.hip
+//
+//   out[c, l, f] = sum_{j <= l} (a[c,l,:] . b[c,j,:]) * v[c,j,f]      (reverse: j >= l)
+//
+// a, b: rows of D elements; v, out: rows of F elements.
+// ---------------------------------------------------------------------------
+constexpr int kGenericMaxDim = 512;
+
+int64_t generic_scan_workspace_bytes(int64_t N, int64_t H, int64_t L, int64_t D, int64_t F);
+
+int generic_scan(const Operand &a, const Operand &b, const Operand &v, const OperandOut &out,
+                 int64_t N, int64_t H, int64_t L, bool reverse, void *workspace,
+                 size_t workspace_bytes, hipStream_t stream);
+
+// Fill every row of `out` with zeros (used for empty contractions).
+int zero_rows(const OperandOut &out, int64_t N, int64_t H, int64_t L, hipStream_t stream);
+
+}  // namespace ftc

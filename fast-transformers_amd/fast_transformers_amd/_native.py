@@ -1,0 +1,100 @@
+"""ctypes binding of ``libftc_causal.so`` (C ABI: ``include/ftc_causal_product.h``).
+
+No torch types cross the boundary: tensors are described by ``ftc_tensor4`` (device
+pointer, dtype code, sizes and strides in elements), the stream is a raw
+``hipStream_t`` and scratch memory is a raw device pointer the caller owns.
+
+There is no fallback: when the library is missing, ``load()`` raises.
+"""
+import ctypes
+import os
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libftc_causal.so")
+
+FTC_F32 = 0
+FTC_BF16 = 1
+_DTYPE_CODE = {torch.float32: FTC_F32, torch.bfloat16: FTC_BF16}
+
+EXPORTED_SYMBOLS = (
+    "ftc_version",
+    "ftc_last_error",
+    "ftc_causal_dot_product_workspace_bytes",
+    "ftc_causal_dot_product",
+    "ftc_causal_dot_backward_workspace_bytes",
+    "ftc_causal_dot_backward",
+)
+
+
+class Tensor4(ctypes.Structure):
+    _fields_ = [
+        ("ptr", ctypes.c_void_p),
+        ("dtype", ctypes.c_int32),
+        ("size", ctypes.c_int64 * 4),
+        ("stride", ctypes.c_int64 * 4),
+    ]
+
+
+_lib = None
+
+
+def load():
+    """Load the HIP library (once).  Raises if it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise RuntimeError(
+            "fast_transformers_amd: %s is missing; build it with "
+            "`python fast-transformers_amd/build.py` (there is no CPU or PyTorch fallback)"
+            % LIB_PATH)
+    lib = ctypes.CDLL(LIB_PATH)
+    t4 = ctypes.POINTER(Tensor4)
+    lib.ftc_version.restype = ctypes.c_int
+    lib.ftc_version.argtypes = []
+    lib.ftc_last_error.restype = ctypes.c_char_p
+    lib.ftc_last_error.argtypes = []
+    for name in ("ftc_causal_dot_product_workspace_bytes",
+                 "ftc_causal_dot_backward_workspace_bytes"):
+        f = getattr(lib, name)
+        f.restype = ctypes.c_int64
+        f.argtypes = [ctypes.c_int64] * 5 + [ctypes.c_int32]
+    lib.ftc_causal_dot_product.restype = ctypes.c_int
+    lib.ftc_causal_dot_product.argtypes = [t4] * 4 + [ctypes.c_void_p, ctypes.c_size_t,
+                                                      ctypes.c_void_p]
+    lib.ftc_causal_dot_backward.restype = ctypes.c_int
+    lib.ftc_causal_dot_backward.argtypes = [t4] * 7 + [ctypes.c_void_p, ctypes.c_size_t,
+                                                       ctypes.c_void_p]
+    _lib = lib
+    return lib
+
+
+def last_error():
+    return load().ftc_last_error().decode("utf-8", "replace")
+
+
+def check(rc, what):
+    if rc < 0:
+        raise RuntimeError("%s failed (status %d): %s" % (what, rc, last_error()))
+    return rc
+
+
+def dtype_code(dtype):
+    try:
+        return _DTYPE_CODE[dtype]
+    except KeyError:
+        raise RuntimeError("causal_dot_product: expected float32 or bfloat16 tensors, got %s"
+                           % dtype) from None
+
+
+def describe(t):
+    """``ftc_tensor4`` view of a 4-d device tensor (no copy)."""
+    d = Tensor4()
+    d.ptr = t.data_ptr() if t.numel() else None
+    d.dtype = dtype_code(t.dtype)
+    for i in range(4):
+        d.size[i] = t.shape[i]
+        d.stride[i] = t.stride(i)
+    return d

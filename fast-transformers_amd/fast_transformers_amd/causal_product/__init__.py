@@ -1,0 +1,150 @@
+"""``causal_dot_product`` on MI355X: same surface as the reference module
+``fast_transformers/causal_product/__init__.py``.
+
+* ``CausalDotProduct`` is a ``torch.autograd.Function`` with the class-level
+  dispatch tables ``dot`` / ``dot_backward`` keyed by ``device.type``
+  (reference ``__init__.py:23-30``).  ROCm PyTorch reports ``"cuda"`` for an AMD
+  GPU, so the HIP kernels register under that key.  There is no ``"cpu"`` entry:
+  this package ships the GPU path only and a CPU tensor raises ``KeyError`` the
+  way an unknown device type does in the reference (``__init__.py:44``).
+* The native functions keep the reference's in-place calling convention
+  (``causal_product_cpu.cpp:82-87,133-141``): ``causal_dot_product(Q, K, V,
+  product)`` and ``causal_dot_backward(Q, K, V, grad_out, grad_Q, grad_K,
+  grad_V)`` write caller-allocated tensors and return ``None``.
+* Q, K, V are float32 (as in the reference) or bfloat16 (fp32 accumulation).  The
+  product is float32 in both cases (``__init__.py:41`` allocates with the default
+  dtype) and the gradients have the dtype of their inputs (``__init__.py:59-61``).
+"""
+import torch
+
+from .. import _native
+
+
+def _prepare(t, name):
+    """The kernels take any N/H/L strides but need unit stride in the last dimension."""
+    if t.dim() != 4:
+        raise RuntimeError("causal_dot_product: %s must be 4-dimensional (N, H, L, X), got %d-d"
+                           % (name, t.dim()))
+    if t.device.type != "cuda":
+        raise RuntimeError("causal_dot_product: %s is on %s, expected a GPU tensor"
+                           % (name, t.device))
+    if t.shape[3] > 1 and t.stride(3) != 1:
+        return t.contiguous()
+    if any(s == 0 and n > 1 for s, n in zip(t.stride()[:3], t.shape[:3])):
+        return t.contiguous()
+    return t
+
+
+def _check_out(t, name):
+    if t.dim() != 4 or t.device.type != "cuda":
+        raise RuntimeError("causal_dot_product: %s must be a 4-dimensional GPU tensor" % name)
+    if t.shape[3] > 1 and t.stride(3) != 1:
+        raise RuntimeError("causal_dot_product: output %s must be contiguous in its last "
+                           "dimension" % name)
+    return t
+
+
+def _workspace(nbytes, device):
+    if nbytes <= 0:
+        return None, 0
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=device)
+    return ws, nbytes
+
+
+def causal_dot_product_hip(queries, keys, values, product):
+    """In-place forward; replaces the reference's native ``causal_dot_product``
+    (``causal_product_cuda.cu:1273-1285``).  Enqueued on the current stream."""
+    lib = _native.load()
+    q, k, v = (_prepare(t, n) for t, n in
+               ((queries, "queries"), (keys, "keys"), (values, "values")))
+    out = _check_out(product, "product")
+    N, H, L, E = q.shape
+    M = v.shape[3]
+    with torch.cuda.device(q.device):
+        nbytes = _native.check(
+            lib.ftc_causal_dot_product_workspace_bytes(N, H, L, E, M, _native.dtype_code(q.dtype)),
+            "ftc_causal_dot_product_workspace_bytes")
+        ws, nbytes = _workspace(nbytes, q.device)
+        dq, dk, dv, do = (_native.describe(t) for t in (q, k, v, out))
+        rc = lib.ftc_causal_dot_product(dq, dk, dv, do, ws.data_ptr() if ws is not None else None,
+                                        nbytes, torch.cuda.current_stream().cuda_stream)
+    _native.check(rc, "ftc_causal_dot_product")
+
+
+def causal_dot_backward_hip(queries, keys, values, grad_out, grad_queries, grad_keys,
+                            grad_values):
+    """In-place backward; replaces the reference's native ``causal_dot_backward``
+    (``causal_product_cuda.cu:1438-1467``).  Enqueued on the current stream."""
+    lib = _native.load()
+    q, k, v, g = (_prepare(t, n) for t, n in
+                  ((queries, "queries"), (keys, "keys"), (values, "values"),
+                   (grad_out, "grad_out")))
+    if g.dtype != torch.float32:
+        g = g.float()
+    gq, gk, gv = (_check_out(t, n) for t, n in
+                  ((grad_queries, "grad_queries"), (grad_keys, "grad_keys"),
+                   (grad_values, "grad_values")))
+    N, H, L, E = q.shape
+    M = v.shape[3]
+    with torch.cuda.device(q.device):
+        nbytes = _native.check(
+            lib.ftc_causal_dot_backward_workspace_bytes(N, H, L, E, M,
+                                                        _native.dtype_code(q.dtype)),
+            "ftc_causal_dot_backward_workspace_bytes")
+        ws, nbytes = _workspace(nbytes, q.device)
+        descs = [_native.describe(t) for t in (q, k, v, g, gq, gk, gv)]
+        rc = lib.ftc_causal_dot_backward(*descs, ws.data_ptr() if ws is not None else None,
+                                         nbytes, torch.cuda.current_stream().cuda_stream)
+    _native.check(rc, "ftc_causal_dot_backward")
+
+
+class CausalDotProduct(torch.autograd.Function):
+    """Compute the weighted sum of values but attending only to previous values
+    (reference ``__init__.py:20-74``)."""
+    dot = {
+        "cuda": causal_dot_product_hip,
+    }
+    dot_backward = {
+        "cuda": causal_dot_backward_hip,
+    }
+
+    @staticmethod
+    def forward(ctx, Q, K, V):
+        ctx.save_for_backward(Q, K, V)
+
+        device = Q.device
+        N, H, L, _ = Q.shape
+        _, _, _, M = V.shape
+        # the kernels overwrite every element, so no zero fill is needed
+        product = torch.empty((N, H, L, M), device=device, dtype=torch.float32)
+
+        CausalDotProduct.dot[device.type](
+            Q.data,
+            K.data,
+            V.data,
+            product
+        )
+        return product
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        Q, K, V = ctx.saved_tensors
+
+        grad_Q = torch.empty_like(Q, memory_format=torch.contiguous_format)
+        grad_K = torch.empty_like(K, memory_format=torch.contiguous_format)
+        grad_V = torch.empty_like(V, memory_format=torch.contiguous_format)
+
+        CausalDotProduct.dot_backward[Q.device.type](
+            Q.data,
+            K.data,
+            V.data,
+            grad_out,
+            grad_Q,
+            grad_K,
+            grad_V
+        )
+        return grad_Q, grad_K, grad_V
+
+
+# Alias the autograd functions to python style snake case naming
+causal_dot_product = CausalDotProduct.apply

@@ -1,0 +1,99 @@
+/*
+ * C ABI of the MI355X (gfx950) causal linear-attention product.
+ *
+ * This is the drop-in boundary for the native functions that
+ * fast_transformers/causal_product/__init__.py:9-17 binds as
+ * causal_dot_product / causal_dot_backward (CPU: causal_product_cpu.cpp:82-87,
+ * 133-141, 212-225; CUDA: causal_product_cuda.cu:1273-1276, 1438-1444,
+ * 1471-1483).  Plain pointers and sizes only: no torch types cross it.
+ *
+ * Conventions
+ *  - Tensors are 4-d views (N, H, L, X) described by ftc_tensor4: a device
+ *    pointer, a dtype code and sizes/strides in ELEMENTS.  The innermost
+ *    stride must be 1 (the reference CUDA path asserts the same,
+ *    causal_product_cuda.cu:774-777); N/H/L strides are free and 64-bit.
+ *  - Outputs are caller-allocated and fully overwritten.  They need not be
+ *    zero-filled (the reference wrapper zero-fills, __init__.py:41,59-61, but
+ *    its CPU kernels overwrite as well, causal_product_cpu.cpp:38-40,70).
+ *  - Q, K, V share one dtype: FTC_F32 or FTC_BF16.  The forward output and the
+ *    upstream gradient are FTC_F32 (the reference allocates the product with
+ *    the default dtype, __init__.py:41); dQ, dK, dV have the input dtype
+ *    (__init__.py:59-61).  Accumulation is always fp32.
+ *  - Every entry point returns 0 on success or a negative ftc_status; the
+ *    message of the last failure on the calling thread is ftc_last_error().
+ *    No exception crosses the boundary.
+ *  - Work is enqueued on `stream` (a hipStream_t; NULL = the default stream)
+ *    of the device that owns the pointers and returns without synchronising.
+ *  - The library allocates nothing.  Scratch memory comes in through
+ *    `workspace` (device memory of at least the number of bytes the matching
+ *    *_workspace_bytes call returns, 256-byte aligned, private to the call
+ *    until the enqueued work has finished).
+ */
+#ifndef FTC_CAUSAL_PRODUCT_H
+#define FTC_CAUSAL_PRODUCT_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum ftc_dtype { FTC_F32 = 0, FTC_BF16 = 1 };
+
+enum ftc_status {
+    FTC_OK = 0,
+    FTC_ERR_INVALID = -1,     /* null pointer, shape or dtype mismatch, inner stride != 1 */
+    FTC_ERR_UNSUPPORTED = -2, /* a size outside what the kernels cover */
+    FTC_ERR_WORKSPACE = -3,   /* workspace missing or too small */
+    FTC_ERR_HIP = -4          /* a HIP runtime call failed; see ftc_last_error() */
+};
+
+typedef struct ftc_tensor4 {
+    void *ptr;         /* device pointer to element (0,0,0,0) */
+    int32_t dtype;     /* enum ftc_dtype */
+    int64_t size[4];   /* N, H, L, X */
+    int64_t stride[4]; /* in elements; stride[3] must be 1 */
+} ftc_tensor4;
+
+/* Library/ABI version: major * 1000 + minor. */
+int ftc_version(void);
+
+/* Message of the last failing call on this thread ("" if none). */
+const char *ftc_last_error(void);
+
+/* Scratch bytes ftc_causal_dot_product needs for these sizes (>= 0), or a negative ftc_status. */
+int64_t ftc_causal_dot_product_workspace_bytes(int64_t N, int64_t H, int64_t L, int64_t E,
+                                               int64_t M, int32_t dtype);
+
+/*
+ * product[n,h,l,:] = sum_{j<=l} (queries[n,h,l,:] . keys[n,h,j,:]) values[n,h,j,:]
+ * Replaces causal_dot_product(queries, keys, values, product)
+ * (causal_product_cpu.cpp:82-124, causal_product_cuda.cu:1273-1285).
+ * queries, keys: (N,H,L,E); values, product: (N,H,L,M).
+ */
+int ftc_causal_dot_product(const ftc_tensor4 *queries, const ftc_tensor4 *keys,
+                           const ftc_tensor4 *values, const ftc_tensor4 *product,
+                           void *workspace, size_t workspace_bytes, void *stream);
+
+/* Scratch bytes ftc_causal_dot_backward needs (>= 0), or a negative ftc_status. */
+int64_t ftc_causal_dot_backward_workspace_bytes(int64_t N, int64_t H, int64_t L, int64_t E,
+                                                int64_t M, int32_t dtype);
+
+/*
+ * Gradients of the product with respect to queries, keys and values given
+ * grad_out = d loss / d product.  Replaces causal_dot_backward(queries, keys,
+ * values, grad_out, grad_queries, grad_keys, grad_values)
+ * (causal_product_cpu.cpp:133-209, causal_product_cuda.cu:1438-1467).
+ * All three gradients are always computed, as in the reference.
+ */
+int ftc_causal_dot_backward(const ftc_tensor4 *queries, const ftc_tensor4 *keys,
+                            const ftc_tensor4 *values, const ftc_tensor4 *grad_out,
+                            const ftc_tensor4 *grad_queries, const ftc_tensor4 *grad_keys,
+                            const ftc_tensor4 *grad_values, void *workspace,
+                            size_t workspace_bytes, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FTC_CAUSAL_PRODUCT_H */

@@ -1,0 +1,258 @@
+"""Parity of the HIP path (through the C ABI) with the CPU checker and the golden vectors.
+
+Tolerances (fp32): per-chain max|a-b| / max|b| <= 1e-4 everywhere; on the reference's own
+test distribution (all inputs U[0,1), L = 100) additionally the reference's metric
+max|a-b| / (|a| + 1e-6) < 1e-5 (test_causal_product_gpu.py:42-84).  With zero-mean values two
+correct fp32 summation orders differ near the zero crossings of the output, so the
+element-wise 1e-5 + 1e-4|b| violation fraction is printed and bounded rather than required to
+be zero.  bf16 inputs: 2e-2 relative to the fp32 result on the same rounded inputs.
+"""
+import glob
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from parity import max_relative_error, scale_error, violation_fraction
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def cp():
+    if not torch.cuda.is_available():
+        pytest.fail("GPU tests need a GPU (torch.cuda.is_available() is False)")
+    from fast_transformers_amd import causal_product
+    from fast_transformers_amd import _native
+    _native.load()  # fail loudly when the HIP library is not built
+    return causal_product
+
+
+def hip_forward(cp, Q, K, V, fill=float("nan")):
+    N, H, L, _ = Q.shape
+    out = torch.full((N, H, L, V.shape[3]), fill, device="cuda", dtype=torch.float32)
+    cp.causal_dot_product_hip(Q.cuda(), K.cuda(), V.cuda(), out)
+    torch.cuda.synchronize()
+    return out.cpu()
+
+
+def hip_backward(cp, Q, K, V, G, fill=float("nan")):
+    Qd, Kd, Vd, Gd = (t.cuda() for t in (Q, K, V, G))
+    grads = [torch.full_like(t, fill) for t in (Qd, Kd, Vd)]
+    cp.causal_dot_backward_hip(Qd, Kd, Vd, Gd, *grads)
+    torch.cuda.synchronize()
+    return [g.cpu() for g in grads]
+
+
+def report(tag, got, want):
+    s, v = scale_error(got, want), violation_fraction(got, want)
+    print("%-28s scale_err %.3e  outside(1e-5+1e-4|b|) %.4f%%" % (tag, s, 100 * v), flush=True)
+    return s, v
+
+
+def _golden_files():
+    here = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+    return sorted(glob.glob(os.path.join(here, "causal_*.npz")))
+
+
+@pytest.mark.parametrize("path", _golden_files(), ids=os.path.basename)
+def test_golden_vectors(cp, path):
+    z = np.load(path)
+    Q, K, V, G = (torch.from_numpy(z[k]) for k in "QKVG")
+    print("golden", os.path.basename(path), tuple(Q.shape), tuple(V.shape), flush=True)
+    out = hip_forward(cp, Q, K, V)
+    dQ, dK, dV = hip_backward(cp, Q, K, V, G)
+    for got, key in ((out, "product"), (dQ, "grad_queries"), (dK, "grad_keys"),
+                     (dV, "grad_values")):
+        want = torch.from_numpy(z[key])
+        assert torch.isfinite(got).all(), key
+        s, _ = report(key, got, want)
+        assert s <= 1e-4, key
+
+
+@pytest.mark.parametrize("trial", range(10))
+def test_reference_gpu_protocol(cp, trial):
+    """tests/causal_product/test_causal_product_gpu.py:42-84 with seeded draws."""
+    rng = np.random.RandomState(1000 + trial)
+    N, H, L = 4, 10, 100
+    E, M = int(rng.randint(10, 512)), int(rng.randint(10, 512))
+    print("protocol trial", trial, "E", E, "M", M, flush=True)
+    Q, K, V, G = oracle.make_inputs(N, H, L, E, M, seed=trial, positive_uniform=True)
+    out = hip_forward(cp, Q, K, V)
+    want = oracle.forward(Q, K, V)
+    assert max_relative_error(want, out) < 1e-5
+    assert torch.allclose(out, want, rtol=1e-4, atol=1e-5)
+    grads = hip_backward(cp, Q, K, V, G)
+    for got, ref in zip(grads, oracle.backward(Q, K, V, G)):
+        assert max_relative_error(ref, got) < 1e-5
+        assert torch.allclose(got, ref, rtol=1e-4, atol=1e-5)
+
+
+CONFIG_SHAPES = {
+    # BASELINE configs 1 and 2 at full size
+    "cfg1": (2, 4, 512, 64, 64, 1),
+    "cfg2": (10, 8, 1000, 64, 64, 2),
+    # config 3's length with 2 of its 16 heads (the CPU checker needs ~1 s per head)
+    "cfg3_2heads": (1, 2, 65536, 64, 64, 3),
+    # config 5's head shape, fp32, shortened
+    "e32_m128": (2, 4, 4096, 32, 128, 5),
+    "odd_l": (3, 5, 777, 64, 64, 6),
+    "e128_m128": (2, 2, 300, 128, 128, 7),
+    "e25_m64": (10, 4, 100, 25, 64, 8),
+    "l1": (2, 3, 1, 16, 16, 9),
+}
+
+
+@pytest.mark.parametrize("name", sorted(CONFIG_SHAPES))
+def test_configs_against_cpu_checker(cp, name):
+    N, H, L, E, M, seed = CONFIG_SHAPES[name]
+    print("config", name, (N, H, L, E, M), flush=True)
+    Q, K, V, G = oracle.make_inputs(N, H, L, E, M, seed)
+    want = oracle.forward(Q, K, V)
+    out = hip_forward(cp, Q, K, V)
+    assert torch.isfinite(out).all()
+    s, v = report(name + " product", out, want)
+    assert s <= 1e-4 and v <= 0.02
+    # neither fp32 order is exact: the HIP result must be as close to float64 as the checker
+    if N * H * L <= 200000:
+        exact = oracle.forward(Q.double(), K.double(), V.double())
+        s_hip, s_cpu = scale_error(out, exact), scale_error(want, exact)
+        print("    vs float64: hip %.3e  cpu %.3e" % (s_hip, s_cpu), flush=True)
+        assert s_hip <= max(4 * s_cpu, 2e-6)
+    grads = hip_backward(cp, Q, K, V, G)
+    for key, got, ref in zip(("dQ", "dK", "dV"), grads, oracle.backward(Q, K, V, G)):
+        assert torch.isfinite(got).all(), key
+        s, v = report(name + " " + key, got, ref)
+        assert s <= 1e-4 and v <= 0.02, key
+
+
+def test_full_config3_size_properties(cp):
+    """N=1, H=16, L=65536 at full size: prefix property, linearity in V, and two heads
+    against the CPU checker."""
+    N, H, L, E, M = 1, 16, 65536, 64, 64
+    Q, K, V, G = oracle.make_inputs(N, H, L, E, M, seed=3)
+    Qd, Kd, Vd = Q.cuda(), K.cuda(), V.cuda()
+    out = torch.empty(N, H, L, M, device="cuda")
+    cp.causal_dot_product_hip(Qd, Kd, Vd, out)
+    # prefix property: a truncated sequence gives the same rows
+    Lp = L // 2 + 13
+    outp = torch.empty(N, H, Lp, M, device="cuda")
+    cp.causal_dot_product_hip(Qd[:, :, :Lp], Kd[:, :, :Lp], Vd[:, :, :Lp], outp)
+    assert scale_error(outp.cpu(), out[:, :, :Lp].cpu()) <= 1e-5
+    # linearity in V
+    out2 = torch.empty_like(out)
+    cp.causal_dot_product_hip(Qd, Kd, 2.0 * Vd, out2)
+    assert scale_error(out2.cpu(), (2.0 * out).cpu()) <= 1e-6
+    want = oracle.forward(Q[:, 5:7].contiguous(), K[:, 5:7].contiguous(), V[:, 5:7].contiguous())
+    s, _ = report("cfg3 heads 5-6", out[:, 5:7].cpu(), want)
+    assert s <= 1e-4
+    # backward: dV is linear in G, and two heads against the checker
+    grads = [torch.empty_like(t) for t in (Qd, Kd, Vd)]
+    cp.causal_dot_backward_hip(Qd, Kd, Vd, G.cuda(), *grads)
+    sl = slice(5, 7)
+    refs = oracle.backward(Q[:, sl].contiguous(), K[:, sl].contiguous(), V[:, sl].contiguous(),
+                           G[:, sl].contiguous())
+    for key, got, ref in zip(("dQ", "dK", "dV"), grads, refs):
+        s, _ = report("cfg3 heads 5-6 " + key, got[:, sl].cpu(), ref)
+        assert s <= 1e-4, key
+
+
+def test_autograd_api_against_normalised_attention(cp):
+    """tests/causal_product/test_causal_product.py:21-62 on the GPU."""
+    rng = np.random.RandomState(7)
+    for t in range(10):
+        N, H, L = 2, 4, 100
+        E, M = int(rng.randint(10, 256)), int(rng.randint(10, 256))
+        print("api trial", t, E, M, flush=True)
+        gen = torch.Generator().manual_seed(t)
+        Q = torch.rand(N, H, L, E, generator=gen).cuda().requires_grad_(True)
+        K = torch.rand(N, H, L, E, generator=gen).cuda().requires_grad_(True)
+        V = torch.randn(N, H, L, M, generator=gen).cuda().requires_grad_(True)
+
+        QK = torch.einsum("nhle,nhse->nhls", Q, K)
+        QK = QK * torch.tril(torch.ones(L, L, device="cuda"))[None, None]
+        QK = QK / (QK.sum(-1, keepdim=True) + 1e-6)
+        V_new = torch.einsum("nhls,nhsm->nhlm", QK, V)
+        V_new.sum().backward()
+        grad = [x.grad.clone() for x in (Q, K, V)]
+        for x in (Q, K, V):
+            x.grad = None
+
+        V_hat = cp.causal_dot_product(Q, K, V)
+        assert V_hat.dtype == torch.float32 and V_hat.shape == (N, H, L, M)
+        Z = torch.einsum("nhle,nhle->nhl", Q, torch.cumsum(K, dim=-2) + 1e-6).unsqueeze(-1)
+        V_hat = V_hat / Z
+        V_hat.sum().backward()   # grad_out arrives as an expanded (stride-0) tensor
+        assert (V_new - V_hat).abs().max().item() < 5e-4
+        for g1, x in zip(grad, (Q, K, V)):
+            assert (g1 - x.grad).abs().max().item() < 5e-4
+
+
+def test_strided_views_and_dirty_outputs(cp):
+    """Inputs as permuted (N, L, H, X) storage; outputs pre-filled with garbage."""
+    N, H, L, E, M = 2, 3, 150, 40, 24
+    gen = torch.Generator().manual_seed(5)
+    store = [torch.rand(N, L, H, E, generator=gen), torch.rand(N, L, H, E, generator=gen),
+             torch.randn(N, L, H, M, generator=gen), torch.randn(N, L, H, M, generator=gen)]
+    Q, K, V, G = (t.permute(0, 2, 1, 3) for t in store)
+    Qd, Kd, Vd, Gd = (t.cuda().permute(0, 2, 1, 3) for t in store)
+    assert not Qd.is_contiguous() and Qd.shape == (N, H, L, E)
+    out = torch.full((N, L, H, M), 3.0, device="cuda").permute(0, 2, 1, 3)
+    cp.causal_dot_product_hip(Qd, Kd, Vd, out)
+    want = oracle.forward(Q.contiguous(), K.contiguous(), V.contiguous())
+    assert scale_error(out.cpu(), want) <= 1e-5
+    grads = [torch.full((N, H, L, X), -5.0, device="cuda") for X in (E, E, M)]
+    cp.causal_dot_backward_hip(Qd, Kd, Vd, Gd, *grads)
+    refs = oracle.backward(Q.contiguous(), K.contiguous(), V.contiguous(), G.contiguous())
+    for got, ref in zip(grads, refs):
+        assert scale_error(got.cpu(), ref) <= 1e-5
+
+
+def test_bf16_inputs_fp32_accumulate(cp):
+    N, H, L, E, M = 2, 4, 2048, 32, 128
+    Q, K, V, G = oracle.make_inputs(N, H, L, E, M, seed=5)
+    Qb, Kb, Vb = (t.bfloat16() for t in (Q, K, V))
+    # fp32 result on the same bf16-rounded inputs
+    want = oracle.forward(Qb.float(), Kb.float(), Vb.float())
+    refs = oracle.backward(Qb.float(), Kb.float(), Vb.float(), G)
+    out = torch.empty(N, H, L, M, device="cuda")
+    cp.causal_dot_product_hip(Qb.cuda(), Kb.cuda(), Vb.cuda(), out)
+    assert scale_error(out.cpu(), want) <= 2e-2
+    grads = [torch.empty_like(t.cuda()) for t in (Qb, Kb, Vb)]
+    cp.causal_dot_backward_hip(Qb.cuda(), Kb.cuda(), Vb.cuda(), G.cuda(), *grads)
+    for key, got, ref in zip(("dQ", "dK", "dV"), grads, refs):
+        assert got.dtype == torch.bfloat16
+        s, _ = report("bf16 " + key, got.float().cpu(), ref)
+        assert s <= 2e-2, key
+    # through autograd: product is fp32, gradients come back as bf16
+    Qg, Kg, Vg = (t.cuda().requires_grad_(True) for t in (Qb, Kb, Vb))
+    o = cp.causal_dot_product(Qg, Kg, Vg)
+    assert o.dtype == torch.float32
+    (o * G.cuda()).sum().backward()
+    assert Qg.grad.dtype == torch.bfloat16 and Vg.grad.dtype == torch.bfloat16
+    assert scale_error(Qg.grad.float().cpu(), refs[0]) <= 2e-2
+
+
+def test_errors_and_empty_inputs(cp):
+    Q = torch.rand(1, 2, 8, 4, device="cuda")
+    V = torch.rand(1, 2, 8, 6, device="cuda")
+    out = torch.empty(1, 2, 8, 6, device="cuda")
+    with pytest.raises(RuntimeError):
+        cp.causal_dot_product_hip(Q, Q[:, :, :7], V, out)          # L mismatch
+    with pytest.raises(RuntimeError):
+        cp.causal_dot_product_hip(Q.half(), Q.half(), V.half(), out)  # unsupported dtype
+    with pytest.raises(RuntimeError):
+        cp.causal_dot_product_hip(Q, Q, V, out.double())            # product must be fp32
+    with pytest.raises(RuntimeError):
+        big = torch.rand(1, 1, 4, 600, device="cuda")
+        cp.causal_dot_product_hip(big, big, V[:, :1, :4], out[:, :1, :4])  # E > 512
+    # zero-length sequence and empty batch are no-ops
+    e = torch.empty(0, 2, 8, 4, device="cuda")
+    cp.causal_dot_product_hip(e, e, torch.empty(0, 2, 8, 6, device="cuda"),
+                              torch.empty(0, 2, 8, 6, device="cuda"))
+    z = torch.empty(1, 2, 0, 4, device="cuda")
+    o = cp.causal_dot_product(z, z, torch.empty(1, 2, 0, 6, device="cuda"))
+    assert o.shape == (1, 2, 0, 6)
+    torch.cuda.synchronize()

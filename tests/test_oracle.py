@@ -1,0 +1,230 @@
+"""Pins the CPU checker (oracle/) before anything is compared against it.
+
+Checks, each chosen so that a plausible mistake fails it:
+  * the reference's own compiled CPU extension (oracle/_ref, when built): bit-exact;
+  * the golden vectors that extension wrote (tests/golden/*.npz);
+  * the dense closed form tril(Q K^T) V and its gradients in float64, with the metric
+    and bound of the reference's tests (test_causal_product_cpu.py:19-20,49,72-74);
+  * brute-force triple loops on tiny inputs (inclusive diagonal, operand order);
+  * special cases: E = 1 is a cumulative sum; causality; the prefix property;
+    time reversal links the forward product to the dK/dV passes.
+"""
+import glob
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+
+
+def max_relative_error(a, b, eps=1e-6):
+    # tests/causal_product/test_causal_product_cpu.py:19-20
+    return torch.abs((a - b) / (torch.abs(a) + eps)).max().item()
+
+
+SHAPES = [(2, 3, 50, 17, 33), (1, 2, 100, 64, 64), (1, 1, 64, 130, 10), (3, 1, 7, 1, 1)]
+
+
+@pytest.mark.skipif(not oracle.reference_extension_available(), reason="oracle/_ref not built")
+@pytest.mark.parametrize("shape", SHAPES)
+def test_restatement_is_bit_exact_with_reference_extension(shape):
+    ref = oracle.load_reference_extension()
+    N, H, L, E, M = shape
+    Q, K, V, G = oracle.make_inputs(N, H, L, E, M, seed=sum(shape))
+    out_ref = torch.zeros(N, H, L, M)
+    ref.causal_dot_product(Q, K, V, out_ref)
+    assert torch.equal(oracle.forward(Q, K, V), out_ref)
+    g_ref = [torch.zeros_like(x) for x in (Q, K, V)]
+    ref.causal_dot_backward(Q, K, V, G, *g_ref)
+    for a, b in zip(oracle.backward(Q, K, V, G), g_ref):
+        assert torch.equal(a, b)
+
+
+@pytest.mark.skipif(not oracle.reference_extension_available(), reason="oracle/_ref not built")
+def test_restatement_matches_reference_extension_on_strided_views():
+    ref = oracle.load_reference_extension()
+    N, H, L, E, M = 2, 3, 40, 20, 24
+    gen = torch.Generator().manual_seed(5)
+    # (N, L, H, X) storage viewed as (N, H, L, X): what a caller gets from permute()
+    Q = torch.rand(N, L, H, E, generator=gen).permute(0, 2, 1, 3)
+    K = torch.rand(N, L, H, E, generator=gen).permute(0, 2, 1, 3)
+    V = torch.randn(N, L, H, M, generator=gen).permute(0, 2, 1, 3)
+    G = torch.randn(N, L, H, M, generator=gen).permute(0, 2, 1, 3)
+    out_ref = torch.zeros(N, H, L, M)
+    ref.causal_dot_product(Q, K, V, out_ref)
+    out = torch.full((N, L, H, M), float("nan")).permute(0, 2, 1, 3)
+    oracle.causal_dot_product(Q, K, V, out)
+    assert torch.equal(out, out_ref)
+    g_ref = [torch.zeros(N, H, L, X) for X in (E, E, M)]
+    ref.causal_dot_backward(Q, K, V, G, *g_ref)
+    g = [torch.full((N, H, L, X), float("nan")) for X in (E, E, M)]
+    oracle.causal_dot_backward(Q, K, V, G, *g)
+    for a, b in zip(g, g_ref):
+        assert torch.equal(a, b)
+
+
+def _golden_files():
+    here = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+    return sorted(glob.glob(os.path.join(here, "causal_*.npz")))
+
+
+def test_golden_vectors_exist():
+    assert len(_golden_files()) >= 6
+
+
+@pytest.mark.parametrize("path", _golden_files(), ids=os.path.basename)
+def test_restatement_reproduces_golden_vectors(path):
+    z = np.load(path)
+    Q, K, V, G = (torch.from_numpy(z[k]) for k in "QKVG")
+    out = oracle.forward(Q, K, V)
+    dQ, dK, dV = oracle.backward(Q, K, V, G)
+    for got, key in ((out, "product"), (dQ, "grad_queries"), (dK, "grad_keys"),
+                     (dV, "grad_values")):
+        want = torch.from_numpy(z[key])
+        scale = want.abs().max().item()
+        assert (got - want).abs().max().item() <= 1e-6 * scale, key
+
+
+@pytest.mark.parametrize("path", _golden_files(), ids=os.path.basename)
+def test_golden_vectors_satisfy_dense_closed_form(path):
+    """The stored reference outputs themselves obey tril(Q K^T) V in float64."""
+    z = np.load(path)
+    Q, K, V, G = (torch.from_numpy(z[k]).double() for k in "QKVG")
+    want = (oracle.dense_forward(Q, K, V),) + oracle.dense_backward(Q, K, V, G)
+    for w, key in zip(want, ("product", "grad_queries", "grad_keys", "grad_values")):
+        got = torch.from_numpy(z[key]).double()
+        assert (got - w).abs().max().item() <= 2e-6 * w.abs().max().item(), key
+
+
+@pytest.mark.parametrize("trial", range(4))
+def test_forward_against_dense_form_reference_protocol(trial):
+    # test_causal_product_cpu.py:32-49 with seeded draws and a smaller batch
+    rng = np.random.RandomState(100 + trial)
+    N, H, L = 3, 4, 100
+    E, M = int(rng.randint(10, 256)), int(rng.randint(10, 256))
+    Q, K, V, _ = oracle.make_inputs(N, H, L, E, M, seed=trial, positive_uniform=True)
+    out = oracle.forward(Q, K, V)
+    dense = oracle.dense_forward(Q.double(), K.double(), V.double()).float()
+    assert max_relative_error(dense, out) < 1e-5
+
+
+@pytest.mark.parametrize("trial", range(4))
+def test_backward_against_autograd_of_dense_form(trial):
+    # test_causal_product_cpu.py:51-74
+    rng = np.random.RandomState(200 + trial)
+    N, H, L = 2, 3, 100
+    E, M = int(rng.randint(10, 256)), int(rng.randint(10, 256))
+    Q, K, V, G = oracle.make_inputs(N, H, L, E, M, seed=50 + trial, positive_uniform=True)
+    dQ, dK, dV = oracle.backward(Q, K, V, G)
+    Qd, Kd, Vd = (x.double().requires_grad_(True) for x in (Q, K, V))
+    out = oracle.dense_forward(Qd, Kd, Vd)
+    torch.einsum("nhlm,nhlm->", out, G.double()).backward()
+    assert max_relative_error(Qd.grad.float(), dQ) < 1e-5
+    assert max_relative_error(Kd.grad.float(), dK) < 1e-5
+    assert max_relative_error(Vd.grad.float(), dV) < 1e-5
+    # and the written-out gradient formulas agree with autograd
+    for a, b in zip(oracle.dense_backward(Q.double(), K.double(), V.double(), G.double()),
+                    (Qd.grad, Kd.grad, Vd.grad)):
+        assert torch.allclose(a, b, rtol=1e-12, atol=1e-12)
+
+
+def test_float64_build_gradients_by_finite_differences():
+    N, H, L, E, M = 1, 1, 6, 3, 4
+    Q, K, V, G = oracle.make_inputs(N, H, L, E, M, seed=9, dtype=torch.float64)
+    dQ, dK, dV = oracle.backward(Q, K, V, G)
+
+    def loss(q, k, v):
+        return (oracle.forward(q, k, v) * G).sum().item()
+
+    eps = 1e-6
+    for x, dx, which in ((Q, dQ, 0), (K, dK, 1), (V, dV, 2)):
+        for idx in [(0, 0, 0, 0), (0, 0, 2, 1), (0, 0, L - 1, x.shape[3] - 1)]:
+            xp, xm = x.clone(), x.clone()
+            xp[idx] += eps
+            xm[idx] -= eps
+            args_p = [Q, K, V]
+            args_m = [Q, K, V]
+            args_p[which], args_m[which] = xp, xm
+            fd = (loss(*args_p) - loss(*args_m)) / (2 * eps)
+            assert abs(fd - dx[idx].item()) < 1e-6 * max(1.0, abs(fd))
+
+
+def test_brute_force_tiny():
+    N, H, L, E, M = 1, 2, 5, 3, 2
+    Q, K, V, G = oracle.make_inputs(N, H, L, E, M, seed=3, dtype=torch.float64)
+    out = oracle.forward(Q, K, V)
+    dQ, dK, dV = oracle.backward(Q, K, V, G)
+    want = torch.zeros(N, H, L, M, dtype=torch.float64)
+    wq, wk, wv = torch.zeros_like(Q), torch.zeros_like(K), torch.zeros_like(V)
+    for h in range(H):
+        for l in range(L):
+            for j in range(l + 1):  # inclusive: position l sees key l
+                qk = sum(Q[0, h, l, e] * K[0, h, j, e] for e in range(E))
+                gv = sum(G[0, h, l, m] * V[0, h, j, m] for m in range(M))
+                for m in range(M):
+                    want[0, h, l, m] += qk * V[0, h, j, m]
+                    wv[0, h, j, m] += qk * G[0, h, l, m]
+                for e in range(E):
+                    wq[0, h, l, e] += gv * K[0, h, j, e]
+                    wk[0, h, j, e] += gv * Q[0, h, l, e]
+    for a, b in ((out, want), (dQ, wq), (dK, wk), (dV, wv)):
+        assert torch.allclose(a, b, rtol=1e-12, atol=1e-12)
+
+
+def test_first_position_and_unit_width():
+    Q, K, V, _ = oracle.make_inputs(2, 2, 9, 1, 5, seed=4, dtype=torch.float64)
+    out = oracle.forward(Q, K, V)
+    # E = 1: out_l = q_l * cumsum_l(k v)
+    want = Q * torch.cumsum(K * V, dim=2)
+    assert torch.allclose(out, want, rtol=1e-12, atol=1e-12)
+    Q, K, V, _ = oracle.make_inputs(1, 1, 4, 6, 3, seed=5, dtype=torch.float64)
+    out = oracle.forward(Q, K, V)
+    assert torch.allclose(out[0, 0, 0], (Q[0, 0, 0] @ K[0, 0, 0]) * V[0, 0, 0])
+    # Q = 1: out = cumsum over L of (sum_e k_e) v
+    ones = torch.ones_like(Q)
+    want = torch.cumsum(K.sum(-1, keepdim=True) * V, dim=2)
+    assert torch.allclose(oracle.forward(ones, K, V), want, rtol=1e-12, atol=1e-12)
+
+
+def test_causality_and_prefix_property():
+    N, H, L, E, M = 1, 2, 40, 8, 8
+    Q, K, V, _ = oracle.make_inputs(N, H, L, E, M, seed=6)
+    out = oracle.forward(Q, K, V)
+    K2, V2 = K.clone(), V.clone()
+    K2[:, :, 25] += 1.0
+    V2[:, :, 25] -= 2.0
+    out2 = oracle.forward(Q, K2, V2)
+    assert torch.equal(out[:, :, :25], out2[:, :, :25])
+    assert not torch.equal(out[:, :, 25], out2[:, :, 25])
+    short = oracle.forward(Q[:, :, :17].contiguous(), K[:, :, :17].contiguous(),
+                           V[:, :, :17].contiguous())
+    assert torch.equal(short, out[:, :, :17])
+
+
+def test_role_and_time_reversal_identities():
+    """dQ = fwd(G, V, K); dK = flip(fwd(flip V, flip G, flip Q)); dV = flip(fwd(flip K, flip Q, flip G))."""
+    Q, K, V, G = oracle.make_inputs(1, 2, 30, 5, 7, seed=7, dtype=torch.float64)
+    dQ, dK, dV = oracle.backward(Q, K, V, G)
+    flip = lambda t: torch.flip(t, dims=[2]).contiguous()
+    assert torch.allclose(dQ, oracle.forward(G, V, K), rtol=1e-12, atol=1e-12)
+    assert torch.allclose(dK, flip(oracle.forward(flip(V), flip(G), flip(Q))), rtol=1e-12,
+                          atol=1e-12)
+    assert torch.allclose(dV, flip(oracle.forward(flip(K), flip(Q), flip(G))), rtol=1e-12,
+                          atol=1e-12)
+
+
+def test_recurrent_form_agrees():
+    # tests/recurrent/attention/self_attention/test_linear_attention.py:54-79 (1e-5 abs)
+    Q, K, V, _ = oracle.make_inputs(2, 2, 60, 25, 64, seed=8, positive_uniform=True)
+    out = oracle.forward(Q, K, V)
+    rec = oracle.recurrent_forward(Q.double(), K.double(), V.double())
+    assert (out.double() - rec).abs().max().item() < 1e-5 * max(1.0, rec.abs().max().item())
+
+
+def test_outputs_need_not_be_zeroed():
+    Q, K, V, G = oracle.make_inputs(1, 1, 10, 4, 4, seed=10)
+    out = torch.full((1, 1, 10, 4), 7.0)
+    oracle.causal_dot_product(Q, K, V, out)
+    assert torch.equal(out, oracle.forward(Q, K, V))
