@@ -69,6 +69,20 @@ int read_dims(const ftc_tensor4 *q, const ftc_tensor4 *v, Dims *d) {
     return FTC_OK;
 }
 
+// Picks the MFMA scan when the operands qualify, else the generic scan.
+int scan(const Operand &a, const Operand &b, const Operand &v, const OperandOut &out, int64_t N,
+         int64_t H, int64_t L, bool reverse, void *workspace, size_t workspace_bytes,
+         hipStream_t stream) {
+    if (mfma_scan_supported(a, b, v, out))
+        return mfma_scan(a, b, v, out, N, H, L, reverse, workspace, workspace_bytes, stream);
+    return generic_scan(a, b, v, out, N, H, L, reverse, workspace, workspace_bytes, stream);
+}
+
+int64_t scan_workspace_bytes(int64_t N, int64_t H, int64_t L, int64_t D, int64_t F) {
+    return std::max(generic_scan_workspace_bytes(N, H, L, D, F),
+                    mfma_scan_workspace_bytes(N, H, L, D, F));
+}
+
 }  // namespace
 }  // namespace ftc
 
@@ -87,7 +101,7 @@ int64_t ftc_causal_dot_product_workspace_bytes(int64_t N, int64_t H, int64_t L, 
     if (N * H * L == 0 || M == 0 || E == 0) return 0;
     if (E > kGenericMaxDim || M > kGenericMaxDim)
         return fail(FTC_ERR_UNSUPPORTED, "E and M must be at most %d", kGenericMaxDim);
-    return generic_scan_workspace_bytes(N, H, L, E, M);
+    return scan_workspace_bytes(N, H, L, E, M);
 }
 
 int ftc_causal_dot_product(const ftc_tensor4 *queries, const ftc_tensor4 *keys,
@@ -105,9 +119,8 @@ int ftc_causal_dot_product(const ftc_tensor4 *queries, const ftc_tensor4 *keys,
     hipStream_t s = (hipStream_t)stream;
     if (d.E == 0)  // an empty contraction: every product row is zero
         return zero_rows(as_operand_out(product), d.N, d.H, d.L, s);
-    return generic_scan(as_operand(queries), as_operand(keys), as_operand(values),
-                        as_operand_out(product), d.N, d.H, d.L, false, workspace, workspace_bytes,
-                        s);
+    return scan(as_operand(queries), as_operand(keys), as_operand(values),
+                as_operand_out(product), d.N, d.H, d.L, false, workspace, workspace_bytes, s);
 }
 
 int64_t ftc_causal_dot_backward_workspace_bytes(int64_t N, int64_t H, int64_t L, int64_t E,
@@ -117,8 +130,7 @@ int64_t ftc_causal_dot_backward_workspace_bytes(int64_t N, int64_t H, int64_t L,
     if (N * H * L == 0 || M == 0 || E == 0) return 0;
     if (E > kGenericMaxDim || M > kGenericMaxDim)
         return fail(FTC_ERR_UNSUPPORTED, "E and M must be at most %d", kGenericMaxDim);
-    return std::max(generic_scan_workspace_bytes(N, H, L, E, M),
-                    generic_scan_workspace_bytes(N, H, L, M, E));
+    return std::max(scan_workspace_bytes(N, H, L, E, M), scan_workspace_bytes(N, H, L, M, E));
 }
 
 int ftc_causal_dot_backward(const ftc_tensor4 *queries, const ftc_tensor4 *keys,
@@ -149,14 +161,14 @@ int ftc_causal_dot_backward(const ftc_tensor4 *queries, const ftc_tensor4 *keys,
     hipStream_t s = (hipStream_t)stream;
     const Operand Q = as_operand(queries), K = as_operand(keys), V = as_operand(values),
                   G = as_operand(grad_out);
-    if ((rc = generic_scan(G, V, K, as_operand_out(grad_queries), d.N, d.H, d.L, false, workspace,
-                           workspace_bytes, s)))
+    if ((rc = scan(G, V, K, as_operand_out(grad_queries), d.N, d.H, d.L, false, workspace,
+                   workspace_bytes, s)))
         return rc;
-    if ((rc = generic_scan(V, G, Q, as_operand_out(grad_keys), d.N, d.H, d.L, true, workspace,
-                           workspace_bytes, s)))
+    if ((rc = scan(V, G, Q, as_operand_out(grad_keys), d.N, d.H, d.L, true, workspace,
+                   workspace_bytes, s)))
         return rc;
-    return generic_scan(K, Q, G, as_operand_out(grad_values), d.N, d.H, d.L, true, workspace,
-                        workspace_bytes, s);
+    return scan(K, Q, G, as_operand_out(grad_values), d.N, d.H, d.L, true, workspace,
+                workspace_bytes, s);
 }
 
 }  // extern "C"
