@@ -73,7 +73,7 @@ int read_dims(const ftc_tensor4 *q, const ftc_tensor4 *v, Dims *d) {
 int scan(const Operand &a, const Operand &b, const Operand &v, const OperandOut &out, int64_t N,
          int64_t H, int64_t L, bool reverse, void *workspace, size_t workspace_bytes,
          hipStream_t stream) {
-    if (mfma_scan_supported(a, b, v, out))
+    if (mfma_scan_supported(a, b, v, out, L))
         return mfma_scan(a, b, v, out, N, H, L, reverse, workspace, workspace_bytes, stream);
     return generic_scan(a, b, v, out, N, H, L, reverse, workspace, workspace_bytes, stream);
 }

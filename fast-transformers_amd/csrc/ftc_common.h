@@ -78,7 +78,7 @@ int generic_scan(const Operand &a, const Operand &b, const Operand &v, const Ope
 // ftc_mfma.hip.  Same contract as generic_scan.
 // ---------------------------------------------------------------------------
 bool mfma_scan_supported(const Operand &a, const Operand &b, const Operand &v,
-                         const OperandOut &out);
+                         const OperandOut &out, int64_t L);
 int64_t mfma_scan_workspace_bytes(int64_t N, int64_t H, int64_t L, int64_t D, int64_t F);
 int mfma_scan(const Operand &a, const Operand &b, const Operand &v, const OperandOut &out,
               int64_t N, int64_t H, int64_t L, bool reverse, void *workspace,

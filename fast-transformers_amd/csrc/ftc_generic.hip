@@ -226,7 +226,10 @@ GenericPlan make_plan(int64_t N, int64_t H, int64_t L, int64_t D, int64_t F) {
     nseg = std::max<int64_t>(1, (L + seg_len - 1) / seg_len);
     pl.nseg = (int)nseg;
     pl.seg_len = (int)seg_len;
-    pl.workspace_bytes = nseg > 1 ? chains * nseg * D * F * (int64_t)sizeof(float) : 0;
+    // the segment states live behind the workspace's control block, which this path never
+    // touches (the MFMA path keeps its tickets and flags there and expects them zero)
+    pl.workspace_bytes =
+        nseg > 1 ? FTC_WORKSPACE_CONTROL_BYTES + chains * nseg * D * F * (int64_t)sizeof(float) : 0;
     return pl;
 }
 
@@ -288,7 +291,8 @@ int generic_scan(const Operand &a, const Operand &b, const Operand &v, const Ope
     args.b = b;
     args.v = v;
     args.out = out;
-    args.states = pl.nseg > 1 ? (float *)workspace : nullptr;
+    args.states =
+        pl.nseg > 1 ? (float *)((char *)workspace + FTC_WORKSPACE_CONTROL_BYTES) : nullptr;
     args.L = L;
     args.H = (int32_t)H;
     args.D = (int32_t)D;

@@ -1,12 +1,11 @@
-// MFMA causal scan for gfx950, fp32 rows, row widths D, F in {32, 64, 128} (D*F <= 4096).
+// MFMA causal scan for gfx950, fp32 rows, (D, F) in {(64,64), (32,128), (128,32)}.
 //
 //   out[c, l, f] = sum_{j <= l} (a[c,l,:] . b[c,j,:]) * v[c,j,f]      (REV: j >= l)
 //
 // One wavefront owns one (chain, L-segment) and walks it in chunks of 32 positions with
-// the whole D x F state in its accumulator registers; wavefronts never synchronise with
-// each other.  Per chunk (i, j index positions of the chunk, all products on
-// v_mfma_f32_32x32x16_bf16, written in the transposed orientation so that every chained
-// operand is already in registers):
+// the whole D x F state in its accumulator registers.  Per chunk (i, j index positions of
+// the chunk; every product on v_mfma_f32_32x32x16_bf16, written in the transposed
+// orientation so that chained operands are already in registers):
 //
 //   (1)  Pt[j][i]  = sum_d b[j][d] a[i][d]            then masked to j <= i (REV: j >= i)
 //   (2a) Ot[f][i]  = sum_j vt[f][j] Pt[j][i]           Pt goes from accumulator to B operand
@@ -19,12 +18,24 @@
 // lo*hi), each exact in the fp32 accumulator.  What is dropped is below 2^-23 of the product,
 // the size of one fp32 rounding.
 //
-// Register-chaining: a 32x32 accumulator holds, in lane (col = lane % 32, g = lane / 32),
+// Register chaining: a 32x32 accumulator holds, in lane (col = lane % 32, g = lane / 32),
 // rows 8*(r/4) + 4*g + (r%4) for r = 0..15.  Registers 8h..8h+7 are therefore 8 values
 // of the contraction index for k-step h, provided the other operand uses the same order:
 // k-slot (g, t) of a 16-wide k-step carries logical index 8*(t/4) + 4*g + (t%4).  LDS
-// tiles are stored with that order inside every 16-block (blocks of 4 swapped: 0,2,1,3),
-// so one ds_read_b128 yields a fragment.
+// tiles are stored with that order inside every 16-block (blocks of four swapped:
+// 0,2,1,3), so one ds_read_b128 yields a fragment.
+//
+// One launch per scan.  A wavefront first sums its segment's own state (reading b and v
+// only), publishes it, obtains the state that precedes its segment by decoupled look-back
+// over the published sums of the segments before it, and then replays its segment (the
+// second read of b and v is served by L2 / Infinity Cache).  Segments are handed out in
+// dependency order through a ticket counter, so a wavefront only ever waits for
+// wavefronts that are already running; every wait is bounded and raises an error word
+// instead of spinning forever.
+//
+// Rows are fetched with raw buffer loads whose descriptor ends at the segment's last row:
+// positions outside the segment read as zero and stores to them are dropped, so tails need
+// no branches.
 #include <algorithm>
 
 #include "ftc_common.h"
@@ -34,12 +45,26 @@ namespace {
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 // LDS is written as 8-byte and read as 16-byte words of the same bf16 data
 typedef uint32_t lds_u32x2 __attribute__((ext_vector_type(2), may_alias));
 typedef uint32_t lds_u32x4 __attribute__((ext_vector_type(4), may_alias));
+typedef __attribute__((address_space(1))) float gfloat;
+typedef __attribute__((address_space(1))) uint32_t gu32;
 
 constexpr int kChunk = 32;
 constexpr int kWave = 64;
+constexpr uint32_t kRsrcFlags = 0x00020000u;  // raw buffer, 32-bit data format
+constexpr int kSpinLimit = 1 << 20;           // bounded wait (about a second in total)
+
+// The workspace starts with a control block of fixed size: a header and one flag word per
+// wavefront.  It must be zero before the first use and every launch leaves it zero, so
+// later calls of any shape can reuse it.  The state slots behind it need no initialisation.
+constexpr int kHdrTicket = 0, kHdrDone = 1, kHdrError = 2;
+constexpr int kHdrWords = 64;
+constexpr int kControlBytes = FTC_WORKSPACE_CONTROL_BYTES;
+constexpr int kMaxWaves = (kControlBytes / 4) - kHdrWords;
+constexpr uint32_t kFlagEmpty = 0, kFlagSum = 1, kFlagPrefix = 2;
 
 struct Frag {
     uint32_t w[4];  // 8 bf16, k-slot t in the low (t even) / high (t odd) half of w[t/2]
@@ -94,149 +119,192 @@ __device__ __forceinline__ f32x16 mfma_split(const Frag (&a)[NS], const Frag (&b
     return acc;
 }
 
-// position of logical index x inside its 16-block for x a multiple of 4
+// position of logical index x (a multiple of 4) inside its 16-block: blocks 0,1,2,3 -> 0,2,1,3
 __device__ __forceinline__ int perm4(int x) {
-    // blocks of four: 0,1,2,3 -> 0,2,1,3
     const int blk = (x >> 2) & 3;
     const int swapped = ((blk & 1) << 1) | (blk >> 1);
     return (x & ~15) | (swapped << 2);
 }
 
-struct MfmaArgs {
-    const float *a, *b, *v;
-    float *out;
-    float *states;  // [chain][segment][D*F], accumulator-register order
+__device__ __forceinline__ float4 buffer_load4(__amdgpu_buffer_rsrc_t rsrc, uint32_t byte_offset) {
+    const u32x4 r = __builtin_amdgcn_raw_buffer_load_b128(rsrc, byte_offset, 0, 0);
+    return make_float4(__uint_as_float(r.x), __uint_as_float(r.y), __uint_as_float(r.z),
+                       __uint_as_float(r.w));
+}
+__device__ __forceinline__ void buffer_store4(__amdgpu_buffer_rsrc_t rsrc, uint32_t byte_offset,
+                                              float x, float y, float z, float w) {
+    const u32x4 r = {__float_as_uint(x), __float_as_uint(y), __float_as_uint(z), __float_as_uint(w)};
+    __builtin_amdgcn_raw_buffer_store_b128(r, rsrc, byte_offset, 0, 0);
+}
+
+// LDS writes of this wavefront are ordered before its later LDS reads (and the reverse).
+__device__ __forceinline__ void wave_lds_fence() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+struct ScanArgs {
     int64_t a_sn, a_sh, a_sl;
     int64_t b_sn, b_sh, b_sl;
     int64_t v_sn, v_sh, v_sl;
     int64_t o_sn, o_sh, o_sl;
     int64_t L;
     int32_t H, seg_len, nseg;
-    int32_t state_only;
+    int32_t total_waves;
 };
 
 template <int D, int F, int NS>
 struct Lds {
-    // per row: NS planes of the row's bf16 values, then 16 bytes of padding (keeps the
-    // row pitch at 4 (mod 8) dwords so that ds_read_b128 by 8 consecutive rows is
-    // conflict free)
-    static constexpr int kRowB = NS * D * 2 + 16;        // B_s[j][plane][pos(d)]
-    static constexpr int kRowT = NS * kChunk * 2 + 16;   // Bt_s[d][plane][pos(j)], Vt_s[f][..]
+    // per row: NS planes of the row's bf16 values, then 16 bytes of padding (keeps the row
+    // pitch at 4 (mod 8) dwords so that ds_read_b128 by 8 consecutive rows is conflict free)
+    static constexpr int kRowB = NS * D * 2 + 16;       // B_s[j][plane][pos(d)]
+    static constexpr int kRowT = NS * kChunk * 2 + 16;  // Bt_s[d][plane][pos(j)], Vt_s[f][..]
     static constexpr int kOffB = 0;
     static constexpr int kOffBt = kOffB + kChunk * kRowB;
     static constexpr int kOffVt = kOffBt + D * kRowT;
     static constexpr int kBytes = kOffVt + F * kRowT;
 };
 
+// Raw rows of one chunk held between the fetch and the split.
+template <int D, int F>
+struct RawChunk {
+    static constexpr int KD = D / 16;
+    static constexpr int BLK_B = (kChunk / 4) * (D / 4) / kWave;  // 4x4 blocks of b per lane
+    static constexpr int BLK_V = (kChunk / 4) * (F / 4) / kWave;
+    float4 a[KD][2];
+    float4 b[BLK_B][4];
+    float4 v[BLK_V][4];
+};
+
 template <int D, int F, int NS, bool REV>
-__global__ __launch_bounds__(kWave) void scan_mfma_kernel(MfmaArgs p) {
+__global__ __launch_bounds__(kWave) void scan_mfma_kernel(const float *__restrict__ a_ptr,
+                                                          const float *__restrict__ b_ptr,
+                                                          const float *__restrict__ v_ptr,
+                                                          float *__restrict__ out_ptr,
+                                                          uint32_t *__restrict__ ws_ptr,
+                                                          ScanArgs p) {
     using Lay = Lds<D, F, NS>;
+    using Raw = RawChunk<D, F>;
     constexpr int DT = D / 32, FT = F / 32;  // state tiles
     constexpr int KD = D / 16;               // k-steps over d
-    constexpr int BLK_B = (kChunk / 4) * (D / 4) / kWave;  // 4x4 blocks of b per lane
-    constexpr int BLK_V = (kChunk / 4) * (F / 4) / kWave;
+    constexpr int BLK_B = Raw::BLK_B, BLK_V = Raw::BLK_V;
+    constexpr int kStateElems = D * F;
     __shared__ __align__(16) unsigned char lds[Lay::kBytes];
 
     const int lane = threadIdx.x;
     const int ln = lane & 31, g = lane >> 5;
 
-    const int64_t wg = blockIdx.x;
-    const int seg = (int)(wg % p.nseg);
-    const int64_t chain = wg / p.nseg;
+    gu32 *hdr = (gu32 *)ws_ptr;
+    gu32 *flags = hdr + kHdrWords;
+    gfloat *sums = (gfloat *)(hdr + kControlBytes / 4);
+    gfloat *prefixes = sums + (int64_t)p.total_waves * kStateElems;
+
+    // ---- which segment: tickets follow the dependency order ----
+    uint32_t ticket = 0;
+    if (p.nseg > 1) {
+        if (lane == 0)
+            ticket = __hip_atomic_fetch_add(hdr + kHdrTicket, 1u, __ATOMIC_RELAXED,
+                                            __HIP_MEMORY_SCOPE_AGENT);
+        ticket = __builtin_amdgcn_readfirstlane(ticket);
+        if (ticket >= (uint32_t)p.total_waves) {
+            // the control block was not zero when the launch started: refuse to run on it
+            if (lane == 0)
+                __hip_atomic_store(hdr + kHdrError, 2u, __ATOMIC_RELAXED,
+                                   __HIP_MEMORY_SCOPE_AGENT);
+            return;
+        }
+    } else {
+        ticket = blockIdx.x;
+    }
+    const int64_t chain = ticket / (uint32_t)p.nseg;
+    const int step = (int)(ticket % (uint32_t)p.nseg);      // position in dependency order
+    const int seg = REV ? p.nseg - 1 - step : step;
     const int n = (int)(chain / p.H), h = (int)(chain % p.H);
     const int64_t lo = (int64_t)seg * p.seg_len;
     const int64_t hi = min(p.L, lo + (int64_t)p.seg_len);
-    const bool full = !p.state_only;
+    const int rows = (int)(hi - lo);
+    const int nchunks = (rows + kChunk - 1) / kChunk;
 
-    const float *a_base = p.a + (int64_t)n * p.a_sn + (int64_t)h * p.a_sh;
-    const float *b_base = p.b + (int64_t)n * p.b_sn + (int64_t)h * p.b_sh;
-    const float *v_base = p.v + (int64_t)n * p.v_sn + (int64_t)h * p.v_sh;
-    float *o_base = p.out + (int64_t)n * p.o_sn + (int64_t)h * p.o_sh;
-    float *my_state = p.states ? p.states + (chain * p.nseg + seg) * (int64_t)(D * F) : nullptr;
+    // descriptors based at the segment's first row and ending with its last row
+    const float *a_seg = a_ptr + (int64_t)n * p.a_sn + (int64_t)h * p.a_sh + lo * p.a_sl;
+    const float *b_seg = b_ptr + (int64_t)n * p.b_sn + (int64_t)h * p.b_sh + lo * p.b_sl;
+    const float *v_seg = v_ptr + (int64_t)n * p.v_sn + (int64_t)h * p.v_sh + lo * p.v_sl;
+    float *o_seg = out_ptr + (int64_t)n * p.o_sn + (int64_t)h * p.o_sh + lo * p.o_sl;
+    const uint32_t a_sl4 = (uint32_t)p.a_sl * 4u, b_sl4 = (uint32_t)p.b_sl * 4u,
+                   v_sl4 = (uint32_t)p.v_sl * 4u, o_sl4 = (uint32_t)p.o_sl * 4u;
+    const __amdgpu_buffer_rsrc_t a_rs = __builtin_amdgcn_make_buffer_rsrc(
+        (void *)a_seg, 0, (rows - 1) * a_sl4 + D * 4, kRsrcFlags);
+    const __amdgpu_buffer_rsrc_t b_rs = __builtin_amdgcn_make_buffer_rsrc(
+        (void *)b_seg, 0, (rows - 1) * b_sl4 + D * 4, kRsrcFlags);
+    const __amdgpu_buffer_rsrc_t v_rs = __builtin_amdgcn_make_buffer_rsrc(
+        (void *)v_seg, 0, (rows - 1) * v_sl4 + F * 4, kRsrcFlags);
+    const __amdgpu_buffer_rsrc_t o_rs = __builtin_amdgcn_make_buffer_rsrc(
+        (void *)o_seg, 0, (rows - 1) * o_sl4 + F * 4, kRsrcFlags);
 
-    f32x16 S[DT][FT];
+    // per-lane byte offsets inside a chunk
+    const uint32_t a_lane = ln * a_sl4 + 16u * g;
+    uint32_t b_lane[BLK_B], v_lane[BLK_V];
+    int b_jb[BLK_B], b_dq[BLK_B], v_jb[BLK_V], v_fq[BLK_V];
 #pragma unroll
-    for (int dt = 0; dt < DT; dt++)
+    for (int u = 0; u < BLK_B; u++) {
+        const int id = lane + kWave * u;
+        b_jb[u] = id / (D / 4);
+        b_dq[u] = id % (D / 4);
+        b_lane[u] = 4u * b_jb[u] * b_sl4 + 16u * b_dq[u];
+    }
 #pragma unroll
-        for (int ft = 0; ft < FT; ft++) {
-            if (full && p.nseg > 1) {
-#pragma unroll
-                for (int r = 0; r < 16; r++)
-                    S[dt][ft][r] = my_state[((dt * FT + ft) * 16 + r) * kWave + lane];
-            } else {
-#pragma unroll
-                for (int r = 0; r < 16; r++) S[dt][ft][r] = 0.f;
-            }
-        }
+    for (int u = 0; u < BLK_V; u++) {
+        const int id = lane + kWave * u;
+        v_jb[u] = id / (F / 4);
+        v_fq[u] = id % (F / 4);
+        v_lane[u] = 4u * v_jb[u] * v_sl4 + 16u * v_fq[u];
+    }
+    const uint32_t o_lane = ln * o_sl4 + 16u * g;
 
-    // raw fp32 of the chunk being staged
-    float4 a_raw[KD][2];
-    float4 b_raw[BLK_B][4];
-    float4 v_raw[BLK_V][4];
-    const float4 zero4 = make_float4(0.f, 0.f, 0.f, 0.f);
+    // first row of chunk c relative to the segment (REV walks down from the end and its
+    // last chunk may start before the segment: those rows read as zero)
+    auto chunk_row0 = [&](int c) -> int { return REV ? rows - kChunk * (c + 1) : kChunk * c; };
 
-    auto chunk_start = [&](int c) -> int64_t {
-        return REV ? hi - (int64_t)kChunk * (c + 1) : lo + (int64_t)kChunk * c;
+    Raw raw;
+    auto fetch_bv = [&](int row0) {
+#pragma unroll
+        for (int u = 0; u < BLK_B; u++)
+#pragma unroll
+            for (int t = 0; t < 4; t++)
+                raw.b[u][t] = buffer_load4(b_rs, b_lane[u] + (uint32_t)(row0 + t) * b_sl4);
+#pragma unroll
+        for (int u = 0; u < BLK_V; u++)
+#pragma unroll
+            for (int t = 0; t < 4; t++)
+                raw.v[u][t] = buffer_load4(v_rs, v_lane[u] + (uint32_t)(row0 + t) * v_sl4);
     };
-    auto load_chunk = [&](int64_t t0) {
-        if (full) {
-            const int64_t t = t0 + ln;
-            const bool ok = t >= lo && t < hi;
-            const float *row = a_base + t * p.a_sl;
+    auto fetch_a = [&](int row0) {
+        const uint32_t off = a_lane + (uint32_t)row0 * a_sl4;
 #pragma unroll
-            for (int ks = 0; ks < KD; ks++) {
-                a_raw[ks][0] = ok ? *(const float4 *)(row + 16 * ks + 4 * g) : zero4;
-                a_raw[ks][1] = ok ? *(const float4 *)(row + 16 * ks + 8 + 4 * g) : zero4;
-            }
-        }
-#pragma unroll
-        for (int u = 0; u < BLK_B; u++) {
-            const int id = lane + kWave * u;
-            const int jb = id / (D / 4), dq = id % (D / 4);
-#pragma unroll
-            for (int t = 0; t < 4; t++) {
-                const int64_t tok = t0 + 4 * jb + t;
-                const bool ok = tok >= lo && tok < hi;
-                b_raw[u][t] = ok ? *(const float4 *)(b_base + tok * p.b_sl + 4 * dq) : zero4;
-            }
-        }
-#pragma unroll
-        for (int u = 0; u < BLK_V; u++) {
-            const int id = lane + kWave * u;
-            const int jb = id / (F / 4), fq = id % (F / 4);
-#pragma unroll
-            for (int t = 0; t < 4; t++) {
-                const int64_t tok = t0 + 4 * jb + t;
-                const bool ok = tok >= lo && tok < hi;
-                v_raw[u][t] = ok ? *(const float4 *)(v_base + tok * p.v_sl + 4 * fq) : zero4;
-            }
+        for (int ks = 0; ks < KD; ks++) {
+            raw.a[ks][0] = buffer_load4(a_rs, off + 64u * ks);
+            raw.a[ks][1] = buffer_load4(a_rs, off + 64u * ks + 32u);
         }
     };
 
-    const int nchunks = (int)((hi - lo + kChunk - 1) / kChunk);
-    if (nchunks > 0) load_chunk(chunk_start(0));
-
-    for (int c = 0; c < nchunks; c++) {
-        const int64_t t0 = chunk_start(c);
-
-        // ---- stage b (row and transposed layouts) and v (transposed) as bf16 pieces ----
+    // split the fetched b and v rows into bf16 pieces and store them to LDS
+    auto stage_bv = [&](bool with_rows) {
 #pragma unroll
         for (int u = 0; u < BLK_B; u++) {
-            const int id = lane + kWave * u;
-            const int jb = id / (D / 4), dq = id % (D / 4);
+            const int jb = b_jb[u], dq = b_dq[u];
             const float xs[4][4] = {
-                {b_raw[u][0].x, b_raw[u][0].y, b_raw[u][0].z, b_raw[u][0].w},
-                {b_raw[u][1].x, b_raw[u][1].y, b_raw[u][1].z, b_raw[u][1].w},
-                {b_raw[u][2].x, b_raw[u][2].y, b_raw[u][2].z, b_raw[u][2].w},
-                {b_raw[u][3].x, b_raw[u][3].y, b_raw[u][3].z, b_raw[u][3].w}};
-            // pieces packed along d (for B_s rows) ...
-            uint32_t row_lo[4][NS], row_hi[4][NS];
+                {raw.b[u][0].x, raw.b[u][0].y, raw.b[u][0].z, raw.b[u][0].w},
+                {raw.b[u][1].x, raw.b[u][1].y, raw.b[u][1].z, raw.b[u][1].w},
+                {raw.b[u][2].x, raw.b[u][2].y, raw.b[u][2].z, raw.b[u][2].w},
+                {raw.b[u][3].x, raw.b[u][3].y, raw.b[u][3].z, raw.b[u][3].w}};
+            uint32_t row_lo[4][NS], row_hi[4][NS];  // pieces packed along d
 #pragma unroll
             for (int t = 0; t < 4; t++) {
                 split_pair<NS>(xs[t][0], xs[t][1], row_lo[t]);
                 split_pair<NS>(xs[t][2], xs[t][3], row_hi[t]);
             }
-            if (full) {
+            if (with_rows) {
 #pragma unroll
                 for (int t = 0; t < 4; t++)
 #pragma unroll
@@ -246,23 +314,18 @@ __global__ __launch_bounds__(kWave) void scan_mfma_kernel(MfmaArgs p) {
                         *(lds_u32x2 *)dst = lds_u32x2{row_lo[t][pl], row_hi[t][pl]};
                     }
             }
-            // ... and along j (for Bt_s rows): same pieces, regrouped by 16-bit halves
+            // the same pieces regrouped along j for the transposed tile
 #pragma unroll
             for (int cdx = 0; cdx < 4; cdx++)
 #pragma unroll
                 for (int pl = 0; pl < NS; pl++) {
-                    uint32_t w0, w1;
                     const uint32_t s0 = (cdx < 2) ? row_lo[0][pl] : row_hi[0][pl];
                     const uint32_t s1 = (cdx < 2) ? row_lo[1][pl] : row_hi[1][pl];
                     const uint32_t s2 = (cdx < 2) ? row_lo[2][pl] : row_hi[2][pl];
                     const uint32_t s3 = (cdx < 2) ? row_lo[3][pl] : row_hi[3][pl];
-                    if ((cdx & 1) == 0) {  // low halves
-                        w0 = __builtin_amdgcn_perm(s1, s0, 0x05040100u);
-                        w1 = __builtin_amdgcn_perm(s3, s2, 0x05040100u);
-                    } else {  // high halves
-                        w0 = __builtin_amdgcn_perm(s1, s0, 0x07060302u);
-                        w1 = __builtin_amdgcn_perm(s3, s2, 0x07060302u);
-                    }
+                    const uint32_t sel = (cdx & 1) ? 0x07060302u : 0x05040100u;
+                    const uint32_t w0 = __builtin_amdgcn_perm(s1, s0, sel);
+                    const uint32_t w1 = __builtin_amdgcn_perm(s3, s2, sel);
                     unsigned char *dst = lds + Lay::kOffBt + (4 * dq + cdx) * Lay::kRowT +
                                          pl * kChunk * 2 + perm4(4 * jb) * 2;
                     *(lds_u32x2 *)dst = lds_u32x2{w0, w1};
@@ -270,13 +333,12 @@ __global__ __launch_bounds__(kWave) void scan_mfma_kernel(MfmaArgs p) {
         }
 #pragma unroll
         for (int u = 0; u < BLK_V; u++) {
-            const int id = lane + kWave * u;
-            const int jb = id / (F / 4), fq = id % (F / 4);
+            const int jb = v_jb[u], fq = v_fq[u];
             const float xs[4][4] = {
-                {v_raw[u][0].x, v_raw[u][0].y, v_raw[u][0].z, v_raw[u][0].w},
-                {v_raw[u][1].x, v_raw[u][1].y, v_raw[u][1].z, v_raw[u][1].w},
-                {v_raw[u][2].x, v_raw[u][2].y, v_raw[u][2].z, v_raw[u][2].w},
-                {v_raw[u][3].x, v_raw[u][3].y, v_raw[u][3].z, v_raw[u][3].w}};
+                {raw.v[u][0].x, raw.v[u][0].y, raw.v[u][0].z, raw.v[u][0].w},
+                {raw.v[u][1].x, raw.v[u][1].y, raw.v[u][1].z, raw.v[u][1].w},
+                {raw.v[u][2].x, raw.v[u][2].y, raw.v[u][2].z, raw.v[u][2].w},
+                {raw.v[u][3].x, raw.v[u][3].y, raw.v[u][3].z, raw.v[u][3].w}};
 #pragma unroll
             for (int cdx = 0; cdx < 4; cdx++) {
                 uint32_t o01[NS], o23[NS];
@@ -290,28 +352,9 @@ __global__ __launch_bounds__(kWave) void scan_mfma_kernel(MfmaArgs p) {
                 }
             }
         }
+    };
 
-        // ---- a: straight into B-operand fragments ----
-        Frag a_frag[KD][NS];
-        if (full) {
-#pragma unroll
-            for (int ks = 0; ks < KD; ks++) {
-                const float x[8] = {a_raw[ks][0].x, a_raw[ks][0].y, a_raw[ks][0].z, a_raw[ks][0].w,
-                                    a_raw[ks][1].x, a_raw[ks][1].y, a_raw[ks][1].z, a_raw[ks][1].w};
-                split8<NS>(x, a_frag[ks]);
-            }
-        }
-
-        // raw registers are free again: fetch the next chunk while this one is computed
-        if (c + 1 < nchunks) load_chunk(chunk_start(c + 1));
-
-        // single wavefront: LDS writes above are ordered before the reads below
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-
-        // fragments of vt: A operand of (2a) and B operand of (3)
-        Frag v_frag[FT][2][NS];
+    auto load_v_frags = [&](Frag (&v_frag)[FT][2][NS]) {
 #pragma unroll
         for (int ft = 0; ft < FT; ft++)
 #pragma unroll
@@ -323,70 +366,11 @@ __global__ __launch_bounds__(kWave) void scan_mfma_kernel(MfmaArgs p) {
                     const lds_u32x4 q = *(const lds_u32x4 *)src;
                     v_frag[ft][hh][pl] = Frag{{q.x, q.y, q.z, q.w}};
                 }
+    };
 
-        if (full) {
-            // (1) Pt = b a^T
-            f32x16 P;
-#pragma unroll
-            for (int r = 0; r < 16; r++) P[r] = 0.f;
-#pragma unroll
-            for (int ks = 0; ks < KD; ks++) {
-                Frag bA[NS];
-#pragma unroll
-                for (int pl = 0; pl < NS; pl++) {
-                    const unsigned char *src = lds + Lay::kOffB + ln * Lay::kRowB + pl * D * 2 +
-                                               (16 * ks + 8 * g) * 2;
-                    const lds_u32x4 q = *(const lds_u32x4 *)src;
-                    bA[pl] = Frag{{q.x, q.y, q.z, q.w}};
-                }
-                P = mfma_split<NS>(bA, a_frag[ks], P);
-            }
-            // causal mask inside the chunk: row j = 8*(r/4) + 4*g + r%4, column i = ln
-#pragma unroll
-            for (int r = 0; r < 16; r++) {
-                const int j = 8 * (r / 4) + 4 * g + (r % 4);
-                const bool keep = REV ? (j >= ln) : (j <= ln);
-                P[r] = keep ? P[r] : 0.f;
-            }
-            Frag p_frag[2][NS];
-#pragma unroll
-            for (int hh = 0; hh < 2; hh++) {
-                const float x[8] = {P[8 * hh + 0], P[8 * hh + 1], P[8 * hh + 2], P[8 * hh + 3],
-                                    P[8 * hh + 4], P[8 * hh + 5], P[8 * hh + 6], P[8 * hh + 7]};
-                split8<NS>(x, p_frag[hh]);
-            }
-
-            // (2a) + (2b) per output tile, then store
-            const int64_t tok = t0 + ln;
-            const bool row_ok = tok >= lo && tok < hi;
-#pragma unroll
-            for (int ft = 0; ft < FT; ft++) {
-                f32x16 O;
-#pragma unroll
-                for (int r = 0; r < 16; r++) O[r] = 0.f;
-#pragma unroll
-                for (int ks = 0; ks < KD; ks++) {
-                    const float x[8] = {S[ks / 2][ft][8 * (ks % 2) + 0], S[ks / 2][ft][8 * (ks % 2) + 1],
-                                        S[ks / 2][ft][8 * (ks % 2) + 2], S[ks / 2][ft][8 * (ks % 2) + 3],
-                                        S[ks / 2][ft][8 * (ks % 2) + 4], S[ks / 2][ft][8 * (ks % 2) + 5],
-                                        S[ks / 2][ft][8 * (ks % 2) + 6], S[ks / 2][ft][8 * (ks % 2) + 7]};
-                    Frag s_frag[NS];
-                    split8<NS>(x, s_frag);
-                    O = mfma_split<NS>(s_frag, a_frag[ks], O);
-                }
-#pragma unroll
-                for (int hh = 0; hh < 2; hh++) O = mfma_split<NS>(v_frag[ft][hh], p_frag[hh], O);
-                if (row_ok) {
-                    float *orow = o_base + tok * p.o_sl + 32 * ft + 4 * g;
-#pragma unroll
-                    for (int q = 0; q < 4; q++)
-                        *(float4 *)(orow + 8 * q) =
-                            make_float4(O[4 * q + 0], O[4 * q + 1], O[4 * q + 2], O[4 * q + 3]);
-                }
-            }
-        }
-
-        // (3) S += b^T v
+    f32x16 S[DT][FT];
+    // (3) S += b^T v from the staged tiles
+    auto update_state = [&](const Frag (&v_frag)[FT][2][NS]) {
 #pragma unroll
         for (int hh = 0; hh < 2; hh++)
 #pragma unroll
@@ -403,85 +387,276 @@ __global__ __launch_bounds__(kWave) void scan_mfma_kernel(MfmaArgs p) {
                 for (int ft = 0; ft < FT; ft++)
                     S[dt][ft] = mfma_split<NS>(btA, v_frag[ft][hh], S[dt][ft]);
             }
+    };
 
-        // the next iteration overwrites the LDS tiles read above
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-    }
+#pragma unroll
+    for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+        for (int ft = 0; ft < FT; ft++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) S[dt][ft][r] = 0.f;
 
-    if (p.state_only) {
+    if (p.nseg > 1) {
+        // ---- pass 1: the segment's own state sum (the last segment in dependency order
+        // has no reader and skips it) ----
+        const bool publish = step + 1 < p.nseg;
+        if (publish) {
+            fetch_bv(chunk_row0(0));
+            for (int c = 0; c < nchunks; c++) {
+                stage_bv(false);
+                if (c + 1 < nchunks) fetch_bv(chunk_row0(c + 1));
+                wave_lds_fence();
+                Frag v_frag[FT][2][NS];
+                load_v_frags(v_frag);
+                update_state(v_frag);
+                wave_lds_fence();
+            }
+            gfloat *slot = sums + (int64_t)ticket * kStateElems;
+#pragma unroll
+            for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+                for (int ft = 0; ft < FT; ft++)
+#pragma unroll
+                    for (int r = 0; r < 16; r++)
+                        slot[((dt * FT + ft) * 16 + r) * kWave + lane] = S[dt][ft][r];
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+            if (lane == 0)
+                __hip_atomic_store(flags + ticket, kFlagSum, __ATOMIC_RELEASE,
+                                   __HIP_MEMORY_SCOPE_AGENT);
+        }
+        // start fetching the first chunk of pass 2 before waiting
+        fetch_a(chunk_row0(0));
+        fetch_bv(chunk_row0(0));
+
+        // ---- decoupled look-back: state before this segment ----
+        f32x16 X[DT][FT];  // exclusive prefix
 #pragma unroll
         for (int dt = 0; dt < DT; dt++)
 #pragma unroll
             for (int ft = 0; ft < FT; ft++)
 #pragma unroll
-                for (int r = 0; r < 16; r++)
-                    my_state[((dt * FT + ft) * 16 + r) * kWave + lane] = S[dt][ft][r];
+                for (int r = 0; r < 16; r++) X[dt][ft][r] = 0.f;
+        bool failed = false;
+        int spins = 0;
+        for (int back = 1; back <= step; back++) {
+            const uint32_t pred = ticket - back;
+            uint32_t f = kFlagEmpty;
+            while (true) {
+                f = __hip_atomic_load(flags + pred, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT);
+                if (f != kFlagEmpty) break;
+                if (++spins > kSpinLimit) {
+                    failed = true;
+                    break;
+                }
+                __builtin_amdgcn_s_sleep(2);
+            }
+            if (failed) break;
+            const gfloat *src = (f == kFlagPrefix ? prefixes : sums) + (int64_t)pred * kStateElems;
+#pragma unroll
+            for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+                for (int ft = 0; ft < FT; ft++)
+#pragma unroll
+                    for (int r = 0; r < 16; r++)
+                        X[dt][ft][r] += src[((dt * FT + ft) * 16 + r) * kWave + lane];
+            if (f == kFlagPrefix) break;
+        }
+        if (failed && lane == 0)
+            __hip_atomic_store(hdr + kHdrError, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (publish) {
+            gfloat *slot = prefixes + (int64_t)ticket * kStateElems;
+#pragma unroll
+            for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+                for (int ft = 0; ft < FT; ft++)
+#pragma unroll
+                    for (int r = 0; r < 16; r++)
+                        slot[((dt * FT + ft) * 16 + r) * kWave + lane] = X[dt][ft][r] + S[dt][ft][r];
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+            if (lane == 0)
+                __hip_atomic_store(flags + ticket, kFlagPrefix, __ATOMIC_RELEASE,
+                                   __HIP_MEMORY_SCOPE_AGENT);
+        }
+#pragma unroll
+        for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+            for (int ft = 0; ft < FT; ft++) S[dt][ft] = X[dt][ft];
+    } else {
+        fetch_a(chunk_row0(0));
+        fetch_bv(chunk_row0(0));
     }
-}
 
-// In place: states[chain][s] <- sum over s' < s (s' > s when reversed); any element order.
-__global__ __launch_bounds__(256) void state_scan_kernel(float *states, int nseg, int64_t elems,
-                                                         int reverse) {
-    const int64_t blocks_per_chain = (elems + 255) / 256;
-    const int64_t chain = blockIdx.x / blocks_per_chain;
-    const int64_t e = (blockIdx.x % blocks_per_chain) * 256 + threadIdx.x;
-    if (e >= elems) return;
-    float *base = states + chain * nseg * elems + e;
-    float run = 0.f;
-    for (int i = 0; i < nseg; i++) {
-        const int s = reverse ? nseg - 1 - i : i;
-        const float x = base[(int64_t)s * elems];
-        base[(int64_t)s * elems] = run;
-        run += x;
+    // ---- pass 2: outputs ----
+    for (int c = 0; c < nchunks; c++) {
+        const int row0 = chunk_row0(c);
+        stage_bv(true);
+        Frag a_frag[KD][NS];  // B-operand fragments of a, straight from the fetched rows
+#pragma unroll
+        for (int ks = 0; ks < KD; ks++) {
+            const float x[8] = {raw.a[ks][0].x, raw.a[ks][0].y, raw.a[ks][0].z, raw.a[ks][0].w,
+                                raw.a[ks][1].x, raw.a[ks][1].y, raw.a[ks][1].z, raw.a[ks][1].w};
+            split8<NS>(x, a_frag[ks]);
+        }
+        // the raw registers are free again: fetch the next chunk while this one is computed
+        if (c + 1 < nchunks) {
+            fetch_a(chunk_row0(c + 1));
+            fetch_bv(chunk_row0(c + 1));
+        }
+        wave_lds_fence();
+
+        Frag v_frag[FT][2][NS];  // A operand of (2a), B operand of (3)
+        load_v_frags(v_frag);
+
+        // (1) Pt = b a^T
+        f32x16 P;
+#pragma unroll
+        for (int r = 0; r < 16; r++) P[r] = 0.f;
+#pragma unroll
+        for (int ks = 0; ks < KD; ks++) {
+            Frag bA[NS];
+#pragma unroll
+            for (int pl = 0; pl < NS; pl++) {
+                const unsigned char *src =
+                    lds + Lay::kOffB + ln * Lay::kRowB + pl * D * 2 + (16 * ks + 8 * g) * 2;
+                const lds_u32x4 q = *(const lds_u32x4 *)src;
+                bA[pl] = Frag{{q.x, q.y, q.z, q.w}};
+            }
+            P = mfma_split<NS>(bA, a_frag[ks], P);
+        }
+        // causal mask inside the chunk: row j = 8*(r/4) + 4*g + r%4, column i = ln
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            const int j = 8 * (r / 4) + 4 * g + (r % 4);
+            const bool keep = REV ? (j >= ln) : (j <= ln);
+            P[r] = keep ? P[r] : 0.f;
+        }
+        Frag p_frag[2][NS];
+#pragma unroll
+        for (int hh = 0; hh < 2; hh++) {
+            const float x[8] = {P[8 * hh + 0], P[8 * hh + 1], P[8 * hh + 2], P[8 * hh + 3],
+                                P[8 * hh + 4], P[8 * hh + 5], P[8 * hh + 6], P[8 * hh + 7]};
+            split8<NS>(x, p_frag[hh]);
+        }
+
+        // (2b) + (2a) per output tile, then store
+        const uint32_t o_off = o_lane + (uint32_t)row0 * o_sl4;
+#pragma unroll
+        for (int ft = 0; ft < FT; ft++) {
+            f32x16 O;
+#pragma unroll
+            for (int r = 0; r < 16; r++) O[r] = 0.f;
+#pragma unroll
+            for (int ks = 0; ks < KD; ks++) {
+                const int o8 = 8 * (ks % 2);
+                const float x[8] = {S[ks / 2][ft][o8 + 0], S[ks / 2][ft][o8 + 1],
+                                    S[ks / 2][ft][o8 + 2], S[ks / 2][ft][o8 + 3],
+                                    S[ks / 2][ft][o8 + 4], S[ks / 2][ft][o8 + 5],
+                                    S[ks / 2][ft][o8 + 6], S[ks / 2][ft][o8 + 7]};
+                Frag s_frag[NS];
+                split8<NS>(x, s_frag);
+                O = mfma_split<NS>(s_frag, a_frag[ks], O);
+            }
+#pragma unroll
+            for (int hh = 0; hh < 2; hh++) O = mfma_split<NS>(v_frag[ft][hh], p_frag[hh], O);
+            // lane (i = ln, g) holds f = 32*ft + 8*q + 4*g + 0..3 in registers 4q..4q+3
+#pragma unroll
+            for (int q = 0; q < 4; q++)
+                buffer_store4(o_rs, o_off + 128u * ft + 32u * q, O[4 * q + 0], O[4 * q + 1],
+                              O[4 * q + 2], O[4 * q + 3]);
+        }
+
+        update_state(v_frag);
+        wave_lds_fence();
+    }
+
+    // ---- the last wavefront to finish leaves the workspace zeroed for the next launch ----
+    if (p.nseg > 1) {
+        uint32_t done = 0;
+        if (lane == 0)
+            done = __hip_atomic_fetch_add(hdr + kHdrDone, 1u, __ATOMIC_ACQ_REL,
+                                          __HIP_MEMORY_SCOPE_AGENT);
+        done = __builtin_amdgcn_readfirstlane(done);
+        if (done == (uint32_t)p.total_waves - 1) {
+            for (int i = lane; i < p.total_waves; i += kWave)
+                __hip_atomic_store(flags + i, kFlagEmpty, __ATOMIC_RELAXED,
+                                   __HIP_MEMORY_SCOPE_AGENT);
+            if (lane == 0) {
+                __hip_atomic_store(hdr + kHdrTicket, 0u, __ATOMIC_RELAXED,
+                                   __HIP_MEMORY_SCOPE_AGENT);
+                __hip_atomic_store(hdr + kHdrDone, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+        }
     }
 }
 
 struct MfmaPlan {
     int nseg, seg_len;
-    int64_t workspace_bytes;
+    int64_t waves, workspace_bytes;
 };
 
 MfmaPlan make_plan(int64_t N, int64_t H, int64_t L, int64_t D, int64_t F) {
     MfmaPlan pl;
     const int64_t chains = std::max<int64_t>(1, N * H);
-    // one wavefront per SIMD is what the LDS footprint allows: aim for ~2 waves of work
-    // per SIMD (2048 wavefronts) with segments of at least 4 chunks
-    int64_t want = (2048 + chains - 1) / chains;
-    int64_t max_seg = std::max<int64_t>(1, L / (4 * kChunk));
-    int64_t nseg = std::max<int64_t>(1, std::min(want, max_seg));
-    int64_t seg_len = (L + nseg - 1) / nseg;
-    seg_len = (seg_len + kChunk - 1) / kChunk * kChunk;
-    nseg = std::max<int64_t>(1, (L + seg_len - 1) / seg_len);
-    pl.nseg = (int)nseg;
-    pl.seg_len = (int)seg_len;
-    pl.workspace_bytes = nseg > 1 ? chains * nseg * D * F * (int64_t)sizeof(float) : 0;
+    const int64_t total_chunks = (L + kChunk - 1) / kChunk;
+    // One wavefront per SIMD is resident (LDS footprint): 1024 slots.  Pick the segment
+    // length (in chunks) that minimises an estimate of the makespan: rounds of resident
+    // wavefronts times the work of one wavefront (pass 1 costs about a third of pass 2,
+    // the look-back about two chunks).
+    int64_t best_c = total_chunks;
+    double best_cost = (double)total_chunks * (double)((chains + 1023) / 1024);
+    for (int64_t c = 1; c < total_chunks && c <= 4096; c++) {
+        const int64_t nseg = (total_chunks + c - 1) / c;
+        const int64_t waves = chains * nseg;
+        if (waves > kMaxWaves) continue;
+        const double rounds = (double)((waves + 1023) / 1024);
+        const double per_wave = nseg > 1 ? c * 1.35 + 2.0 : (double)c;
+        const double cost = rounds * per_wave;
+        if (cost < best_cost - 1e-9) {
+            best_cost = cost;
+            best_c = c;
+        }
+    }
+    pl.seg_len = (int)(best_c * kChunk);
+    pl.nseg = (int)((L + pl.seg_len - 1) / pl.seg_len);
+    pl.waves = chains * pl.nseg;
+    pl.workspace_bytes = 0;
+    if (pl.nseg > 1)
+        pl.workspace_bytes = kControlBytes + 2 * pl.waves * D * F * (int64_t)sizeof(float);
     return pl;
 }
 
 template <int D, int F>
-void launch(const MfmaArgs &args, int64_t wgs, bool reverse, hipStream_t stream) {
+void launch(const Operand &a, const Operand &b, const Operand &v, const OperandOut &out,
+            void *workspace, const ScanArgs &args, bool reverse, hipStream_t stream) {
+    const dim3 grid((unsigned)args.total_waves), block(kWave);
     if (reverse)
-        hipLaunchKernelGGL((scan_mfma_kernel<D, F, 3, true>), dim3((unsigned)wgs), dim3(kWave), 0,
-                           stream, args);
+        hipLaunchKernelGGL((scan_mfma_kernel<D, F, 3, true>), grid, block, 0, stream,
+                           (const float *)a.ptr, (const float *)b.ptr, (const float *)v.ptr,
+                           (float *)out.ptr, (uint32_t *)workspace, args);
     else
-        hipLaunchKernelGGL((scan_mfma_kernel<D, F, 3, false>), dim3((unsigned)wgs), dim3(kWave), 0,
-                           stream, args);
+        hipLaunchKernelGGL((scan_mfma_kernel<D, F, 3, false>), grid, block, 0, stream,
+                           (const float *)a.ptr, (const float *)b.ptr, (const float *)v.ptr,
+                           (float *)out.ptr, (uint32_t *)workspace, args);
 }
 
 bool aligned16(const void *ptr, int64_t s0, int64_t s1, int64_t s2) {
     return ((uintptr_t)ptr % 16 == 0) && s0 % 4 == 0 && s1 % 4 == 0 && s2 % 4 == 0;
 }
 
+// row strides must keep a segment's byte extent inside a 32-bit buffer descriptor
+bool stride_ok(int64_t stride_l) { return stride_l > 0 && stride_l <= (1 << 16); }
+
 }  // namespace
 
 bool mfma_scan_supported(const Operand &a, const Operand &b, const Operand &v,
-                         const OperandOut &out) {
+                         const OperandOut &out, int64_t L) {
     const int D = a.width, F = v.width;
     const bool shape_ok = (D == 64 && F == 64) || (D == 32 && F == 128) || (D == 128 && F == 32);
     if (!shape_ok) return false;
     if (a.dtype != FTC_F32 || b.dtype != FTC_F32 || v.dtype != FTC_F32 || out.dtype != FTC_F32)
+        return false;
+    if (L > 1 && !(stride_ok(a.stride_l) && stride_ok(b.stride_l) && stride_ok(v.stride_l) &&
+                   stride_ok(out.stride_l)))
         return false;
     return aligned16(a.ptr, a.stride_n, a.stride_h, a.stride_l) &&
            aligned16(b.ptr, b.stride_n, b.stride_h, b.stride_l) &&
@@ -501,16 +676,16 @@ int mfma_scan(const Operand &a, const Operand &b, const Operand &v, const Operan
     if (pl.workspace_bytes > 0 && (!workspace || workspace_bytes < (size_t)pl.workspace_bytes))
         return fail(FTC_ERR_WORKSPACE, "workspace of %lld bytes needed, %zu given",
                     (long long)pl.workspace_bytes, workspace_bytes);
-    const int64_t chains = N * H;
-    const int64_t wgs = chains * pl.nseg;
-    if (wgs > 0x7fffffffLL) return fail(FTC_ERR_UNSUPPORTED, "too many workgroups");
+    if (pl.waves > 0x3fffffffLL) return fail(FTC_ERR_UNSUPPORTED, "too many wavefronts");
+    if (pl.workspace_bytes > 0 && (uintptr_t)workspace % 256 != 0)
+        return fail(FTC_ERR_WORKSPACE, "workspace must be 256-byte aligned");
+    // buffer descriptors address a segment with 32-bit byte offsets
+    const int64_t max_stride = std::max(std::max(a.stride_l, b.stride_l),
+                                        std::max(v.stride_l, out.stride_l));
+    if ((int64_t)(pl.seg_len + kChunk) * max_stride * 4 >= 0x7fffffffLL)
+        return fail(FTC_ERR_UNSUPPORTED, "segment too long for 32-bit offsets");
 
-    MfmaArgs args;
-    args.a = (const float *)a.ptr;
-    args.b = (const float *)b.ptr;
-    args.v = (const float *)v.ptr;
-    args.out = (float *)out.ptr;
-    args.states = pl.nseg > 1 ? (float *)workspace : nullptr;
+    ScanArgs args;
     args.a_sn = a.stride_n, args.a_sh = a.stride_h, args.a_sl = a.stride_l;
     args.b_sn = b.stride_n, args.b_sh = b.stride_h, args.b_sl = b.stride_l;
     args.v_sn = v.stride_n, args.v_sh = v.stride_h, args.v_sl = v.stride_l;
@@ -519,22 +694,14 @@ int mfma_scan(const Operand &a, const Operand &b, const Operand &v, const Operan
     args.H = (int32_t)H;
     args.seg_len = pl.seg_len;
     args.nseg = pl.nseg;
+    args.total_waves = (int32_t)pl.waves;
 
-    auto run = [&](const MfmaArgs &x) {
-        if (D == 64 && F == 64) launch<64, 64>(x, wgs, reverse, stream);
-        else if (D == 32 && F == 128) launch<32, 128>(x, wgs, reverse, stream);
-        else launch<128, 32>(x, wgs, reverse, stream);
-    };
-    if (pl.nseg > 1) {
-        args.state_only = 1;
-        run(args);
-        const int64_t elems = (int64_t)D * F;
-        const int64_t scan_wgs = (elems + 255) / 256 * chains;
-        hipLaunchKernelGGL(state_scan_kernel, dim3((unsigned)scan_wgs), dim3(256), 0, stream,
-                           args.states, pl.nseg, elems, reverse ? 1 : 0);
-    }
-    args.state_only = 0;
-    run(args);
+    if (D == 64 && F == 64)
+        launch<64, 64>(a, b, v, out, workspace, args, reverse, stream);
+    else if (D == 32 && F == 128)
+        launch<32, 128>(a, b, v, out, workspace, args, reverse, stream);
+    else
+        launch<128, 32>(a, b, v, out, workspace, args, reverse, stream);
     hipError_t err = hipGetLastError();
     if (err != hipSuccess)
         return fail(FTC_ERR_HIP, "MFMA scan launch failed: %s", hipGetErrorString(err));

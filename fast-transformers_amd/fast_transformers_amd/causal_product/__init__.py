@@ -44,11 +44,28 @@ def _check_out(t, name):
     return t
 
 
+# One scratch buffer per (device, stream), grown on demand.  The library wants the control
+# block at its start zeroed before the first use and restores it after every call, so the
+# buffer is allocated zero-filled once and then handed to every later call on that stream.
+_workspaces = {}
+
+
 def _workspace(nbytes, device):
     if nbytes <= 0:
         return None, 0
-    ws = torch.empty(nbytes, dtype=torch.uint8, device=device)
-    return ws, nbytes
+    key = (device.index if device.index is not None else torch.cuda.current_device(),
+           torch.cuda.current_stream(device).cuda_stream)
+    ws = _workspaces.get(key)
+    if ws is None or ws.numel() < nbytes:
+        ws = torch.zeros(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
+        _workspaces[key] = ws
+    return ws, ws.numel()
+
+
+def workspace_error_words():
+    """Error word of every cached workspace (synchronises).  All zero unless a wavefront
+    gave up waiting for another one, which a correct launch never does."""
+    return {key: int(ws[8:12].view(torch.int32).item()) for key, ws in _workspaces.items()}
 
 
 def causal_dot_product_hip(queries, keys, values, product):

@@ -25,9 +25,16 @@
  *  - Work is enqueued on `stream` (a hipStream_t; NULL = the default stream)
  *    of the device that owns the pointers and returns without synchronising.
  *  - The library allocates nothing.  Scratch memory comes in through
- *    `workspace` (device memory of at least the number of bytes the matching
+ *    `workspace`: device memory of at least the number of bytes the matching
  *    *_workspace_bytes call returns, 256-byte aligned, private to the call
- *    until the enqueued work has finished).
+ *    until the enqueued work has finished.  Its first
+ *    FTC_WORKSPACE_CONTROL_BYTES bytes are a control block (segment tickets
+ *    and ready flags): they must be zero before the first call that uses the
+ *    buffer and every call leaves them zero again, so one buffer can serve
+ *    any sequence of calls, of any shapes, one at a time.  The rest needs no
+ *    initialisation.  Word 2 of the control block is an error word: it stays
+ *    zero unless a wavefront gave up waiting for another one (which a correct
+ *    launch never does); a caller may read it after synchronising.
  */
 #ifndef FTC_CAUSAL_PRODUCT_H
 #define FTC_CAUSAL_PRODUCT_H
@@ -38,6 +45,8 @@
 #ifdef __cplusplus
 extern "C" {
 #endif
+
+#define FTC_WORKSPACE_CONTROL_BYTES 65536
 
 enum ftc_dtype { FTC_F32 = 0, FTC_BF16 = 1 };
 

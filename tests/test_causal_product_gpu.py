@@ -235,6 +235,14 @@ def test_bf16_inputs_fp32_accumulate(cp):
     assert scale_error(Qg.grad.float().cpu(), refs[0]) <= 2e-2
 
 
+def test_zz_no_wavefront_gave_up_waiting(cp):
+    """Runs after the parity tests: the bounded waits of the look-back never expired."""
+    torch.cuda.synchronize()
+    words = cp.workspace_error_words()
+    assert words, "no workspace was used: the MFMA path did not run"
+    assert all(w == 0 for w in words.values()), words
+
+
 def test_errors_and_empty_inputs(cp):
     Q = torch.rand(1, 2, 8, 4, device="cuda")
     V = torch.rand(1, 2, 8, 6, device="cuda")
