@@ -37,6 +37,7 @@
 // positions outside the segment read as zero and stores to them are dropped, so tails need
 // no branches.
 #include <algorithm>
+#include <cstdlib>
 
 #include "ftc_common.h"
 
@@ -64,7 +65,8 @@ constexpr int kHdrTicket = 0, kHdrDone = 1, kHdrError = 2;
 constexpr int kHdrWords = 64;
 constexpr int kControlBytes = FTC_WORKSPACE_CONTROL_BYTES;
 constexpr int kMaxWaves = (kControlBytes / 4) - kHdrWords;
-constexpr uint32_t kFlagEmpty = 0, kFlagSum = 1, kFlagPrefix = 2;
+constexpr uint32_t kFlagEmpty = 0, kFlagSum = 1, kFlagTotal = 2;
+constexpr int kCoherentAux = 16;  // sc1: the access is performed at agent scope
 
 struct Frag {
     uint32_t w[4];  // 8 bf16, k-slot t in the low (t even) / high (t odd) half of w[t/2]
@@ -137,6 +139,14 @@ __device__ __forceinline__ void buffer_store4(__amdgpu_buffer_rsrc_t rsrc, uint3
     __builtin_amdgcn_raw_buffer_store_b128(r, rsrc, byte_offset, 0, 0);
 }
 
+// States travel between wavefronts (possibly on different XCDs, whose L2s are not coherent
+// with each other) through buffer accesses flagged sc1, which are performed at agent scope
+// themselves.  That keeps cache-wide write-back / invalidate operations out of the kernel:
+// the writer only has to wait for its stores to be acknowledged before it raises the flag.
+__device__ __forceinline__ void wait_for_stores() {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+}
+
 // LDS writes of this wavefront are ordered before its later LDS reads (and the reverse).
 __device__ __forceinline__ void wave_lds_fence() {
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
@@ -152,6 +162,8 @@ struct ScanArgs {
     int64_t L;
     int32_t H, seg_len, nseg;
     int32_t total_waves;
+    int32_t group;  // steps per group of the two-level state sum
+    int32_t use_ticket;
 };
 
 template <int D, int F, int NS>
@@ -198,11 +210,10 @@ __global__ __launch_bounds__(kWave) void scan_mfma_kernel(const float *__restric
     gu32 *hdr = (gu32 *)ws_ptr;
     gu32 *flags = hdr + kHdrWords;
     gfloat *sums = (gfloat *)(hdr + kControlBytes / 4);
-    gfloat *prefixes = sums + (int64_t)p.total_waves * kStateElems;
 
     // ---- which segment: tickets follow the dependency order ----
     uint32_t ticket = 0;
-    if (p.nseg > 1) {
+    if (p.nseg > 1 && p.use_ticket) {
         if (lane == 0)
             ticket = __hip_atomic_fetch_add(hdr + kHdrTicket, 1u, __ATOMIC_RELAXED,
                                             __HIP_MEMORY_SCOPE_AGENT);
@@ -397,86 +408,140 @@ __global__ __launch_bounds__(kWave) void scan_mfma_kernel(const float *__restric
             for (int r = 0; r < 16; r++) S[dt][ft][r] = 0.f;
 
     if (p.nseg > 1) {
-        // ---- pass 1: the segment's own state sum (the last segment in dependency order
-        // has no reader and skips it) ----
-        const bool publish = step + 1 < p.nseg;
-        if (publish) {
-            fetch_bv(chunk_row0(0));
-            for (int c = 0; c < nchunks; c++) {
+        // Segments of a chain form groups of p.group consecutive steps.  The state before
+        // step s is (sum of the totals of the groups before its group) + (sum of the sums
+        // of the steps before it in its group), always added in ascending order, so the
+        // result does not depend on timing.  Every step but the last of its group publishes
+        // its own sum; the last step of every group but the last publishes the group total.
+        const int G = p.group;
+        const int grp = step / G;
+        const int grp_first = grp * G;
+        const int grp_last = min(grp_first + G, p.nseg) - 1;
+        const bool is_last_of_group = step == grp_last;
+        const bool need_own_sum = step + 1 < p.nseg;  // the very last step has no reader
+        const __amdgpu_buffer_rsrc_t st_rs = __builtin_amdgcn_make_buffer_rsrc(
+            (void *)sums, 0, (uint32_t)(2 * p.total_waves) * (uint32_t)(kStateElems * 4),
+            kRsrcFlags);
+        const uint32_t lane16 = 16u * lane;
+        auto slot_offset = [&](uint32_t slot) -> uint32_t { return slot * (kStateElems * 4); };
+        auto publish_state = [&](uint32_t slot, const f32x16 (&T)[DT][FT], uint32_t flag_value) {
+            const uint32_t base = slot_offset(slot) + lane16;
+#pragma unroll
+            for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+                for (int ft = 0; ft < FT; ft++)
+#pragma unroll
+                    for (int q4 = 0; q4 < 4; q4++) {
+                        const u32x4 w = {__float_as_uint(T[dt][ft][4 * q4 + 0]),
+                                         __float_as_uint(T[dt][ft][4 * q4 + 1]),
+                                         __float_as_uint(T[dt][ft][4 * q4 + 2]),
+                                         __float_as_uint(T[dt][ft][4 * q4 + 3])};
+                        __builtin_amdgcn_raw_buffer_store_b128(
+                            w, st_rs, base + (uint32_t)(((dt * FT + ft) * 4 + q4) * kWave * 16), 0,
+                            kCoherentAux);
+                    }
+            wait_for_stores();
+            if (lane == 0)
+                __hip_atomic_store(flags + ticket, flag_value, __ATOMIC_RELAXED,
+                                   __HIP_MEMORY_SCOPE_AGENT);
+        };
+        auto add_state = [&](uint32_t slot, f32x16 (&T)[DT][FT]) {
+            const uint32_t base = slot_offset(slot) + lane16;
+#pragma unroll
+            for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+                for (int ft = 0; ft < FT; ft++)
+#pragma unroll
+                    for (int q4 = 0; q4 < 4; q4++) {
+                        const u32x4 w = __builtin_amdgcn_raw_buffer_load_b128(
+                            st_rs, base + (uint32_t)(((dt * FT + ft) * 4 + q4) * kWave * 16), 0,
+                            kCoherentAux);
+                        T[dt][ft][4 * q4 + 0] += __uint_as_float(w.x);
+                        T[dt][ft][4 * q4 + 1] += __uint_as_float(w.y);
+                        T[dt][ft][4 * q4 + 2] += __uint_as_float(w.z);
+                        T[dt][ft][4 * q4 + 3] += __uint_as_float(w.w);
+                    }
+        };
+        int spins = 0;
+        bool failed = false;
+        // wait until `count` wavefronts, tickets first, first + stride, ..., show `bit`
+        auto wait_flags = [&](uint32_t first, uint32_t stride, int count, uint32_t bit) {
+            const bool mine = lane < count;
+            const gu32 *f = flags + first + stride * (uint32_t)lane;
+            while (!failed) {
+                const uint32_t x =
+                    mine ? __hip_atomic_load(f, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : bit;
+                if (__builtin_amdgcn_ballot_w64((x & bit) == 0) == 0) break;
+                if (++spins > kSpinLimit) failed = true;
+                __builtin_amdgcn_s_sleep(4);
+            }
+        };
+
+        // ---- pass 1: the segment's own state sum, walked against the direction of pass 2
+        // so that pass 2 starts on the rows read last ----
+        if (need_own_sum) {
+            fetch_bv(chunk_row0(nchunks - 1));
+            for (int c = nchunks - 1; c >= 0; c--) {
                 stage_bv(false);
-                if (c + 1 < nchunks) fetch_bv(chunk_row0(c + 1));
+                if (c > 0) fetch_bv(chunk_row0(c - 1));
                 wave_lds_fence();
                 Frag v_frag[FT][2][NS];
                 load_v_frags(v_frag);
                 update_state(v_frag);
                 wave_lds_fence();
             }
-            gfloat *slot = sums + (int64_t)ticket * kStateElems;
-#pragma unroll
-            for (int dt = 0; dt < DT; dt++)
-#pragma unroll
-                for (int ft = 0; ft < FT; ft++)
-#pragma unroll
-                    for (int r = 0; r < 16; r++)
-                        slot[((dt * FT + ft) * 16 + r) * kWave + lane] = S[dt][ft][r];
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
-            if (lane == 0)
-                __hip_atomic_store(flags + ticket, kFlagSum, __ATOMIC_RELEASE,
-                                   __HIP_MEMORY_SCOPE_AGENT);
+            if (!is_last_of_group) publish_state(ticket, S, kFlagSum);
         }
         // start fetching the first chunk of pass 2 before waiting
         fetch_a(chunk_row0(0));
         fetch_bv(chunk_row0(0));
 
-        // ---- decoupled look-back: state before this segment ----
-        f32x16 X[DT][FT];  // exclusive prefix
+        // ---- sums of the earlier steps of this group ----
+        f32x16 X[DT][FT];
 #pragma unroll
         for (int dt = 0; dt < DT; dt++)
 #pragma unroll
             for (int ft = 0; ft < FT; ft++)
 #pragma unroll
                 for (int r = 0; r < 16; r++) X[dt][ft][r] = 0.f;
-        bool failed = false;
-        int spins = 0;
-        for (int back = 1; back <= step; back++) {
-            const uint32_t pred = ticket - back;
-            uint32_t f = kFlagEmpty;
-            while (true) {
-                f = __hip_atomic_load(flags + pred, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT);
-                if (f != kFlagEmpty) break;
-                if (++spins > kSpinLimit) {
-                    failed = true;
-                    break;
-                }
-                __builtin_amdgcn_s_sleep(2);
-            }
-            if (failed) break;
-            const gfloat *src = (f == kFlagPrefix ? prefixes : sums) + (int64_t)pred * kStateElems;
+        const int in_group = step - grp_first;
+        const uint32_t chain_ticket0 = ticket - (uint32_t)step;
+        if (in_group > 0) {
+            wait_flags(chain_ticket0 + grp_first, 1, in_group, kFlagSum);
+            if (!failed)
+                for (int i = 0; i < in_group; i++) add_state(chain_ticket0 + grp_first + i, X);
+        }
+        if (is_last_of_group && need_own_sum && !failed) {
+            // group total = sums of the group in ascending order (own sum last)
 #pragma unroll
             for (int dt = 0; dt < DT; dt++)
 #pragma unroll
-                for (int ft = 0; ft < FT; ft++)
+                for (int ft = 0; ft < FT; ft++) S[dt][ft] = X[dt][ft] + S[dt][ft];
+            publish_state((uint32_t)p.total_waves + ticket, S, kFlagTotal);
+        }
+        // ---- totals of the earlier groups, then the in-group part on top ----
+        if (grp > 0 && !failed) {
+            wait_flags(chain_ticket0 + (uint32_t)(G - 1), (uint32_t)G, grp, kFlagTotal);
+            if (!failed) {
 #pragma unroll
-                    for (int r = 0; r < 16; r++)
-                        X[dt][ft][r] += src[((dt * FT + ft) * 16 + r) * kWave + lane];
-            if (f == kFlagPrefix) break;
+                for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+                    for (int ft = 0; ft < FT; ft++) {
+                        S[dt][ft] = X[dt][ft];
+#pragma unroll
+                        for (int r = 0; r < 16; r++) X[dt][ft][r] = 0.f;
+                    }
+                for (int gq = 0; gq < grp; gq++)
+                    add_state((uint32_t)p.total_waves + chain_ticket0 + (uint32_t)(gq * G + G - 1),
+                              X);
+#pragma unroll
+                for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+                    for (int ft = 0; ft < FT; ft++) X[dt][ft] = X[dt][ft] + S[dt][ft];
+            }
         }
         if (failed && lane == 0)
             __hip_atomic_store(hdr + kHdrError, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        if (publish) {
-            gfloat *slot = prefixes + (int64_t)ticket * kStateElems;
-#pragma unroll
-            for (int dt = 0; dt < DT; dt++)
-#pragma unroll
-                for (int ft = 0; ft < FT; ft++)
-#pragma unroll
-                    for (int r = 0; r < 16; r++)
-                        slot[((dt * FT + ft) * 16 + r) * kWave + lane] = X[dt][ft][r] + S[dt][ft][r];
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
-            if (lane == 0)
-                __hip_atomic_store(flags + ticket, kFlagPrefix, __ATOMIC_RELEASE,
-                                   __HIP_MEMORY_SCOPE_AGENT);
-        }
 #pragma unroll
         for (int dt = 0; dt < DT; dt++)
 #pragma unroll
@@ -573,7 +638,7 @@ __global__ __launch_bounds__(kWave) void scan_mfma_kernel(const float *__restric
     if (p.nseg > 1) {
         uint32_t done = 0;
         if (lane == 0)
-            done = __hip_atomic_fetch_add(hdr + kHdrDone, 1u, __ATOMIC_ACQ_REL,
+            done = __hip_atomic_fetch_add(hdr + kHdrDone, 1u, __ATOMIC_RELAXED,
                                           __HIP_MEMORY_SCOPE_AGENT);
         done = __builtin_amdgcn_readfirstlane(done);
         if (done == (uint32_t)p.total_waves - 1) {
@@ -607,7 +672,7 @@ MfmaPlan make_plan(int64_t N, int64_t H, int64_t L, int64_t D, int64_t F) {
     for (int64_t c = 1; c < total_chunks && c <= 4096; c++) {
         const int64_t nseg = (total_chunks + c - 1) / c;
         const int64_t waves = chains * nseg;
-        if (waves > kMaxWaves) continue;
+        if (waves > kMaxWaves || nseg > 4096) continue;  // 64 groups of 64 steps at most
         const double rounds = (double)((waves + 1023) / 1024);
         const double per_wave = nseg > 1 ? c * 1.35 + 2.0 : (double)c;
         const double cost = rounds * per_wave;
@@ -695,6 +760,12 @@ int mfma_scan(const Operand &a, const Operand &b, const Operand &v, const Operan
     args.seg_len = pl.seg_len;
     args.nseg = pl.nseg;
     args.total_waves = (int32_t)pl.waves;
+    args.group = 1;
+    while (args.group * args.group < pl.nseg) args.group++;
+    {
+        const char *e = getenv("FTC_USE_TICKET");
+        args.use_ticket = e ? atoi(e) : 1;
+    }
 
     if (D == 64 && F == 64)
         launch<64, 64>(a, b, v, out, workspace, args, reverse, stream);
