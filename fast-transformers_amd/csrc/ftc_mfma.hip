@@ -21,23 +21,28 @@
 // Register chaining: a 32x32 accumulator holds, in lane (col = lane % 32, g = lane / 32),
 // rows 8*(r/4) + 4*g + (r%4) for r = 0..15.  Registers 8h..8h+7 are therefore 8 values
 // of the contraction index for k-step h, provided the other operand uses the same order:
-// k-slot (g, t) of a 16-wide k-step carries logical index 8*(t/4) + 4*g + (t%4).  LDS
-// tiles are stored with that order inside every 16-block (blocks of four swapped:
-// 0,2,1,3), so one ds_read_b128 yields a fragment.
+// k-slot (g, t) of a 16-wide k-step carries logical index 8*(t/4) + 4*g + (t%4).
+//
+// No LDS: every operand fragment is loaded from global memory directly in the register
+// layout its MFMA wants.  Row-major fragments (a, and b for (1)) are two 16-byte loads per
+// k-step; position-major fragments (b for (3), v) are 4-byte loads in which the 32 lanes
+// of a half-wave read 32 consecutive floats of one row, so every load instruction still
+// covers whole 128-byte lines.  b is read in both layouts; the second read hits L1/L2.
+// (An earlier version transposed b and v through LDS: bank conflicts took 79 % of its LDS
+// cycles and the write -> wait -> read round trip per chunk could not be hidden with the
+// one wavefront per SIMD that the register budget allows.)
 //
 // One launch per scan.  A wavefront first sums its segment's own state (reading b and v
-// only), publishes it, obtains the state that precedes its segment by decoupled look-back
-// over the published sums of the segments before it, and then replays its segment (the
-// second read of b and v is served by L2 / Infinity Cache).  Segments are handed out in
-// dependency order through a ticket counter, so a wavefront only ever waits for
-// wavefronts that are already running; every wait is bounded and raises an error word
-// instead of spinning forever.
+// only), publishes it, obtains the state that precedes its segment from the published
+// sums of the segments before it (two levels, fixed order), and then replays its segment.
+// The wavefronts launched for a chain take its segments in the order in which they start
+// running, so a wavefront only ever waits for wavefronts that are already running; every
+// wait is bounded and raises an error word instead of spinning forever.
 //
 // Rows are fetched with raw buffer loads whose descriptor ends at the segment's last row:
 // positions outside the segment read as zero and stores to them are dropped, so tails need
 // no branches.
 #include <algorithm>
-#include <cstdlib>
 
 #include "ftc_common.h"
 
@@ -47,9 +52,6 @@ namespace {
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-// LDS is written as 8-byte and read as 16-byte words of the same bf16 data
-typedef uint32_t lds_u32x2 __attribute__((ext_vector_type(2), may_alias));
-typedef uint32_t lds_u32x4 __attribute__((ext_vector_type(4), may_alias));
 typedef __attribute__((address_space(1))) float gfloat;
 typedef __attribute__((address_space(1))) uint32_t gu32;
 
@@ -61,10 +63,11 @@ constexpr int kSpinLimit = 1 << 20;           // bounded wait (about a second in
 // The workspace starts with a control block of fixed size: a header and one flag word per
 // wavefront.  It must be zero before the first use and every launch leaves it zero, so
 // later calls of any shape can reuse it.  The state slots behind it need no initialisation.
-constexpr int kHdrTicket = 0, kHdrDone = 1, kHdrError = 2;
+constexpr int kHdrDone = 1, kHdrError = 2;
 constexpr int kHdrWords = 64;
 constexpr int kControlBytes = FTC_WORKSPACE_CONTROL_BYTES;
-constexpr int kMaxWaves = (kControlBytes / 4) - kHdrWords;
+// words: [header][one flag per wavefront][one ticket counter per chain]
+constexpr int kMaxWaves = ((kControlBytes / 4) - kHdrWords) / 2;
 constexpr uint32_t kFlagEmpty = 0, kFlagSum = 1, kFlagTotal = 2;
 constexpr int kCoherentAux = 16;  // sc1: the access is performed at agent scope
 
@@ -121,17 +124,13 @@ __device__ __forceinline__ f32x16 mfma_split(const Frag (&a)[NS], const Frag (&b
     return acc;
 }
 
-// position of logical index x (a multiple of 4) inside its 16-block: blocks 0,1,2,3 -> 0,2,1,3
-__device__ __forceinline__ int perm4(int x) {
-    const int blk = (x >> 2) & 3;
-    const int swapped = ((blk & 1) << 1) | (blk >> 1);
-    return (x & ~15) | (swapped << 2);
-}
-
 __device__ __forceinline__ float4 buffer_load4(__amdgpu_buffer_rsrc_t rsrc, uint32_t byte_offset) {
     const u32x4 r = __builtin_amdgcn_raw_buffer_load_b128(rsrc, byte_offset, 0, 0);
     return make_float4(__uint_as_float(r.x), __uint_as_float(r.y), __uint_as_float(r.z),
                        __uint_as_float(r.w));
+}
+__device__ __forceinline__ float buffer_load1(__amdgpu_buffer_rsrc_t rsrc, uint32_t byte_offset) {
+    return __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(rsrc, byte_offset, 0, 0));
 }
 __device__ __forceinline__ void buffer_store4(__amdgpu_buffer_rsrc_t rsrc, uint32_t byte_offset,
                                               float x, float y, float z, float w) {
@@ -147,13 +146,6 @@ __device__ __forceinline__ void wait_for_stores() {
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 }
 
-// LDS writes of this wavefront are ordered before its later LDS reads (and the reverse).
-__device__ __forceinline__ void wave_lds_fence() {
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-}
-
 struct ScanArgs {
     int64_t a_sn, a_sh, a_sl;
     int64_t b_sn, b_sh, b_sl;
@@ -163,30 +155,6 @@ struct ScanArgs {
     int32_t H, seg_len, nseg;
     int32_t total_waves;
     int32_t group;  // steps per group of the two-level state sum
-    int32_t use_ticket;
-};
-
-template <int D, int F, int NS>
-struct Lds {
-    // per row: NS planes of the row's bf16 values, then 16 bytes of padding (keeps the row
-    // pitch at 4 (mod 8) dwords so that ds_read_b128 by 8 consecutive rows is conflict free)
-    static constexpr int kRowB = NS * D * 2 + 16;       // B_s[j][plane][pos(d)]
-    static constexpr int kRowT = NS * kChunk * 2 + 16;  // Bt_s[d][plane][pos(j)], Vt_s[f][..]
-    static constexpr int kOffB = 0;
-    static constexpr int kOffBt = kOffB + kChunk * kRowB;
-    static constexpr int kOffVt = kOffBt + D * kRowT;
-    static constexpr int kBytes = kOffVt + F * kRowT;
-};
-
-// Raw rows of one chunk held between the fetch and the split.
-template <int D, int F>
-struct RawChunk {
-    static constexpr int KD = D / 16;
-    static constexpr int BLK_B = (kChunk / 4) * (D / 4) / kWave;  // 4x4 blocks of b per lane
-    static constexpr int BLK_V = (kChunk / 4) * (F / 4) / kWave;
-    float4 a[KD][2];
-    float4 b[BLK_B][4];
-    float4 v[BLK_V][4];
 };
 
 template <int D, int F, int NS, bool REV>
@@ -196,13 +164,9 @@ __global__ __launch_bounds__(kWave) void scan_mfma_kernel(const float *__restric
                                                           float *__restrict__ out_ptr,
                                                           uint32_t *__restrict__ ws_ptr,
                                                           ScanArgs p) {
-    using Lay = Lds<D, F, NS>;
-    using Raw = RawChunk<D, F>;
     constexpr int DT = D / 32, FT = F / 32;  // state tiles
     constexpr int KD = D / 16;               // k-steps over d
-    constexpr int BLK_B = Raw::BLK_B, BLK_V = Raw::BLK_V;
     constexpr int kStateElems = D * F;
-    __shared__ __align__(16) unsigned char lds[Lay::kBytes];
 
     const int lane = threadIdx.x;
     const int ln = lane & 31, g = lane >> 5;
@@ -211,14 +175,19 @@ __global__ __launch_bounds__(kWave) void scan_mfma_kernel(const float *__restric
     gu32 *flags = hdr + kHdrWords;
     gfloat *sums = (gfloat *)(hdr + kControlBytes / 4);
 
-    // ---- which segment: tickets follow the dependency order ----
+    // ---- which segment: the wavefronts launched for a chain take that chain's steps in
+    // the order in which they start running, so a step only ever waits for steps that are
+    // already running ----
     uint32_t ticket = 0;
-    if (p.nseg > 1 && p.use_ticket) {
+    if (p.nseg > 1) {
+        const uint32_t my_chain = blockIdx.x / (uint32_t)p.nseg;
+        uint32_t order = 0;
         if (lane == 0)
-            ticket = __hip_atomic_fetch_add(hdr + kHdrTicket, 1u, __ATOMIC_RELAXED,
-                                            __HIP_MEMORY_SCOPE_AGENT);
-        ticket = __builtin_amdgcn_readfirstlane(ticket);
-        if (ticket >= (uint32_t)p.total_waves) {
+            order = __hip_atomic_fetch_add(flags + kMaxWaves + my_chain, 1u, __ATOMIC_RELAXED,
+                                           __HIP_MEMORY_SCOPE_AGENT);
+        order = __builtin_amdgcn_readfirstlane(order);
+        ticket = my_chain * (uint32_t)p.nseg + order;
+        if (order >= (uint32_t)p.nseg) {
             // the control block was not zero when the launch started: refuse to run on it
             if (lane == 0)
                 __hip_atomic_store(hdr + kHdrError, 2u, __ATOMIC_RELAXED,
@@ -254,150 +223,75 @@ __global__ __launch_bounds__(kWave) void scan_mfma_kernel(const float *__restric
         (void *)o_seg, 0, (rows - 1) * o_sl4 + F * 4, kRsrcFlags);
 
     // per-lane byte offsets inside a chunk
+    //  row-major fragments: lane (row = ln, g) reads 4 floats at column 16*ks + 4*g (+8)
+    //  position-major fragments: lane (col = ln, g), k-slot t of k-step hh is row
+    //  16*hh + 8*(t/4) + 4*g + (t%4)
     const uint32_t a_lane = ln * a_sl4 + 16u * g;
-    uint32_t b_lane[BLK_B], v_lane[BLK_V];
-    int b_jb[BLK_B], b_dq[BLK_B], v_jb[BLK_V], v_fq[BLK_V];
-#pragma unroll
-    for (int u = 0; u < BLK_B; u++) {
-        const int id = lane + kWave * u;
-        b_jb[u] = id / (D / 4);
-        b_dq[u] = id % (D / 4);
-        b_lane[u] = 4u * b_jb[u] * b_sl4 + 16u * b_dq[u];
-    }
-#pragma unroll
-    for (int u = 0; u < BLK_V; u++) {
-        const int id = lane + kWave * u;
-        v_jb[u] = id / (F / 4);
-        v_fq[u] = id % (F / 4);
-        v_lane[u] = 4u * v_jb[u] * v_sl4 + 16u * v_fq[u];
-    }
+    const uint32_t b_lane = ln * b_sl4 + 16u * g;
+    const uint32_t bt_lane = 4u * g * b_sl4 + 4u * ln;
+    const uint32_t vt_lane = 4u * g * v_sl4 + 4u * ln;
     const uint32_t o_lane = ln * o_sl4 + 16u * g;
 
     // first row of chunk c relative to the segment (REV walks down from the end and its
     // last chunk may start before the segment: those rows read as zero)
     auto chunk_row0 = [&](int c) -> int { return REV ? rows - kChunk * (c + 1) : kChunk * c; };
 
-    Raw raw;
-    auto fetch_bv = [&](int row0) {
-#pragma unroll
-        for (int u = 0; u < BLK_B; u++)
-#pragma unroll
-            for (int t = 0; t < 4; t++)
-                raw.b[u][t] = buffer_load4(b_rs, b_lane[u] + (uint32_t)(row0 + t) * b_sl4);
-#pragma unroll
-        for (int u = 0; u < BLK_V; u++)
-#pragma unroll
-            for (int t = 0; t < 4; t++)
-                raw.v[u][t] = buffer_load4(v_rs, v_lane[u] + (uint32_t)(row0 + t) * v_sl4);
-    };
-    auto fetch_a = [&](int row0) {
-        const uint32_t off = a_lane + (uint32_t)row0 * a_sl4;
+    // raw fp32 of the chunk being fetched
+    float4 a_raw[KD][2];   // a rows, B operand of (1) and (2b)
+    float4 b_raw[KD][2];   // b rows, A operand of (1)
+    float bt_raw[DT][2][8];  // b by position, A operand of (3)
+    float vt_raw[FT][2][8];  // v by position, A operand of (2a), B operand of (3)
+
+    auto fetch_rows = [&](__amdgpu_buffer_rsrc_t rs, uint32_t lane_off, uint32_t sl4, int row0,
+                          float4 (&raw)[KD][2]) {
+        const uint32_t off = lane_off + (uint32_t)row0 * sl4;
 #pragma unroll
         for (int ks = 0; ks < KD; ks++) {
-            raw.a[ks][0] = buffer_load4(a_rs, off + 64u * ks);
-            raw.a[ks][1] = buffer_load4(a_rs, off + 64u * ks + 32u);
+            raw[ks][0] = buffer_load4(rs, off + 64u * ks);
+            raw[ks][1] = buffer_load4(rs, off + 64u * ks + 32u);
         }
     };
-
-    // split the fetched b and v rows into bf16 pieces and store them to LDS
-    auto stage_bv = [&](bool with_rows) {
+    auto fetch_bt = [&](int row0) {
+        const uint32_t off = bt_lane + (uint32_t)row0 * b_sl4;
 #pragma unroll
-        for (int u = 0; u < BLK_B; u++) {
-            const int jb = b_jb[u], dq = b_dq[u];
-            const float xs[4][4] = {
-                {raw.b[u][0].x, raw.b[u][0].y, raw.b[u][0].z, raw.b[u][0].w},
-                {raw.b[u][1].x, raw.b[u][1].y, raw.b[u][1].z, raw.b[u][1].w},
-                {raw.b[u][2].x, raw.b[u][2].y, raw.b[u][2].z, raw.b[u][2].w},
-                {raw.b[u][3].x, raw.b[u][3].y, raw.b[u][3].z, raw.b[u][3].w}};
-            uint32_t row_lo[4][NS], row_hi[4][NS];  // pieces packed along d
+        for (int dt = 0; dt < DT; dt++)
 #pragma unroll
-            for (int t = 0; t < 4; t++) {
-                split_pair<NS>(xs[t][0], xs[t][1], row_lo[t]);
-                split_pair<NS>(xs[t][2], xs[t][3], row_hi[t]);
-            }
-            if (with_rows) {
+            for (int hh = 0; hh < 2; hh++)
 #pragma unroll
-                for (int t = 0; t < 4; t++)
-#pragma unroll
-                    for (int pl = 0; pl < NS; pl++) {
-                        unsigned char *dst = lds + Lay::kOffB + (4 * jb + t) * Lay::kRowB +
-                                             pl * D * 2 + perm4(4 * dq) * 2;
-                        *(lds_u32x2 *)dst = lds_u32x2{row_lo[t][pl], row_hi[t][pl]};
-                    }
-            }
-            // the same pieces regrouped along j for the transposed tile
-#pragma unroll
-            for (int cdx = 0; cdx < 4; cdx++)
-#pragma unroll
-                for (int pl = 0; pl < NS; pl++) {
-                    const uint32_t s0 = (cdx < 2) ? row_lo[0][pl] : row_hi[0][pl];
-                    const uint32_t s1 = (cdx < 2) ? row_lo[1][pl] : row_hi[1][pl];
-                    const uint32_t s2 = (cdx < 2) ? row_lo[2][pl] : row_hi[2][pl];
-                    const uint32_t s3 = (cdx < 2) ? row_lo[3][pl] : row_hi[3][pl];
-                    const uint32_t sel = (cdx & 1) ? 0x07060302u : 0x05040100u;
-                    const uint32_t w0 = __builtin_amdgcn_perm(s1, s0, sel);
-                    const uint32_t w1 = __builtin_amdgcn_perm(s3, s2, sel);
-                    unsigned char *dst = lds + Lay::kOffBt + (4 * dq + cdx) * Lay::kRowT +
-                                         pl * kChunk * 2 + perm4(4 * jb) * 2;
-                    *(lds_u32x2 *)dst = lds_u32x2{w0, w1};
-                }
-        }
-#pragma unroll
-        for (int u = 0; u < BLK_V; u++) {
-            const int jb = v_jb[u], fq = v_fq[u];
-            const float xs[4][4] = {
-                {raw.v[u][0].x, raw.v[u][0].y, raw.v[u][0].z, raw.v[u][0].w},
-                {raw.v[u][1].x, raw.v[u][1].y, raw.v[u][1].z, raw.v[u][1].w},
-                {raw.v[u][2].x, raw.v[u][2].y, raw.v[u][2].z, raw.v[u][2].w},
-                {raw.v[u][3].x, raw.v[u][3].y, raw.v[u][3].z, raw.v[u][3].w}};
-#pragma unroll
-            for (int cdx = 0; cdx < 4; cdx++) {
-                uint32_t o01[NS], o23[NS];
-                split_pair<NS>(xs[0][cdx], xs[1][cdx], o01);
-                split_pair<NS>(xs[2][cdx], xs[3][cdx], o23);
-#pragma unroll
-                for (int pl = 0; pl < NS; pl++) {
-                    unsigned char *dst = lds + Lay::kOffVt + (4 * fq + cdx) * Lay::kRowT +
-                                         pl * kChunk * 2 + perm4(4 * jb) * 2;
-                    *(lds_u32x2 *)dst = lds_u32x2{o01[pl], o23[pl]};
-                }
-            }
-        }
+                for (int t = 0; t < 8; t++)
+                    bt_raw[dt][hh][t] = buffer_load1(
+                        b_rs, off + (uint32_t)(16 * hh + 8 * (t / 4) + (t % 4)) * b_sl4 + 128u * dt);
     };
-
-    auto load_v_frags = [&](Frag (&v_frag)[FT][2][NS]) {
+    auto fetch_vt = [&](int row0) {
+        const uint32_t off = vt_lane + (uint32_t)row0 * v_sl4;
 #pragma unroll
         for (int ft = 0; ft < FT; ft++)
 #pragma unroll
             for (int hh = 0; hh < 2; hh++)
 #pragma unroll
-                for (int pl = 0; pl < NS; pl++) {
-                    const unsigned char *src = lds + Lay::kOffVt + (32 * ft + ln) * Lay::kRowT +
-                                               pl * kChunk * 2 + (16 * hh + 8 * g) * 2;
-                    const lds_u32x4 q = *(const lds_u32x4 *)src;
-                    v_frag[ft][hh][pl] = Frag{{q.x, q.y, q.z, q.w}};
-                }
+                for (int t = 0; t < 8; t++)
+                    vt_raw[ft][hh][t] = buffer_load1(
+                        v_rs, off + (uint32_t)(16 * hh + 8 * (t / 4) + (t % 4)) * v_sl4 + 128u * ft);
+    };
+    auto split_rows = [&](const float4 (&raw)[KD][2], Frag (&frag)[KD][NS]) {
+#pragma unroll
+        for (int ks = 0; ks < KD; ks++) {
+            const float x[8] = {raw[ks][0].x, raw[ks][0].y, raw[ks][0].z, raw[ks][0].w,
+                                raw[ks][1].x, raw[ks][1].y, raw[ks][1].z, raw[ks][1].w};
+            split8<NS>(x, frag[ks]);
+        }
     };
 
     f32x16 S[DT][FT];
-    // (3) S += b^T v from the staged tiles
-    auto update_state = [&](const Frag (&v_frag)[FT][2][NS]) {
+    // (3) S += b^T v
+    auto update_state = [&](const Frag (&bt_frag)[DT][2][NS], const Frag (&v_frag)[FT][2][NS]) {
 #pragma unroll
         for (int hh = 0; hh < 2; hh++)
 #pragma unroll
-            for (int dt = 0; dt < DT; dt++) {
-                Frag btA[NS];
-#pragma unroll
-                for (int pl = 0; pl < NS; pl++) {
-                    const unsigned char *src = lds + Lay::kOffBt + (32 * dt + ln) * Lay::kRowT +
-                                               pl * kChunk * 2 + (16 * hh + 8 * g) * 2;
-                    const lds_u32x4 q = *(const lds_u32x4 *)src;
-                    btA[pl] = Frag{{q.x, q.y, q.z, q.w}};
-                }
+            for (int dt = 0; dt < DT; dt++)
 #pragma unroll
                 for (int ft = 0; ft < FT; ft++)
-                    S[dt][ft] = mfma_split<NS>(btA, v_frag[ft][hh], S[dt][ft]);
-            }
+                    S[dt][ft] = mfma_split<NS>(bt_frag[dt][hh], v_frag[ft][hh], S[dt][ft]);
     };
 
 #pragma unroll
@@ -447,19 +341,24 @@ __global__ __launch_bounds__(kWave) void scan_mfma_kernel(const float *__restric
         };
         auto add_state = [&](uint32_t slot, f32x16 (&T)[DT][FT]) {
             const uint32_t base = slot_offset(slot) + lane16;
+            // all loads of a state are in flight together, then added in a fixed order
+            u32x4 w[DT * FT * 4];
+#pragma unroll
+            for (int i = 0; i < DT * FT * 4; i++)
+                w[i] = __builtin_amdgcn_raw_buffer_load_b128(
+                    st_rs, base + (uint32_t)(i * kWave * 16), 0, kCoherentAux);
+            __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int dt = 0; dt < DT; dt++)
 #pragma unroll
                 for (int ft = 0; ft < FT; ft++)
 #pragma unroll
                     for (int q4 = 0; q4 < 4; q4++) {
-                        const u32x4 w = __builtin_amdgcn_raw_buffer_load_b128(
-                            st_rs, base + (uint32_t)(((dt * FT + ft) * 4 + q4) * kWave * 16), 0,
-                            kCoherentAux);
-                        T[dt][ft][4 * q4 + 0] += __uint_as_float(w.x);
-                        T[dt][ft][4 * q4 + 1] += __uint_as_float(w.y);
-                        T[dt][ft][4 * q4 + 2] += __uint_as_float(w.z);
-                        T[dt][ft][4 * q4 + 3] += __uint_as_float(w.w);
+                        const u32x4 x = w[(dt * FT + ft) * 4 + q4];
+                        T[dt][ft][4 * q4 + 0] += __uint_as_float(x.x);
+                        T[dt][ft][4 * q4 + 1] += __uint_as_float(x.y);
+                        T[dt][ft][4 * q4 + 2] += __uint_as_float(x.z);
+                        T[dt][ft][4 * q4 + 3] += __uint_as_float(x.w);
                     }
         };
         int spins = 0;
@@ -480,21 +379,31 @@ __global__ __launch_bounds__(kWave) void scan_mfma_kernel(const float *__restric
         // ---- pass 1: the segment's own state sum, walked against the direction of pass 2
         // so that pass 2 starts on the rows read last ----
         if (need_own_sum) {
-            fetch_bv(chunk_row0(nchunks - 1));
+            fetch_bt(chunk_row0(nchunks - 1));
+            fetch_vt(chunk_row0(nchunks - 1));
             for (int c = nchunks - 1; c >= 0; c--) {
-                stage_bv(false);
-                if (c > 0) fetch_bv(chunk_row0(c - 1));
-                wave_lds_fence();
-                Frag v_frag[FT][2][NS];
-                load_v_frags(v_frag);
-                update_state(v_frag);
-                wave_lds_fence();
+                Frag bt_frag[DT][2][NS], v_frag[FT][2][NS];
+#pragma unroll
+                for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+                    for (int hh = 0; hh < 2; hh++) split8<NS>(bt_raw[dt][hh], bt_frag[dt][hh]);
+#pragma unroll
+                for (int ft = 0; ft < FT; ft++)
+#pragma unroll
+                    for (int hh = 0; hh < 2; hh++) split8<NS>(vt_raw[ft][hh], v_frag[ft][hh]);
+                if (c > 0) {
+                    fetch_bt(chunk_row0(c - 1));
+                    fetch_vt(chunk_row0(c - 1));
+                }
+                update_state(bt_frag, v_frag);
             }
             if (!is_last_of_group) publish_state(ticket, S, kFlagSum);
         }
         // start fetching the first chunk of pass 2 before waiting
-        fetch_a(chunk_row0(0));
-        fetch_bv(chunk_row0(0));
+        fetch_rows(a_rs, a_lane, a_sl4, chunk_row0(0), a_raw);
+        fetch_rows(b_rs, b_lane, b_sl4, chunk_row0(0), b_raw);
+        fetch_vt(chunk_row0(0));
+        fetch_bt(chunk_row0(0));
 
         // ---- sums of the earlier steps of this group ----
         f32x16 X[DT][FT];
@@ -547,47 +456,34 @@ __global__ __launch_bounds__(kWave) void scan_mfma_kernel(const float *__restric
 #pragma unroll
             for (int ft = 0; ft < FT; ft++) S[dt][ft] = X[dt][ft];
     } else {
-        fetch_a(chunk_row0(0));
-        fetch_bv(chunk_row0(0));
+        fetch_rows(a_rs, a_lane, a_sl4, chunk_row0(0), a_raw);
+        fetch_rows(b_rs, b_lane, b_sl4, chunk_row0(0), b_raw);
+        fetch_vt(chunk_row0(0));
+        fetch_bt(chunk_row0(0));
     }
 
     // ---- pass 2: outputs ----
     for (int c = 0; c < nchunks; c++) {
         const int row0 = chunk_row0(c);
-        stage_bv(true);
-        Frag a_frag[KD][NS];  // B-operand fragments of a, straight from the fetched rows
-#pragma unroll
-        for (int ks = 0; ks < KD; ks++) {
-            const float x[8] = {raw.a[ks][0].x, raw.a[ks][0].y, raw.a[ks][0].z, raw.a[ks][0].w,
-                                raw.a[ks][1].x, raw.a[ks][1].y, raw.a[ks][1].z, raw.a[ks][1].w};
-            split8<NS>(x, a_frag[ks]);
-        }
-        // the raw registers are free again: fetch the next chunk while this one is computed
-        if (c + 1 < nchunks) {
-            fetch_a(chunk_row0(c + 1));
-            fetch_bv(chunk_row0(c + 1));
-        }
-        wave_lds_fence();
+        const bool more = c + 1 < nchunks;
+        const int next0 = chunk_row0(c + 1);
 
-        Frag v_frag[FT][2][NS];  // A operand of (2a), B operand of (3)
-        load_v_frags(v_frag);
+        // each operand is cut into pieces as soon as it is needed and its raw registers
+        // are refilled with the next chunk right away
+        Frag a_frag[KD][NS], b_frag[KD][NS];
+        split_rows(a_raw, a_frag);
+        split_rows(b_raw, b_frag);
+        if (more) {
+            fetch_rows(a_rs, a_lane, a_sl4, next0, a_raw);
+            fetch_rows(b_rs, b_lane, b_sl4, next0, b_raw);
+        }
 
         // (1) Pt = b a^T
         f32x16 P;
 #pragma unroll
         for (int r = 0; r < 16; r++) P[r] = 0.f;
 #pragma unroll
-        for (int ks = 0; ks < KD; ks++) {
-            Frag bA[NS];
-#pragma unroll
-            for (int pl = 0; pl < NS; pl++) {
-                const unsigned char *src =
-                    lds + Lay::kOffB + ln * Lay::kRowB + pl * D * 2 + (16 * ks + 8 * g) * 2;
-                const lds_u32x4 q = *(const lds_u32x4 *)src;
-                bA[pl] = Frag{{q.x, q.y, q.z, q.w}};
-            }
-            P = mfma_split<NS>(bA, a_frag[ks], P);
-        }
+        for (int ks = 0; ks < KD; ks++) P = mfma_split<NS>(b_frag[ks], a_frag[ks], P);
         // causal mask inside the chunk: row j = 8*(r/4) + 4*g + r%4, column i = ln
 #pragma unroll
         for (int r = 0; r < 16; r++) {
@@ -602,6 +498,13 @@ __global__ __launch_bounds__(kWave) void scan_mfma_kernel(const float *__restric
                                 P[8 * hh + 4], P[8 * hh + 5], P[8 * hh + 6], P[8 * hh + 7]};
             split8<NS>(x, p_frag[hh]);
         }
+
+        Frag v_frag[FT][2][NS];  // A operand of (2a), B operand of (3)
+#pragma unroll
+        for (int ft = 0; ft < FT; ft++)
+#pragma unroll
+            for (int hh = 0; hh < 2; hh++) split8<NS>(vt_raw[ft][hh], v_frag[ft][hh]);
+        if (more) fetch_vt(next0);
 
         // (2b) + (2a) per output tile, then store
         const uint32_t o_off = o_lane + (uint32_t)row0 * o_sl4;
@@ -630,8 +533,13 @@ __global__ __launch_bounds__(kWave) void scan_mfma_kernel(const float *__restric
                               O[4 * q + 2], O[4 * q + 3]);
         }
 
-        update_state(v_frag);
-        wave_lds_fence();
+        Frag bt_frag[DT][2][NS];
+#pragma unroll
+        for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+            for (int hh = 0; hh < 2; hh++) split8<NS>(bt_raw[dt][hh], bt_frag[dt][hh]);
+        if (more) fetch_bt(next0);
+        update_state(bt_frag, v_frag);
     }
 
     // ---- the last wavefront to finish leaves the workspace zeroed for the next launch ----
@@ -645,11 +553,11 @@ __global__ __launch_bounds__(kWave) void scan_mfma_kernel(const float *__restric
             for (int i = lane; i < p.total_waves; i += kWave)
                 __hip_atomic_store(flags + i, kFlagEmpty, __ATOMIC_RELAXED,
                                    __HIP_MEMORY_SCOPE_AGENT);
-            if (lane == 0) {
-                __hip_atomic_store(hdr + kHdrTicket, 0u, __ATOMIC_RELAXED,
+            for (int i = lane; i < p.total_waves / p.nseg; i += kWave)
+                __hip_atomic_store(flags + kMaxWaves + i, 0u, __ATOMIC_RELAXED,
                                    __HIP_MEMORY_SCOPE_AGENT);
+            if (lane == 0)
                 __hip_atomic_store(hdr + kHdrDone, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            }
         }
     }
 }
@@ -708,8 +616,9 @@ bool aligned16(const void *ptr, int64_t s0, int64_t s1, int64_t s2) {
     return ((uintptr_t)ptr % 16 == 0) && s0 % 4 == 0 && s1 % 4 == 0 && s2 % 4 == 0;
 }
 
+// rows must not overlap (the descriptor's end marks the first row outside the segment) and
 // row strides must keep a segment's byte extent inside a 32-bit buffer descriptor
-bool stride_ok(int64_t stride_l) { return stride_l > 0 && stride_l <= (1 << 16); }
+bool stride_ok(int64_t stride_l, int width) { return stride_l >= width && stride_l <= (1 << 16); }
 
 }  // namespace
 
@@ -720,8 +629,8 @@ bool mfma_scan_supported(const Operand &a, const Operand &b, const Operand &v,
     if (!shape_ok) return false;
     if (a.dtype != FTC_F32 || b.dtype != FTC_F32 || v.dtype != FTC_F32 || out.dtype != FTC_F32)
         return false;
-    if (L > 1 && !(stride_ok(a.stride_l) && stride_ok(b.stride_l) && stride_ok(v.stride_l) &&
-                   stride_ok(out.stride_l)))
+    if (L > 1 && !(stride_ok(a.stride_l, D) && stride_ok(b.stride_l, D) &&
+                   stride_ok(v.stride_l, F) && stride_ok(out.stride_l, F)))
         return false;
     return aligned16(a.ptr, a.stride_n, a.stride_h, a.stride_l) &&
            aligned16(b.ptr, b.stride_n, b.stride_h, b.stride_l) &&
@@ -760,11 +669,12 @@ int mfma_scan(const Operand &a, const Operand &b, const Operand &v, const Operan
     args.seg_len = pl.seg_len;
     args.nseg = pl.nseg;
     args.total_waves = (int32_t)pl.waves;
-    args.group = 1;
-    while (args.group * args.group < pl.nseg) args.group++;
-    {
-        const char *e = getenv("FTC_USE_TICKET");
-        args.use_ticket = e ? atoi(e) : 1;
+    // short chains: one level (every step adds the sums of all steps before it); long
+    // chains: groups of about sqrt(nseg) steps
+    args.group = pl.nseg;
+    if (pl.nseg > 16) {
+        args.group = 1;
+        while (args.group * args.group < pl.nseg) args.group++;
     }
 
     if (D == 64 && F == 64)
