@@ -69,18 +69,37 @@ int read_dims(const ftc_tensor4 *q, const ftc_tensor4 *v, Dims *d) {
     return FTC_OK;
 }
 
-// Picks the MFMA scan when the operands qualify, else the generic scan.
-int scan(const Operand &a, const Operand &b, const Operand &v, const OperandOut &out, int64_t N,
-         int64_t H, int64_t L, bool reverse, void *workspace, size_t workspace_bytes,
-         hipStream_t stream) {
-    if (mfma_scan_supported(a, b, v, out, L))
-        return mfma_scan(a, b, v, out, N, H, L, reverse, workspace, workspace_bytes, stream);
-    return generic_scan(a, b, v, out, N, H, L, reverse, workspace, workspace_bytes, stream);
+// Runs a list of independent scans: consecutive scans that qualify for the MFMA path and
+// share their row widths go out in one launch, the rest through the generic path.
+int run_scans(const ScanDesc *scans, int n, int64_t N, int64_t H, int64_t L, void *workspace,
+              size_t workspace_bytes, hipStream_t stream) {
+    int i = 0;
+    while (i < n) {
+        if (mfma_scan_supported(scans[i], L)) {
+            int k = 1;
+            while (i + k < n && k < kMfmaMaxScans && mfma_scan_supported(scans[i + k], L) &&
+                   scans[i + k].a.width == scans[i].a.width &&
+                   scans[i + k].v.width == scans[i].v.width)
+                k++;
+            int rc = mfma_scan(scans + i, k, N, H, L, workspace, workspace_bytes, stream);
+            if (rc) return rc;
+            i += k;
+        } else {
+            int rc = generic_scan(scans[i].a, scans[i].b, scans[i].v, scans[i].out, N, H, L,
+                                  scans[i].reverse, workspace, workspace_bytes, stream);
+            if (rc) return rc;
+            i++;
+        }
+    }
+    return FTC_OK;
 }
 
+// Upper bound over every way run_scans may group scans of these widths.
 int64_t scan_workspace_bytes(int64_t N, int64_t H, int64_t L, int64_t D, int64_t F) {
-    return std::max(generic_scan_workspace_bytes(N, H, L, D, F),
-                    mfma_scan_workspace_bytes(N, H, L, D, F));
+    int64_t need = generic_scan_workspace_bytes(N, H, L, D, F);
+    for (int k = 1; k <= kMfmaMaxScans; k++)
+        need = std::max(need, mfma_scan_workspace_bytes(N, H, L, D, F, k));
+    return need;
 }
 
 }  // namespace
@@ -119,8 +138,9 @@ int ftc_causal_dot_product(const ftc_tensor4 *queries, const ftc_tensor4 *keys,
     hipStream_t s = (hipStream_t)stream;
     if (d.E == 0)  // an empty contraction: every product row is zero
         return zero_rows(as_operand_out(product), d.N, d.H, d.L, s);
-    return scan(as_operand(queries), as_operand(keys), as_operand(values),
-                as_operand_out(product), d.N, d.H, d.L, false, workspace, workspace_bytes, s);
+    const ScanDesc fwd = {as_operand(queries), as_operand(keys), as_operand(values),
+                          as_operand_out(product), false};
+    return run_scans(&fwd, 1, d.N, d.H, d.L, workspace, workspace_bytes, s);
 }
 
 int64_t ftc_causal_dot_backward_workspace_bytes(int64_t N, int64_t H, int64_t L, int64_t E,
@@ -161,14 +181,12 @@ int ftc_causal_dot_backward(const ftc_tensor4 *queries, const ftc_tensor4 *keys,
     hipStream_t s = (hipStream_t)stream;
     const Operand Q = as_operand(queries), K = as_operand(keys), V = as_operand(values),
                   G = as_operand(grad_out);
-    if ((rc = scan(G, V, K, as_operand_out(grad_queries), d.N, d.H, d.L, false, workspace,
-                   workspace_bytes, s)))
-        return rc;
-    if ((rc = scan(V, G, Q, as_operand_out(grad_keys), d.N, d.H, d.L, true, workspace,
-                   workspace_bytes, s)))
-        return rc;
-    return scan(K, Q, G, as_operand_out(grad_values), d.N, d.H, d.L, true, workspace,
-                workspace_bytes, s);
+    const ScanDesc scans[3] = {
+        {G, V, K, as_operand_out(grad_queries), false},  // dQ: state M x E, walks up
+        {V, G, Q, as_operand_out(grad_keys), true},      // dK: state M x E, walks down
+        {K, Q, G, as_operand_out(grad_values), true},    // dV: state E x M, walks down
+    };
+    return run_scans(scans, 3, d.N, d.H, d.L, workspace, workspace_bytes, s);
 }
 
 }  // extern "C"

@@ -77,12 +77,20 @@ int generic_scan(const Operand &a, const Operand &b, const Operand &v, const Ope
 // MFMA scan (fp32 rows, (D, F) in {(64,64), (32,128), (128,32)}, 16-byte aligned rows):
 // ftc_mfma.hip.  Same contract as generic_scan.
 // ---------------------------------------------------------------------------
-bool mfma_scan_supported(const Operand &a, const Operand &b, const Operand &v,
-                         const OperandOut &out, int64_t L);
-int64_t mfma_scan_workspace_bytes(int64_t N, int64_t H, int64_t L, int64_t D, int64_t F);
-int mfma_scan(const Operand &a, const Operand &b, const Operand &v, const OperandOut &out,
-              int64_t N, int64_t H, int64_t L, bool reverse, void *workspace,
-              size_t workspace_bytes, hipStream_t stream);
+struct ScanDesc {
+    Operand a, b, v;
+    OperandOut out;
+    bool reverse;
+};
+constexpr int kMfmaMaxScans = 3;
+
+bool mfma_scan_supported(const ScanDesc &scan, int64_t L);
+// Workspace for `nscans` scans of one (D, F) run side by side in one launch.
+int64_t mfma_scan_workspace_bytes(int64_t N, int64_t H, int64_t L, int64_t D, int64_t F,
+                                  int nscans);
+// Runs scans[0..nscans) (all of the same row widths) in one launch.
+int mfma_scan(const ScanDesc *scans, int nscans, int64_t N, int64_t H, int64_t L,
+              void *workspace, size_t workspace_bytes, hipStream_t stream);
 
 // Fill every row of `out` with zeros (used for empty contractions).
 int zero_rows(const OperandOut &out, int64_t N, int64_t H, int64_t L, hipStream_t stream);

@@ -146,23 +146,32 @@ __device__ __forceinline__ void wait_for_stores() {
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 }
 
-struct ScanArgs {
+// One scan of a launch.  A launch runs up to kMaxScans independent scans of the same
+// (D, F, N, H, L) side by side (the three gradients of a backward call), so that their
+// launch gaps and wait times overlap.
+struct ScanOperands {
+    const float *a, *b, *v;
+    float *out;
     int64_t a_sn, a_sh, a_sl;
     int64_t b_sn, b_sh, b_sl;
     int64_t v_sn, v_sh, v_sl;
     int64_t o_sn, o_sh, o_sl;
+    int32_t rev;  // 0: j <= l, walk up; 1: j >= l, walk down
+    int32_t pad;
+};
+constexpr int kMaxScans = 3;
+
+struct ScanArgs {
+    ScanOperands scan[kMaxScans];
     int64_t L;
     int32_t H, seg_len, nseg;
-    int32_t total_waves;
-    int32_t group;  // steps per group of the two-level state sum
+    int32_t waves_per_scan;
+    int32_t total_waves;  // nscans * waves_per_scan
+    int32_t group;        // steps per group of the two-level state sum
 };
 
-template <int D, int F, int NS, bool REV>
-__global__ __launch_bounds__(kWave) void scan_mfma_kernel(const float *__restrict__ a_ptr,
-                                                          const float *__restrict__ b_ptr,
-                                                          const float *__restrict__ v_ptr,
-                                                          float *__restrict__ out_ptr,
-                                                          uint32_t *__restrict__ ws_ptr,
+template <int D, int F, int NS>
+__global__ __launch_bounds__(kWave) void scan_mfma_kernel(uint32_t *__restrict__ ws_ptr,
                                                           ScanArgs p) {
     constexpr int DT = D / 32, FT = F / 32;  // state tiles
     constexpr int KD = D / 16;               // k-steps over d
@@ -178,6 +187,12 @@ __global__ __launch_bounds__(kWave) void scan_mfma_kernel(const float *__restric
     // ---- which segment: the wavefronts launched for a chain take that chain's steps in
     // the order in which they start running, so a step only ever waits for steps that are
     // already running ----
+    // chains of all scans are numbered consecutively: global chain = scan * chains + chain
+    const uint32_t scan_id = blockIdx.x / (uint32_t)p.waves_per_scan;
+    const ScanOperands &op = p.scan[scan_id];
+    const bool REV = op.rev != 0;
+    const float *a_ptr = op.a, *b_ptr = op.b, *v_ptr = op.v;
+    float *out_ptr = op.out;
     uint32_t ticket = 0;
     if (p.nseg > 1) {
         const uint32_t my_chain = blockIdx.x / (uint32_t)p.nseg;
@@ -197,7 +212,7 @@ __global__ __launch_bounds__(kWave) void scan_mfma_kernel(const float *__restric
     } else {
         ticket = blockIdx.x;
     }
-    const int64_t chain = ticket / (uint32_t)p.nseg;
+    const int64_t chain = (ticket - scan_id * (uint32_t)p.waves_per_scan) / (uint32_t)p.nseg;
     const int step = (int)(ticket % (uint32_t)p.nseg);      // position in dependency order
     const int seg = REV ? p.nseg - 1 - step : step;
     const int n = (int)(chain / p.H), h = (int)(chain % p.H);
@@ -207,12 +222,12 @@ __global__ __launch_bounds__(kWave) void scan_mfma_kernel(const float *__restric
     const int nchunks = (rows + kChunk - 1) / kChunk;
 
     // descriptors based at the segment's first row and ending with its last row
-    const float *a_seg = a_ptr + (int64_t)n * p.a_sn + (int64_t)h * p.a_sh + lo * p.a_sl;
-    const float *b_seg = b_ptr + (int64_t)n * p.b_sn + (int64_t)h * p.b_sh + lo * p.b_sl;
-    const float *v_seg = v_ptr + (int64_t)n * p.v_sn + (int64_t)h * p.v_sh + lo * p.v_sl;
-    float *o_seg = out_ptr + (int64_t)n * p.o_sn + (int64_t)h * p.o_sh + lo * p.o_sl;
-    const uint32_t a_sl4 = (uint32_t)p.a_sl * 4u, b_sl4 = (uint32_t)p.b_sl * 4u,
-                   v_sl4 = (uint32_t)p.v_sl * 4u, o_sl4 = (uint32_t)p.o_sl * 4u;
+    const float *a_seg = a_ptr + (int64_t)n * op.a_sn + (int64_t)h * op.a_sh + lo * op.a_sl;
+    const float *b_seg = b_ptr + (int64_t)n * op.b_sn + (int64_t)h * op.b_sh + lo * op.b_sl;
+    const float *v_seg = v_ptr + (int64_t)n * op.v_sn + (int64_t)h * op.v_sh + lo * op.v_sl;
+    float *o_seg = out_ptr + (int64_t)n * op.o_sn + (int64_t)h * op.o_sh + lo * op.o_sl;
+    const uint32_t a_sl4 = (uint32_t)op.a_sl * 4u, b_sl4 = (uint32_t)op.b_sl * 4u,
+                   v_sl4 = (uint32_t)op.v_sl * 4u, o_sl4 = (uint32_t)op.o_sl * 4u;
     const __amdgpu_buffer_rsrc_t a_rs = __builtin_amdgcn_make_buffer_rsrc(
         (void *)a_seg, 0, (rows - 1) * a_sl4 + D * 4, kRsrcFlags);
     const __amdgpu_buffer_rsrc_t b_rs = __builtin_amdgcn_make_buffer_rsrc(
@@ -235,6 +250,8 @@ __global__ __launch_bounds__(kWave) void scan_mfma_kernel(const float *__restric
     // first row of chunk c relative to the segment (REV walks down from the end and its
     // last chunk may start before the segment: those rows read as zero)
     auto chunk_row0 = [&](int c) -> int { return REV ? rows - kChunk * (c + 1) : kChunk * c; };
+    // pass 1 walks the chunks downwards; "chunk -1" must lie outside the descriptor
+    auto pass1_row0 = [&](int c) -> int { return c < 0 ? -2 * kChunk : chunk_row0(c); };
 
     // raw fp32 of the chunk being fetched
     float4 a_raw[KD][2];   // a rows, B operand of (1) and (2b)
@@ -391,10 +408,8 @@ __global__ __launch_bounds__(kWave) void scan_mfma_kernel(const float *__restric
                 for (int ft = 0; ft < FT; ft++)
 #pragma unroll
                     for (int hh = 0; hh < 2; hh++) split8<NS>(vt_raw[ft][hh], v_frag[ft][hh]);
-                if (c > 0) {
-                    fetch_bt(chunk_row0(c - 1));
-                    fetch_vt(chunk_row0(c - 1));
-                }
+                fetch_bt(pass1_row0(c - 1));
+                fetch_vt(pass1_row0(c - 1));
                 update_state(bt_frag, v_frag);
             }
             if (!is_last_of_group) publish_state(ticket, S, kFlagSum);
@@ -465,7 +480,8 @@ __global__ __launch_bounds__(kWave) void scan_mfma_kernel(const float *__restric
     // ---- pass 2: outputs ----
     for (int c = 0; c < nchunks; c++) {
         const int row0 = chunk_row0(c);
-        const bool more = c + 1 < nchunks;
+        // rows of the chunk after the last one are outside the descriptor and read as zero,
+        // so the prefetch needs no branch
         const int next0 = chunk_row0(c + 1);
 
         // each operand is cut into pieces as soon as it is needed and its raw registers
@@ -473,10 +489,8 @@ __global__ __launch_bounds__(kWave) void scan_mfma_kernel(const float *__restric
         Frag a_frag[KD][NS], b_frag[KD][NS];
         split_rows(a_raw, a_frag);
         split_rows(b_raw, b_frag);
-        if (more) {
-            fetch_rows(a_rs, a_lane, a_sl4, next0, a_raw);
-            fetch_rows(b_rs, b_lane, b_sl4, next0, b_raw);
-        }
+        fetch_rows(a_rs, a_lane, a_sl4, next0, a_raw);
+        fetch_rows(b_rs, b_lane, b_sl4, next0, b_raw);
 
         // (1) Pt = b a^T
         f32x16 P;
@@ -504,7 +518,7 @@ __global__ __launch_bounds__(kWave) void scan_mfma_kernel(const float *__restric
         for (int ft = 0; ft < FT; ft++)
 #pragma unroll
             for (int hh = 0; hh < 2; hh++) split8<NS>(vt_raw[ft][hh], v_frag[ft][hh]);
-        if (more) fetch_vt(next0);
+        fetch_vt(next0);
 
         // (2b) + (2a) per output tile, then store
         const uint32_t o_off = o_lane + (uint32_t)row0 * o_sl4;
@@ -538,7 +552,7 @@ __global__ __launch_bounds__(kWave) void scan_mfma_kernel(const float *__restric
         for (int dt = 0; dt < DT; dt++)
 #pragma unroll
             for (int hh = 0; hh < 2; hh++) split8<NS>(bt_raw[dt][hh], bt_frag[dt][hh]);
-        if (more) fetch_bt(next0);
+        fetch_bt(next0);
         update_state(bt_frag, v_frag);
     }
 
@@ -567,22 +581,22 @@ struct MfmaPlan {
     int64_t waves, workspace_bytes;
 };
 
-MfmaPlan make_plan(int64_t N, int64_t H, int64_t L, int64_t D, int64_t F) {
+MfmaPlan make_plan(int64_t N, int64_t H, int64_t L, int64_t D, int64_t F, int nscans) {
     MfmaPlan pl;
     const int64_t chains = std::max<int64_t>(1, N * H);
     const int64_t total_chunks = (L + kChunk - 1) / kChunk;
     // One wavefront per SIMD is resident (LDS footprint): 1024 slots.  Pick the segment
     // length (in chunks) that minimises an estimate of the makespan: rounds of resident
-    // wavefronts times the work of one wavefront (pass 1 costs about a third of pass 2,
-    // the look-back about two chunks).
+    // wavefronts times the work of one wavefront (pass 1 costs about half of pass 2, the
+    // exchange of segment sums about three chunks).
     int64_t best_c = total_chunks;
-    double best_cost = (double)total_chunks * (double)((chains + 1023) / 1024);
+    double best_cost = (double)total_chunks * (double)((chains * nscans + 1023) / 1024);
     for (int64_t c = 1; c < total_chunks && c <= 4096; c++) {
         const int64_t nseg = (total_chunks + c - 1) / c;
         const int64_t waves = chains * nseg;
-        if (waves > kMaxWaves || nseg > 4096) continue;  // 64 groups of 64 steps at most
-        const double rounds = (double)((waves + 1023) / 1024);
-        const double per_wave = nseg > 1 ? c * 1.35 + 2.0 : (double)c;
+        if (waves * nscans > kMaxWaves || nseg > 4096) continue;  // <= 64 groups of 64 steps
+        const double rounds = (double)((waves * nscans + 1023) / 1024);
+        const double per_wave = nseg > 1 ? c * 1.5 + 3.0 : (double)c;
         const double cost = rounds * per_wave;
         if (cost < best_cost - 1e-9) {
             best_cost = cost;
@@ -594,22 +608,15 @@ MfmaPlan make_plan(int64_t N, int64_t H, int64_t L, int64_t D, int64_t F) {
     pl.waves = chains * pl.nseg;
     pl.workspace_bytes = 0;
     if (pl.nseg > 1)
-        pl.workspace_bytes = kControlBytes + 2 * pl.waves * D * F * (int64_t)sizeof(float);
+        pl.workspace_bytes =
+            kControlBytes + 2 * nscans * pl.waves * D * F * (int64_t)sizeof(float);
     return pl;
 }
 
 template <int D, int F>
-void launch(const Operand &a, const Operand &b, const Operand &v, const OperandOut &out,
-            void *workspace, const ScanArgs &args, bool reverse, hipStream_t stream) {
-    const dim3 grid((unsigned)args.total_waves), block(kWave);
-    if (reverse)
-        hipLaunchKernelGGL((scan_mfma_kernel<D, F, 3, true>), grid, block, 0, stream,
-                           (const float *)a.ptr, (const float *)b.ptr, (const float *)v.ptr,
-                           (float *)out.ptr, (uint32_t *)workspace, args);
-    else
-        hipLaunchKernelGGL((scan_mfma_kernel<D, F, 3, false>), grid, block, 0, stream,
-                           (const float *)a.ptr, (const float *)b.ptr, (const float *)v.ptr,
-                           (float *)out.ptr, (uint32_t *)workspace, args);
+void launch(void *workspace, const ScanArgs &args, hipStream_t stream) {
+    hipLaunchKernelGGL((scan_mfma_kernel<D, F, 3>), dim3((unsigned)args.total_waves), dim3(kWave),
+                       0, stream, (uint32_t *)workspace, args);
 }
 
 bool aligned16(const void *ptr, int64_t s0, int64_t s1, int64_t s2) {
@@ -622,8 +629,9 @@ bool stride_ok(int64_t stride_l, int width) { return stride_l >= width && stride
 
 }  // namespace
 
-bool mfma_scan_supported(const Operand &a, const Operand &b, const Operand &v,
-                         const OperandOut &out, int64_t L) {
+bool mfma_scan_supported(const ScanDesc &sd, int64_t L) {
+    const Operand &a = sd.a, &b = sd.b, &v = sd.v;
+    const OperandOut &out = sd.out;
     const int D = a.width, F = v.width;
     const bool shape_ok = (D == 64 && F == 64) || (D == 32 && F == 128) || (D == 128 && F == 32);
     if (!shape_ok) return false;
@@ -638,37 +646,48 @@ bool mfma_scan_supported(const Operand &a, const Operand &b, const Operand &v,
            aligned16(out.ptr, out.stride_n, out.stride_h, out.stride_l);
 }
 
-int64_t mfma_scan_workspace_bytes(int64_t N, int64_t H, int64_t L, int64_t D, int64_t F) {
-    return make_plan(N, H, L, D, F).workspace_bytes;
+int64_t mfma_scan_workspace_bytes(int64_t N, int64_t H, int64_t L, int64_t D, int64_t F,
+                                  int nscans) {
+    const MfmaPlan pl = make_plan(N, H, L, D, F, nscans);
+    return pl.workspace_bytes;
 }
 
-int mfma_scan(const Operand &a, const Operand &b, const Operand &v, const OperandOut &out,
-              int64_t N, int64_t H, int64_t L, bool reverse, void *workspace,
-              size_t workspace_bytes, hipStream_t stream) {
-    const int D = a.width, F = v.width;
-    const MfmaPlan pl = make_plan(N, H, L, D, F);
+int mfma_scan(const ScanDesc *scans, int nscans, int64_t N, int64_t H, int64_t L,
+              void *workspace, size_t workspace_bytes, hipStream_t stream) {
+    if (nscans < 1 || nscans > kMaxScans) return fail(FTC_ERR_INVALID, "bad scan count");
+    const int D = scans[0].a.width, F = scans[0].v.width;
+    const MfmaPlan pl = make_plan(N, H, L, D, F, nscans);
     if (pl.workspace_bytes > 0 && (!workspace || workspace_bytes < (size_t)pl.workspace_bytes))
         return fail(FTC_ERR_WORKSPACE, "workspace of %lld bytes needed, %zu given",
                     (long long)pl.workspace_bytes, workspace_bytes);
-    if (pl.waves > 0x3fffffffLL) return fail(FTC_ERR_UNSUPPORTED, "too many wavefronts");
     if (pl.workspace_bytes > 0 && (uintptr_t)workspace % 256 != 0)
         return fail(FTC_ERR_WORKSPACE, "workspace must be 256-byte aligned");
-    // buffer descriptors address a segment with 32-bit byte offsets
-    const int64_t max_stride = std::max(std::max(a.stride_l, b.stride_l),
-                                        std::max(v.stride_l, out.stride_l));
-    if ((int64_t)(pl.seg_len + kChunk) * max_stride * 4 >= 0x7fffffffLL)
-        return fail(FTC_ERR_UNSUPPORTED, "segment too long for 32-bit offsets");
 
     ScanArgs args;
-    args.a_sn = a.stride_n, args.a_sh = a.stride_h, args.a_sl = a.stride_l;
-    args.b_sn = b.stride_n, args.b_sh = b.stride_h, args.b_sl = b.stride_l;
-    args.v_sn = v.stride_n, args.v_sh = v.stride_h, args.v_sl = v.stride_l;
-    args.o_sn = out.stride_n, args.o_sh = out.stride_h, args.o_sl = out.stride_l;
+    int64_t max_stride = 0;
+    for (int i = 0; i < kMaxScans; i++) {
+        const ScanDesc &sd = scans[i < nscans ? i : 0];
+        ScanOperands &o = args.scan[i];
+        o.a = (const float *)sd.a.ptr, o.b = (const float *)sd.b.ptr, o.v = (const float *)sd.v.ptr;
+        o.out = (float *)sd.out.ptr;
+        o.a_sn = sd.a.stride_n, o.a_sh = sd.a.stride_h, o.a_sl = sd.a.stride_l;
+        o.b_sn = sd.b.stride_n, o.b_sh = sd.b.stride_h, o.b_sl = sd.b.stride_l;
+        o.v_sn = sd.v.stride_n, o.v_sh = sd.v.stride_h, o.v_sl = sd.v.stride_l;
+        o.o_sn = sd.out.stride_n, o.o_sh = sd.out.stride_h, o.o_sl = sd.out.stride_l;
+        o.rev = sd.reverse ? 1 : 0;
+        o.pad = 0;
+        max_stride = std::max(max_stride, std::max(std::max(sd.a.stride_l, sd.b.stride_l),
+                                                   std::max(sd.v.stride_l, sd.out.stride_l)));
+    }
+    // buffer descriptors address a segment with 32-bit byte offsets
+    if ((int64_t)(pl.seg_len + 2 * kChunk) * max_stride * 4 >= 0x7fffffffLL)
+        return fail(FTC_ERR_UNSUPPORTED, "segment too long for 32-bit offsets");
     args.L = L;
     args.H = (int32_t)H;
     args.seg_len = pl.seg_len;
     args.nseg = pl.nseg;
-    args.total_waves = (int32_t)pl.waves;
+    args.waves_per_scan = (int32_t)pl.waves;
+    args.total_waves = (int32_t)(pl.waves * nscans);
     // short chains: one level (every step adds the sums of all steps before it); long
     // chains: groups of about sqrt(nseg) steps
     args.group = pl.nseg;
@@ -678,11 +697,11 @@ int mfma_scan(const Operand &a, const Operand &b, const Operand &v, const Operan
     }
 
     if (D == 64 && F == 64)
-        launch<64, 64>(a, b, v, out, workspace, args, reverse, stream);
+        launch<64, 64>(workspace, args, stream);
     else if (D == 32 && F == 128)
-        launch<32, 128>(a, b, v, out, workspace, args, reverse, stream);
+        launch<32, 128>(workspace, args, stream);
     else
-        launch<128, 32>(a, b, v, out, workspace, args, reverse, stream);
+        launch<128, 32>(workspace, args, stream);
     hipError_t err = hipGetLastError();
     if (err != hipSuccess)
         return fail(FTC_ERR_HIP, "MFMA scan launch failed: %s", hipGetErrorString(err));
