@@ -99,10 +99,36 @@ def main():
                 torch.empty(N, H, L, M, device=dev, dtype=tdtype)]
         sets.append((ins, outs))
 
+    # The timed path is the C ABI itself: descriptors, workspace and stream are prepared
+    # once, a step is two library calls (the Python wrapper's per-call cost is reported
+    # separately as wrapper_overhead_us).
+    import ctypes
+    lib = _native.load()
+    code = _native.dtype_code(tdtype)
+    ws_bytes = max(lib.ftc_causal_dot_product_workspace_bytes(N, H, L, E, M, code),
+                   lib.ftc_causal_dot_backward_workspace_bytes(N, H, L, E, M, code))
+    assert ws_bytes >= 0, _native.last_error()
+    ws = torch.zeros(max(ws_bytes, 256), dtype=torch.uint8, device=dev)
+    ws_ptr = ctypes.c_void_p(ws.data_ptr())
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    keep_alive = [[_native.describe(t) for t in ins + outs] for ins, outs in sets]
+    descs = [[ctypes.byref(d) for d in row] for row in keep_alive]
+
+    def fwd(i):
+        q, k, v, g, o, dq, dk, dv = descs[i % nsets]
+        rc = lib.ftc_causal_dot_product(q, k, v, o, ws_ptr, ws_bytes, stream)
+        if rc:
+            raise RuntimeError(_native.last_error())
+
+    def bwd(i):
+        q, k, v, g, o, dq, dk, dv = descs[i % nsets]
+        rc = lib.ftc_causal_dot_backward(q, k, v, g, dq, dk, dv, ws_ptr, ws_bytes, stream)
+        if rc:
+            raise RuntimeError(_native.last_error())
+
     def step(i):
-        (q, k, v, g), (o, dq, dk, dv) = sets[i % nsets]
-        causal_dot_product_hip(q, k, v, o)
-        causal_dot_backward_hip(q, k, v, g, dq, dk, dv)
+        fwd(i)
+        bwd(i)
 
     for i in range(args.warmup):
         step(i)
@@ -117,13 +143,22 @@ def main():
     # per-direction device time with events on the launch stream
     ev = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(args.steps)]
     for i in range(args.steps):
-        (q, k, v, g), (o, dq, dk, dv) = sets[i % nsets]
         ev[i][0].record()
-        causal_dot_product_hip(q, k, v, o)
+        fwd(i)
         ev[i][1].record()
-        causal_dot_backward_hip(q, k, v, g, dq, dk, dv)
+        bwd(i)
         ev[i][2].record()
     torch.cuda.synchronize()
+    assert int(ws[8:12].view(torch.int32).item()) == 0, "a wavefront gave up waiting"
+
+    # cost of going through the Python wrapper instead (same work, wall clock)
+    t2 = time.perf_counter()
+    for i in range(args.steps):
+        (q, k, v, g), (o, dq, dk, dv) = sets[i % nsets]
+        causal_dot_product_hip(q, k, v, o)
+        causal_dot_backward_hip(q, k, v, g, dq, dk, dv)
+    torch.cuda.synchronize()
+    wrapper_ms = (time.perf_counter() - t2) * 1e3 / args.steps
     fwd_ms = sorted(e[0].elapsed_time(e[1]) for e in ev)
     bwd_ms = sorted(e[1].elapsed_time(e[2]) for e in ev)
     fwd_avg, bwd_avg = sum(fwd_ms) / len(fwd_ms), sum(bwd_ms) / len(bwd_ms)
@@ -151,6 +186,7 @@ def main():
                                % (args.workload, N, H, L, E, M, dtype),
                    "input_sets_rotated": nsets,
                    "token_heads_per_s": round(TH / (ms_per_step * 1e-3), 1),
+                   "python_wrapper_ms_per_step": round(wrapper_ms, 5),
                    "fwd_ms_avg": round(fwd_avg, 5), "fwd_ms_min": round(fwd_ms[0], 5),
                    "bwd_ms_avg": round(bwd_avg, 5), "bwd_ms_min": round(bwd_ms[0], 5),
                    "fwd_alg_GBps": round(fwd_gbps, 1),

@@ -43,6 +43,7 @@
 // positions outside the segment read as zero and stores to them are dropped, so tails need
 // no branches.
 #include <algorithm>
+#include <cstdlib>
 
 #include "ftc_common.h"
 
@@ -601,6 +602,14 @@ MfmaPlan make_plan(int64_t N, int64_t H, int64_t L, int64_t D, int64_t F, int ns
         if (cost < best_cost - 1e-9) {
             best_cost = cost;
             best_c = c;
+        }
+    }
+    // tuning aid: FTC_SEG_CHUNKS=<n> forces segments of n chunks
+    if (const char *env = getenv("FTC_SEG_CHUNKS")) {
+        const int64_t forced = atoll(env);
+        if (forced >= 1 && forced <= total_chunks) {
+            const int64_t nseg = (total_chunks + forced - 1) / forced;
+            if (chains * nseg * nscans <= kMaxWaves && nseg <= 4096) best_c = forced;
         }
     }
     pl.seg_len = (int)(best_c * kChunk);
