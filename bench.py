@@ -30,6 +30,12 @@ for p in (ROOT, os.path.join(ROOT, "fast-transformers_amd")):
 HBM_PEAK_GBPS = 8000.0          # MI355X HBM3E, published
 MFMA_FP32_PEAK_TFLOPS = 157.3   # MI355X dense fp32 matrix, published
 
+# HBM bytes per scan-kernel launch (mean of the forward and the backward launch) from
+# rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script, scaled by what the same
+# counters read for the 256 MiB copy of --calibrate-copy; the runs are summarised in
+# profiles/scan_mfma_kernel_cfg2_traffic.md.  None = not measured for that workload.
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {"cfg2": 245216602}
+
 WORKLOADS = {
     # name: (N, H, L, E, M, dtype, seed)
     "cfg2": (10, 8, 1000, 64, 64, "f32", 2),
@@ -55,6 +61,9 @@ def main():
     ap.add_argument("--workload", default="cfg2", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--sets", type=int, default=0, help="input sets to rotate over (0 = auto)")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run one 256 MiB device copy (a known-size kernel for scaling "
+                         "the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU (the path shards over N*H with no "
@@ -130,6 +139,13 @@ def main():
         fwd(i)
         bwd(i)
 
+    if args.calibrate_copy:
+        src = torch.empty(64 << 20, dtype=torch.float32, device=dev).normal_()
+        dst = torch.empty_like(src)
+        dst.copy_(src)          # reads 256 MiB, writes 256 MiB
+        torch.cuda.synchronize()
+        del src, dst
+
     for i in range(args.warmup):
         step(i)
     torch.cuda.synchronize()
@@ -168,6 +184,13 @@ def main():
     bwd_gbps = bb * TH / (bwd_avg * 1e-3) / 1e9
     fwd_gbps = fb * TH / (fwd_avg * 1e-3) / 1e9
     value = N * L / (ms_per_step * 1e-3) / 1e6
+    # The dominant kernel is the scan kernel: with E = M one step launches it twice (forward:
+    # one scan; backward: three scans side by side).  Its roofline entry averages over those
+    # two launches: algorithmic bytes per launch = (fwd + bwd bytes) / 2, duration = mean of
+    # the two event-timed launches.
+    launch_ms = (fwd_avg + bwd_avg) / 2
+    launch_bytes = (fb + bb) * TH / 2
+    launch_gbps = launch_bytes / (launch_ms * 1e-3) / 1e9
 
     result = {
         "metric": "causal_dot_product fwd+bwd Mtokens/s (H=8,E=M=64); % of HBM/MFMA roofline",
@@ -194,9 +217,14 @@ def main():
                    "fwdbwd_alg_TFLOPs": round(14 * E * M * TH / (ms_per_step * 1e-3) / 1e12, 2),
                    "fwdbwd_frac_of_hbm_roofline":
                        round((fb + bb) * TH / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)},
-        "roofline": {"bound": "hbm", "kernel": "backward launch sequence",
-                     "achieved": round(bwd_gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": round(bwd_gbps / HBM_PEAK_GBPS, 4), "traffic": None},
+        "roofline": {"bound": "hbm",
+                     "kernel": "scan_mfma_kernel (mean of its forward and backward launch)"
+                               if dtype == "f32" else "generic_scan_kernel launches",
+                     "achieved": round(launch_gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": round(launch_gbps / HBM_PEAK_GBPS, 4),
+                     "launch_ms_avg": round(launch_ms, 5),
+                     "alg_bytes_per_launch": int(launch_bytes),
+                     "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH.get(args.workload)},
     }
 
     if not args.no_cpu:
