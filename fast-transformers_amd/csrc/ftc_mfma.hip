@@ -244,8 +244,12 @@ __global__ __launch_bounds__(kWave) void scan_mfma_kernel(uint32_t *__restrict__
     //  16*hh + 8*(t/4) + 4*g + (t%4)
     const uint32_t a_lane = ln * a_sl4 + 16u * g;
     const uint32_t b_lane = ln * b_sl4 + 16u * g;
-    const uint32_t bt_lane = 4u * g * b_sl4 + 4u * ln;
-    const uint32_t vt_lane = 4u * g * v_sl4 + 4u * ln;
+    // position-major operands pass through LDS as fp32 rows: 16-byte global loads (lane =
+    // (row within the load, 4 columns)), 16-byte LDS writes, 4-byte LDS reads by column
+    constexpr int kBtLoads = D / 8, kVtLoads = F / 8;            // loads per 32-row tile
+    constexpr int kBtRows = 64 / (D / 4), kVtRows = 64 / (F / 4);  // rows per load
+    const uint32_t bt_lane = (uint32_t)(lane / (D / 4)) * b_sl4 + 16u * (lane % (D / 4));
+    const uint32_t vt_lane = (uint32_t)(lane / (F / 4)) * v_sl4 + 16u * (lane % (F / 4));
     const uint32_t o_lane = ln * o_sl4 + 16u * g;
 
     // first row of chunk c relative to the segment (REV walks down from the end and its
@@ -257,8 +261,10 @@ __global__ __launch_bounds__(kWave) void scan_mfma_kernel(uint32_t *__restrict__
     // raw fp32 of the chunk being fetched
     float4 a_raw[KD][2];   // a rows, B operand of (1) and (2b)
     float4 b_raw[KD][2];   // b rows, A operand of (1)
-    float bt_raw[DT][2][8];  // b by position, A operand of (3)
-    float vt_raw[FT][2][8];  // v by position, A operand of (2a), B operand of (3)
+    float4 bt_raw[kBtLoads];  // b rows on their way to LDS (A operand of (3))
+    float4 vt_raw[kVtLoads];  // v rows on their way to LDS (A operand of (2a), B of (3))
+    __shared__ __align__(16) float bt_lds[2][kChunk * D];
+    __shared__ __align__(16) float vt_lds[2][kChunk * F];
 
     auto fetch_rows = [&](__amdgpu_buffer_rsrc_t rs, uint32_t lane_off, uint32_t sl4, int row0,
                           float4 (&raw)[KD][2]) {
@@ -272,24 +278,37 @@ __global__ __launch_bounds__(kWave) void scan_mfma_kernel(uint32_t *__restrict__
     auto fetch_bt = [&](int row0) {
         const uint32_t off = bt_lane + (uint32_t)row0 * b_sl4;
 #pragma unroll
-        for (int dt = 0; dt < DT; dt++)
-#pragma unroll
-            for (int hh = 0; hh < 2; hh++)
-#pragma unroll
-                for (int t = 0; t < 8; t++)
-                    bt_raw[dt][hh][t] = buffer_load1(
-                        b_rs, off + (uint32_t)(16 * hh + 8 * (t / 4) + (t % 4)) * b_sl4 + 128u * dt);
+        for (int i = 0; i < kBtLoads; i++)
+            bt_raw[i] = buffer_load4(b_rs, off + (uint32_t)(i * kBtRows) * b_sl4);
     };
     auto fetch_vt = [&](int row0) {
         const uint32_t off = vt_lane + (uint32_t)row0 * v_sl4;
 #pragma unroll
-        for (int ft = 0; ft < FT; ft++)
+        for (int i = 0; i < kVtLoads; i++)
+            vt_raw[i] = buffer_load4(v_rs, off + (uint32_t)(i * kVtRows) * v_sl4);
+    };
+    // fetched rows -> LDS tile `buf` (row-major, 32 x width floats)
+    auto stash_bt = [&](int buf) {
 #pragma unroll
-            for (int hh = 0; hh < 2; hh++)
+        for (int i = 0; i < kBtLoads; i++)
+            *(float4 *)&bt_lds[buf][(i * kBtRows + lane / (D / 4)) * D + 4 * (lane % (D / 4))] =
+                bt_raw[i];
+    };
+    auto stash_vt = [&](int buf) {
 #pragma unroll
-                for (int t = 0; t < 8; t++)
-                    vt_raw[ft][hh][t] = buffer_load1(
-                        v_rs, off + (uint32_t)(16 * hh + 8 * (t / 4) + (t % 4)) * v_sl4 + 128u * ft);
+        for (int i = 0; i < kVtLoads; i++)
+            *(float4 *)&vt_lds[buf][(i * kVtRows + lane / (F / 4)) * F + 4 * (lane % (F / 4))] =
+                vt_raw[i];
+    };
+    // LDS tile -> the NS fragments of k-step hh for the 32 columns of tile `tile`:
+    // lane (col = ln, g), k-slot t is row 16*hh + 8*(t/4) + 4*g + (t%4)
+    auto frag_from_lds = [&](const float *tile_base, int width, int tile, int hh,
+                             Frag (&frag)[NS]) {
+        float x[8];
+#pragma unroll
+        for (int t = 0; t < 8; t++)
+            x[t] = tile_base[(16 * hh + 8 * (t / 4) + 4 * g + (t % 4)) * width + 32 * tile + ln];
+        split8<NS>(x, frag);
     };
     auto split_rows = [&](const float4 (&raw)[KD][2], Frag (&frag)[KD][NS]) {
 #pragma unroll
@@ -400,17 +419,22 @@ __global__ __launch_bounds__(kWave) void scan_mfma_kernel(uint32_t *__restrict__
             fetch_bt(chunk_row0(nchunks - 1));
             fetch_vt(chunk_row0(nchunks - 1));
             for (int c = nchunks - 1; c >= 0; c--) {
+                const int buf = c & 1;
+                stash_bt(buf);
+                stash_vt(buf);
+                fetch_bt(pass1_row0(c - 1));
+                fetch_vt(pass1_row0(c - 1));
                 Frag bt_frag[DT][2][NS], v_frag[FT][2][NS];
 #pragma unroll
                 for (int dt = 0; dt < DT; dt++)
 #pragma unroll
-                    for (int hh = 0; hh < 2; hh++) split8<NS>(bt_raw[dt][hh], bt_frag[dt][hh]);
+                    for (int hh = 0; hh < 2; hh++)
+                        frag_from_lds(bt_lds[buf], D, dt, hh, bt_frag[dt][hh]);
 #pragma unroll
                 for (int ft = 0; ft < FT; ft++)
 #pragma unroll
-                    for (int hh = 0; hh < 2; hh++) split8<NS>(vt_raw[ft][hh], v_frag[ft][hh]);
-                fetch_bt(pass1_row0(c - 1));
-                fetch_vt(pass1_row0(c - 1));
+                    for (int hh = 0; hh < 2; hh++)
+                        frag_from_lds(vt_lds[buf], F, ft, hh, v_frag[ft][hh]);
                 update_state(bt_frag, v_frag);
             }
             if (!is_last_of_group) publish_state(ticket, S, kFlagSum);
@@ -514,12 +538,17 @@ __global__ __launch_bounds__(kWave) void scan_mfma_kernel(uint32_t *__restrict__
             split8<NS>(x, p_frag[hh]);
         }
 
+        // this chunk's position-major rows go to LDS, the next chunk's are requested
+        const int buf = c & 1;
+        stash_vt(buf);
+        stash_bt(buf);
+        fetch_vt(next0);
+        fetch_bt(next0);
         Frag v_frag[FT][2][NS];  // A operand of (2a), B operand of (3)
 #pragma unroll
         for (int ft = 0; ft < FT; ft++)
 #pragma unroll
-            for (int hh = 0; hh < 2; hh++) split8<NS>(vt_raw[ft][hh], v_frag[ft][hh]);
-        fetch_vt(next0);
+            for (int hh = 0; hh < 2; hh++) frag_from_lds(vt_lds[buf], F, ft, hh, v_frag[ft][hh]);
 
         // (2b) + (2a) per output tile, then store
         const uint32_t o_off = o_lane + (uint32_t)row0 * o_sl4;
@@ -552,8 +581,7 @@ __global__ __launch_bounds__(kWave) void scan_mfma_kernel(uint32_t *__restrict__
 #pragma unroll
         for (int dt = 0; dt < DT; dt++)
 #pragma unroll
-            for (int hh = 0; hh < 2; hh++) split8<NS>(bt_raw[dt][hh], bt_frag[dt][hh]);
-        fetch_bt(next0);
+            for (int hh = 0; hh < 2; hh++) frag_from_lds(bt_lds[buf], D, dt, hh, bt_frag[dt][hh]);
         update_state(bt_frag, v_frag);
     }
 
