@@ -275,31 +275,35 @@ __global__ __launch_bounds__(kWave) void scan_mfma_kernel(uint32_t *__restrict__
             raw[ks][1] = buffer_load4(rs, off + 64u * ks + 32u);
         }
     };
-    auto fetch_bt = [&](int row0) {
+    auto fetch_bt_into = [&](int row0, float4 (&raw)[kBtLoads]) {
         const uint32_t off = bt_lane + (uint32_t)row0 * b_sl4;
 #pragma unroll
         for (int i = 0; i < kBtLoads; i++)
-            bt_raw[i] = buffer_load4(b_rs, off + (uint32_t)(i * kBtRows) * b_sl4);
+            raw[i] = buffer_load4(b_rs, off + (uint32_t)(i * kBtRows) * b_sl4);
     };
-    auto fetch_vt = [&](int row0) {
+    auto fetch_vt_into = [&](int row0, float4 (&raw)[kVtLoads]) {
         const uint32_t off = vt_lane + (uint32_t)row0 * v_sl4;
 #pragma unroll
         for (int i = 0; i < kVtLoads; i++)
-            vt_raw[i] = buffer_load4(v_rs, off + (uint32_t)(i * kVtRows) * v_sl4);
+            raw[i] = buffer_load4(v_rs, off + (uint32_t)(i * kVtRows) * v_sl4);
     };
     // fetched rows -> LDS tile `buf` (row-major, 32 x width floats)
-    auto stash_bt = [&](int buf) {
+    auto stash_bt_from = [&](int buf, const float4 (&raw)[kBtLoads]) {
 #pragma unroll
         for (int i = 0; i < kBtLoads; i++)
             *(float4 *)&bt_lds[buf][(i * kBtRows + lane / (D / 4)) * D + 4 * (lane % (D / 4))] =
-                bt_raw[i];
+                raw[i];
     };
-    auto stash_vt = [&](int buf) {
+    auto stash_vt_from = [&](int buf, const float4 (&raw)[kVtLoads]) {
 #pragma unroll
         for (int i = 0; i < kVtLoads; i++)
             *(float4 *)&vt_lds[buf][(i * kVtRows + lane / (F / 4)) * F + 4 * (lane % (F / 4))] =
-                vt_raw[i];
+                raw[i];
     };
+    auto fetch_bt = [&](int row0) { fetch_bt_into(row0, bt_raw); };
+    auto fetch_vt = [&](int row0) { fetch_vt_into(row0, vt_raw); };
+    auto stash_bt = [&](int buf) { stash_bt_from(buf, bt_raw); };
+    auto stash_vt = [&](int buf) { stash_vt_from(buf, vt_raw); };
     // LDS tile -> the NS fragments of k-step hh for the 32 columns of tile `tile`:
     // lane (col = ln, g), k-slot t is row 16*hh + 8*(t/4) + 4*g + (t%4)
     auto frag_from_lds = [&](const float *tile_base, int width, int tile, int hh,
@@ -416,14 +420,10 @@ __global__ __launch_bounds__(kWave) void scan_mfma_kernel(uint32_t *__restrict__
         // ---- pass 1: the segment's own state sum, walked against the direction of pass 2
         // so that pass 2 starts on the rows read last ----
         if (need_own_sum) {
-            fetch_bt(chunk_row0(nchunks - 1));
-            fetch_vt(chunk_row0(nchunks - 1));
-            for (int c = nchunks - 1; c >= 0; c--) {
-                const int buf = c & 1;
-                stash_bt(buf);
-                stash_vt(buf);
-                fetch_bt(pass1_row0(c - 1));
-                fetch_vt(pass1_row0(c - 1));
+            // rows are requested two chunks ahead (pass 1 has registers to spare and its
+            // chunks are short compared with the memory latency)
+            float4 bt_raw2[kBtLoads], vt_raw2[kVtLoads];
+            auto sum_chunk = [&](int buf) {
                 Frag bt_frag[DT][2][NS], v_frag[FT][2][NS];
 #pragma unroll
                 for (int dt = 0; dt < DT; dt++)
@@ -436,6 +436,23 @@ __global__ __launch_bounds__(kWave) void scan_mfma_kernel(uint32_t *__restrict__
                     for (int hh = 0; hh < 2; hh++)
                         frag_from_lds(vt_lds[buf], F, ft, hh, v_frag[ft][hh]);
                 update_state(bt_frag, v_frag);
+            };
+            fetch_bt_into(pass1_row0(nchunks - 1), bt_raw);
+            fetch_vt_into(pass1_row0(nchunks - 1), vt_raw);
+            fetch_bt_into(pass1_row0(nchunks - 2), bt_raw2);
+            fetch_vt_into(pass1_row0(nchunks - 2), vt_raw2);
+            for (int c = nchunks - 1; c >= 0; c -= 2) {
+                stash_bt_from(0, bt_raw);
+                stash_vt_from(0, vt_raw);
+                fetch_bt_into(pass1_row0(c - 2), bt_raw);
+                fetch_vt_into(pass1_row0(c - 2), vt_raw);
+                sum_chunk(0);
+                if (c == 0) break;
+                stash_bt_from(1, bt_raw2);
+                stash_vt_from(1, vt_raw2);
+                fetch_bt_into(pass1_row0(c - 3), bt_raw2);
+                fetch_vt_into(pass1_row0(c - 3), vt_raw2);
+                sum_chunk(1);
             }
             if (!is_last_of_group) publish_state(ticket, S, kFlagSum);
         }
