@@ -78,8 +78,7 @@ int run_scans(const ScanDesc *scans, int n, int64_t N, int64_t H, int64_t L, voi
         if (mfma_scan_supported(scans[i], L)) {
             int k = 1;
             while (i + k < n && k < kMfmaMaxScans && mfma_scan_supported(scans[i + k], L) &&
-                   scans[i + k].a.width == scans[i].a.width &&
-                   scans[i + k].v.width == scans[i].v.width)
+                   mfma_scan_same_launch(scans[i], scans[i + k]))
                 k++;
             int rc = mfma_scan(scans + i, k, N, H, L, workspace, workspace_bytes, stream);
             if (rc) return rc;

@@ -74,8 +74,8 @@ int generic_scan(const Operand &a, const Operand &b, const Operand &v, const Ope
                  size_t workspace_bytes, hipStream_t stream);
 
 // ---------------------------------------------------------------------------
-// MFMA scan (fp32 rows, (D, F) in {(64,64), (32,128), (128,32)}, 16-byte aligned rows):
-// ftc_mfma.hip.  Same contract as generic_scan.
+// MFMA scan ((D, F) in {(64,64), (32,128), (128,32)}, 16-byte aligned rows; all-fp32 operands
+// or the bf16 combinations of a forward / backward call): ftc_mfma.hip + ftc_mfma_kernel.h.
 // ---------------------------------------------------------------------------
 struct ScanDesc {
     Operand a, b, v;
@@ -85,6 +85,8 @@ struct ScanDesc {
 constexpr int kMfmaMaxScans = 3;
 
 bool mfma_scan_supported(const ScanDesc &scan, int64_t L);
+// true when two supported scans can share a launch (same widths, same element types)
+bool mfma_scan_same_launch(const ScanDesc &x, const ScanDesc &y);
 // Workspace for `nscans` scans of one (D, F) run side by side in one launch.
 int64_t mfma_scan_workspace_bytes(int64_t N, int64_t H, int64_t L, int64_t D, int64_t F,
                                   int nscans);

@@ -1,0 +1,11 @@
+// MFMA scan kernels for one combination of element types (a, b, v, out) =
+// (fp32, fp32, fp32, fp32); see ftc_mfma_kernel.h.
+#include "ftc_mfma_kernel.h"
+
+namespace ftc {
+namespace mfma {
+void launch_scan_ffff(int D, int F, void *ws, const ScanArgs &args, hipStream_t stream) {
+    launch_scan<float, float, float, float>(D, F, ws, args, stream);
+}
+}  // namespace mfma
+}  // namespace ftc
