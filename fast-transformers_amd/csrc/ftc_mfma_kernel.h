@@ -275,7 +275,24 @@ __global__ __launch_bounds__(kWave) void scan_mfma_kernel(uint32_t *__restrict__
     // the order in which they start running, so a step only ever waits for steps that are
     // already running ----
     // chains of all scans are numbered consecutively: global chain = scan * chains + chain
-    const uint32_t scan_id = blockIdx.x / (uint32_t)p.waves_per_scan;
+    // Workgroups are dispatched round-robin over the 8 XCDs.  Blocks are numbered so that
+    // wavefront w of every scan of the launch lands on the same XCD at about the same time
+    // (groups of 8 consecutive blocks per scan): scans that read the same rows in the same
+    // direction (dK and dV) then find each other's lines in that XCD's L2.
+    const uint32_t wps = (uint32_t)p.waves_per_scan;
+    const uint32_t nscans = (uint32_t)p.total_waves / wps;
+    const uint32_t full = (wps / 8u) * 8u;
+    uint32_t scan_id, wave_in_scan;
+    if (blockIdx.x < full * nscans) {
+        const uint32_t grp = blockIdx.x / (8u * nscans), r = blockIdx.x % (8u * nscans);
+        scan_id = r / 8u;
+        wave_in_scan = grp * 8u + r % 8u;
+    } else {
+        const uint32_t t = blockIdx.x - full * nscans;
+        scan_id = t / (wps - full);
+        wave_in_scan = full + t % (wps - full);
+    }
+    const uint32_t vblock = scan_id * wps + wave_in_scan;  // block id in scan-major order
     const ScanOperands &op = p.scan[scan_id];
     const bool REV = op.rev != 0;
     const char *a_ptr = (const char *)op.a, *b_ptr = (const char *)op.b,
@@ -283,7 +300,7 @@ __global__ __launch_bounds__(kWave) void scan_mfma_kernel(uint32_t *__restrict__
     char *out_ptr = (char *)op.out;
     uint32_t ticket = 0;
     if (p.nseg > 1) {
-        const uint32_t my_chain = blockIdx.x / (uint32_t)p.nseg;
+        const uint32_t my_chain = vblock / (uint32_t)p.nseg;
         uint32_t order = 0;
         if (lane == 0)
             order = __hip_atomic_fetch_add(flags + kMaxWaves + my_chain, 1u, __ATOMIC_RELAXED,
@@ -298,7 +315,7 @@ __global__ __launch_bounds__(kWave) void scan_mfma_kernel(uint32_t *__restrict__
             return;
         }
     } else {
-        ticket = blockIdx.x;
+        ticket = vblock;
     }
     const int64_t chain = (ticket - scan_id * (uint32_t)p.waves_per_scan) / (uint32_t)p.nseg;
     const int step = (int)(ticket % (uint32_t)p.nseg);      // position in dependency order
