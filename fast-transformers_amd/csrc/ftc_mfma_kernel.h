@@ -228,6 +228,155 @@ __device__ __forceinline__ void wait_for_stores() {
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 }
 
+// Exchange of segment states between the wavefronts of a chain.
+//
+// Segments of a chain form groups of `group` consecutive steps (steps are numbered in
+// dependency order).  The state before step s is (sum of the totals of the groups before
+// its group) + (sum of the sums of the steps before it in its group), always added in
+// ascending order, so the result does not depend on timing.  Every step but the last of its
+// group publishes its own sum; the last step of every group but the last publishes the
+// group total.  States travel as sc1 buffer accesses; flags as agent-scope atomics; every
+// wait is bounded.
+template <int DT, int FT>
+struct StateExchange {
+    static constexpr int kStateBytes = DT * FT * 16 * kWave * 4;
+    gu32 *flags;
+    __amdgpu_buffer_rsrc_t st_rs;
+    uint32_t total_slots, ticket, chain_ticket0;
+    int step, nseg, G, grp, grp_first, lane;
+    bool is_last_of_group, need_own_sum, failed;
+    int spins;
+
+    // `slots`: 2 * total_slots states; `ticket`: this wavefront's slot, its chain's step-0
+    // slot being ticket - step
+    __device__ __forceinline__ StateExchange(gu32 *flags_, gfloat *slots, uint32_t total_slots_,
+                                             uint32_t ticket_, int step_, int nseg_, int group,
+                                             int lane_)
+        : flags(flags_), total_slots(total_slots_), ticket(ticket_),
+          chain_ticket0(ticket_ - (uint32_t)step_), step(step_), nseg(nseg_), G(group),
+          lane(lane_), failed(false), spins(0) {
+        st_rs = __builtin_amdgcn_make_buffer_rsrc(
+            (void *)slots, 0, (2u * total_slots) * (uint32_t)kStateBytes, kRsrcFlags);
+        grp = step / G;
+        grp_first = grp * G;
+        const int grp_last = min(grp_first + G, nseg) - 1;
+        is_last_of_group = step == grp_last;
+        need_own_sum = step + 1 < nseg;  // the very last step has no reader
+    }
+
+    __device__ __forceinline__ void publish_state(uint32_t slot, const f32x16 (&T)[DT][FT],
+                                                  uint32_t flag_value) {
+        const uint32_t base = slot * (uint32_t)kStateBytes + 16u * lane;
+#pragma unroll
+        for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+            for (int ft = 0; ft < FT; ft++)
+#pragma unroll
+                for (int q4 = 0; q4 < 4; q4++) {
+                    const u32x4 w = {__float_as_uint(T[dt][ft][4 * q4 + 0]),
+                                     __float_as_uint(T[dt][ft][4 * q4 + 1]),
+                                     __float_as_uint(T[dt][ft][4 * q4 + 2]),
+                                     __float_as_uint(T[dt][ft][4 * q4 + 3])};
+                    __builtin_amdgcn_raw_buffer_store_b128(
+                        w, st_rs, base + (uint32_t)(((dt * FT + ft) * 4 + q4) * kWave * 16), 0,
+                        kCoherentAux);
+                }
+        wait_for_stores();
+        if (lane == 0)
+            __hip_atomic_store(flags + ticket, flag_value, __ATOMIC_RELAXED,
+                               __HIP_MEMORY_SCOPE_AGENT);
+    }
+
+    __device__ __forceinline__ void add_state(uint32_t slot, f32x16 (&T)[DT][FT]) {
+        const uint32_t base = slot * (uint32_t)kStateBytes + 16u * lane;
+        // all loads of a state are in flight together, then added in a fixed order
+        u32x4 w[DT * FT * 4];
+#pragma unroll
+        for (int i = 0; i < DT * FT * 4; i++)
+            w[i] = __builtin_amdgcn_raw_buffer_load_b128(st_rs, base + (uint32_t)(i * kWave * 16),
+                                                         0, kCoherentAux);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+            for (int ft = 0; ft < FT; ft++)
+#pragma unroll
+                for (int q4 = 0; q4 < 4; q4++) {
+                    const u32x4 x = w[(dt * FT + ft) * 4 + q4];
+                    T[dt][ft][4 * q4 + 0] += __uint_as_float(x.x);
+                    T[dt][ft][4 * q4 + 1] += __uint_as_float(x.y);
+                    T[dt][ft][4 * q4 + 2] += __uint_as_float(x.z);
+                    T[dt][ft][4 * q4 + 3] += __uint_as_float(x.w);
+                }
+    }
+
+    // wait until `count` wavefronts, slots first, first + stride, ..., show `bit`
+    __device__ __forceinline__ void wait_flags(uint32_t first, uint32_t stride, int count,
+                                               uint32_t bit) {
+        const bool mine = lane < count;
+        const gu32 *f = flags + first + stride * (uint32_t)lane;
+        while (!failed) {
+            const uint32_t x =
+                mine ? __hip_atomic_load(f, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : bit;
+            if (__builtin_amdgcn_ballot_w64((x & bit) == 0) == 0) break;
+            if (++spins > kSpinLimit) failed = true;
+            __builtin_amdgcn_s_sleep(4);
+        }
+    }
+
+    // after pass 1: make this step's own sum visible to the later steps of its group
+    __device__ __forceinline__ void publish_sum(const f32x16 (&S)[DT][FT]) {
+        if (need_own_sum && !is_last_of_group) publish_state(ticket, S, kFlagSum);
+    }
+
+    // X <- state before this step (S = this step's own sum, left untouched)
+    __device__ __forceinline__ void gather(const f32x16 (&S)[DT][FT], f32x16 (&X)[DT][FT]) {
+#pragma unroll
+        for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+            for (int ft = 0; ft < FT; ft++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) X[dt][ft][r] = 0.f;
+        // ---- sums of the earlier steps of this group ----
+        const int in_group = step - grp_first;
+        if (in_group > 0) {
+            wait_flags(chain_ticket0 + grp_first, 1, in_group, kFlagSum);
+            if (!failed)
+                for (int i = 0; i < in_group; i++) add_state(chain_ticket0 + grp_first + i, X);
+        }
+        if (is_last_of_group && need_own_sum && !failed) {
+            // group total = sums of the group in ascending order (own sum last)
+            f32x16 T[DT][FT];
+#pragma unroll
+            for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+                for (int ft = 0; ft < FT; ft++) T[dt][ft] = X[dt][ft] + S[dt][ft];
+            publish_state(total_slots + ticket, T, kFlagTotal);
+        }
+        // ---- totals of the earlier groups, then the in-group part on top ----
+        if (grp > 0 && !failed) {
+            wait_flags(chain_ticket0 + (uint32_t)(G - 1), (uint32_t)G, grp, kFlagTotal);
+            if (!failed) {
+                f32x16 T[DT][FT];
+#pragma unroll
+                for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+                    for (int ft = 0; ft < FT; ft++) {
+                        T[dt][ft] = X[dt][ft];
+#pragma unroll
+                        for (int r = 0; r < 16; r++) X[dt][ft][r] = 0.f;
+                    }
+                for (int gq = 0; gq < grp; gq++)
+                    add_state(total_slots + chain_ticket0 + (uint32_t)(gq * G + G - 1), X);
+#pragma unroll
+                for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+                    for (int ft = 0; ft < FT; ft++) X[dt][ft] = X[dt][ft] + T[dt][ft];
+            }
+        }
+    }
+};
+
 // One scan of a launch.  A launch runs up to kMaxScans independent scans of the same
 // (D, F, N, H, L) side by side (the three gradients of a backward call), so that their
 // launch gaps and wait times overlap.
@@ -458,83 +607,12 @@ __global__ __launch_bounds__(kWave) void scan_mfma_kernel(uint32_t *__restrict__
             for (int r = 0; r < 16; r++) S[dt][ft][r] = 0.f;
 
     if (p.nseg > 1) {
-        // Segments of a chain form groups of p.group consecutive steps.  The state before
-        // step s is (sum of the totals of the groups before its group) + (sum of the sums
-        // of the steps before it in its group), always added in ascending order, so the
-        // result does not depend on timing.  Every step but the last of its group publishes
-        // its own sum; the last step of every group but the last publishes the group total.
-        const int G = p.group;
-        const int grp = step / G;
-        const int grp_first = grp * G;
-        const int grp_last = min(grp_first + G, p.nseg) - 1;
-        const bool is_last_of_group = step == grp_last;
-        const bool need_own_sum = step + 1 < p.nseg;  // the very last step has no reader
-        const __amdgpu_buffer_rsrc_t st_rs = __builtin_amdgcn_make_buffer_rsrc(
-            (void *)sums, 0, (uint32_t)(2 * p.total_waves) * (uint32_t)(kStateElems * 4),
-            kRsrcFlags);
-        const uint32_t lane16 = 16u * lane;
-        auto slot_offset = [&](uint32_t slot) -> uint32_t { return slot * (kStateElems * 4); };
-        auto publish_state = [&](uint32_t slot, const f32x16 (&T)[DT][FT], uint32_t flag_value) {
-            const uint32_t base = slot_offset(slot) + lane16;
-#pragma unroll
-            for (int dt = 0; dt < DT; dt++)
-#pragma unroll
-                for (int ft = 0; ft < FT; ft++)
-#pragma unroll
-                    for (int q4 = 0; q4 < 4; q4++) {
-                        const u32x4 w = {__float_as_uint(T[dt][ft][4 * q4 + 0]),
-                                         __float_as_uint(T[dt][ft][4 * q4 + 1]),
-                                         __float_as_uint(T[dt][ft][4 * q4 + 2]),
-                                         __float_as_uint(T[dt][ft][4 * q4 + 3])};
-                        __builtin_amdgcn_raw_buffer_store_b128(
-                            w, st_rs, base + (uint32_t)(((dt * FT + ft) * 4 + q4) * kWave * 16), 0,
-                            kCoherentAux);
-                    }
-            wait_for_stores();
-            if (lane == 0)
-                __hip_atomic_store(flags + ticket, flag_value, __ATOMIC_RELAXED,
-                                   __HIP_MEMORY_SCOPE_AGENT);
-        };
-        auto add_state = [&](uint32_t slot, f32x16 (&T)[DT][FT]) {
-            const uint32_t base = slot_offset(slot) + lane16;
-            // all loads of a state are in flight together, then added in a fixed order
-            u32x4 w[DT * FT * 4];
-#pragma unroll
-            for (int i = 0; i < DT * FT * 4; i++)
-                w[i] = __builtin_amdgcn_raw_buffer_load_b128(
-                    st_rs, base + (uint32_t)(i * kWave * 16), 0, kCoherentAux);
-            __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-            for (int dt = 0; dt < DT; dt++)
-#pragma unroll
-                for (int ft = 0; ft < FT; ft++)
-#pragma unroll
-                    for (int q4 = 0; q4 < 4; q4++) {
-                        const u32x4 x = w[(dt * FT + ft) * 4 + q4];
-                        T[dt][ft][4 * q4 + 0] += __uint_as_float(x.x);
-                        T[dt][ft][4 * q4 + 1] += __uint_as_float(x.y);
-                        T[dt][ft][4 * q4 + 2] += __uint_as_float(x.z);
-                        T[dt][ft][4 * q4 + 3] += __uint_as_float(x.w);
-                    }
-        };
-        int spins = 0;
-        bool failed = false;
-        // wait until `count` wavefronts, tickets first, first + stride, ..., show `bit`
-        auto wait_flags = [&](uint32_t first, uint32_t stride, int count, uint32_t bit) {
-            const bool mine = lane < count;
-            const gu32 *f = flags + first + stride * (uint32_t)lane;
-            while (!failed) {
-                const uint32_t x =
-                    mine ? __hip_atomic_load(f, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : bit;
-                if (__builtin_amdgcn_ballot_w64((x & bit) == 0) == 0) break;
-                if (++spins > kSpinLimit) failed = true;
-                __builtin_amdgcn_s_sleep(4);
-            }
-        };
+        StateExchange<DT, FT> xch(flags, sums, (uint32_t)p.total_waves, ticket, step, p.nseg,
+                                  p.group, lane);
 
         // ---- pass 1: the segment's own state sum, walked against the direction of pass 2
         // so that pass 2 starts on the rows read last ----
-        if (need_own_sum) {
+        if (xch.need_own_sum) {
             // rows are requested two chunks ahead (pass 1 has registers to spare and its
             // chunks are short compared with the memory latency)
             u32x4 bt_raw2[kBtLoads], vt_raw2[kVtLoads];
@@ -567,7 +645,7 @@ __global__ __launch_bounds__(kWave) void scan_mfma_kernel(uint32_t *__restrict__
                 fetch_vt_into(pass1_row0(c - 3), vt_raw2);
                 sum_chunk(1);
             }
-            if (!is_last_of_group) publish_state(ticket, S, kFlagSum);
+            xch.publish_sum(S);
         }
         // start fetching the first chunk of pass 2 before waiting
         fetch_a(chunk_row0(0));
@@ -575,51 +653,9 @@ __global__ __launch_bounds__(kWave) void scan_mfma_kernel(uint32_t *__restrict__
         fetch_vt(chunk_row0(0));
         fetch_bt(chunk_row0(0));
 
-        // ---- sums of the earlier steps of this group ----
         f32x16 X[DT][FT];
-#pragma unroll
-        for (int dt = 0; dt < DT; dt++)
-#pragma unroll
-            for (int ft = 0; ft < FT; ft++)
-#pragma unroll
-                for (int r = 0; r < 16; r++) X[dt][ft][r] = 0.f;
-        const int in_group = step - grp_first;
-        const uint32_t chain_ticket0 = ticket - (uint32_t)step;
-        if (in_group > 0) {
-            wait_flags(chain_ticket0 + grp_first, 1, in_group, kFlagSum);
-            if (!failed)
-                for (int i = 0; i < in_group; i++) add_state(chain_ticket0 + grp_first + i, X);
-        }
-        if (is_last_of_group && need_own_sum && !failed) {
-            // group total = sums of the group in ascending order (own sum last)
-#pragma unroll
-            for (int dt = 0; dt < DT; dt++)
-#pragma unroll
-                for (int ft = 0; ft < FT; ft++) S[dt][ft] = X[dt][ft] + S[dt][ft];
-            publish_state((uint32_t)p.total_waves + ticket, S, kFlagTotal);
-        }
-        // ---- totals of the earlier groups, then the in-group part on top ----
-        if (grp > 0 && !failed) {
-            wait_flags(chain_ticket0 + (uint32_t)(G - 1), (uint32_t)G, grp, kFlagTotal);
-            if (!failed) {
-#pragma unroll
-                for (int dt = 0; dt < DT; dt++)
-#pragma unroll
-                    for (int ft = 0; ft < FT; ft++) {
-                        S[dt][ft] = X[dt][ft];
-#pragma unroll
-                        for (int r = 0; r < 16; r++) X[dt][ft][r] = 0.f;
-                    }
-                for (int gq = 0; gq < grp; gq++)
-                    add_state((uint32_t)p.total_waves + chain_ticket0 + (uint32_t)(gq * G + G - 1),
-                              X);
-#pragma unroll
-                for (int dt = 0; dt < DT; dt++)
-#pragma unroll
-                    for (int ft = 0; ft < FT; ft++) X[dt][ft] = X[dt][ft] + S[dt][ft];
-            }
-        }
-        if (failed && lane == 0)
+        xch.gather(S, X);
+        if (xch.failed && lane == 0)
             __hip_atomic_store(hdr + kHdrError, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 #pragma unroll
         for (int dt = 0; dt < DT; dt++)
