@@ -58,7 +58,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="cfg2", choices=sorted(WORKLOADS))
+    ap.add_argument("--workload", default="cfg2", choices=sorted(WORKLOADS) + ["cfg4"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--sets", type=int, default=0, help="input sets to rotate over (0 = auto)")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -74,6 +74,9 @@ def main():
     from fast_transformers_amd import _native
     from fast_transformers_amd.causal_product import causal_dot_product_hip, \
         causal_dot_backward_hip
+
+    if args.workload == "cfg4":
+        return encoder_workload(args)
 
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible", file=sys.stderr)
@@ -230,6 +233,64 @@ def main():
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(N, H, L, E, M, seed, args.workload)
     print(json.dumps(result))
+
+
+def encoder_workload(args):
+    """Config 4: eval forward of an 8-layer causal-linear encoder (8 heads, query/value
+    dims 64, d_model 512, FFN 1024, random-init weights) on rand(10, 4096, 512).  A step is
+    one forward pass; the share of causal_dot_product is timed with events around the
+    native call inside the attention module."""
+    import torch
+    from fast_transformers_amd.attention import build_causal_linear_encoder
+    from fast_transformers_amd.attention import causal_linear_attention as cla
+    from fast_transformers_amd.masking import TriangularCausalMask
+
+    torch.cuda.set_device(0)
+    torch.manual_seed(4)
+    N, L, D = 10, 4096, 512
+    enc = build_causal_linear_encoder(8, 8, 64, 64, 1024).cuda().eval()
+    x = torch.rand(N, L, D, generator=torch.Generator().manual_seed(4)).cuda()
+    mask = TriangularCausalMask(L, device="cuda")
+    op_events = []
+    native = cla.causal_dot_product_hip
+
+    def timed(*a):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        native(*a)
+        e1.record()
+        op_events.append((e0, e1))
+
+    with torch.no_grad():
+        for _ in range(args.warmup):
+            enc(x, attn_mask=mask)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            enc(x, attn_mask=mask)
+        torch.cuda.synchronize()
+        ms = (time.perf_counter() - t0) * 1e3 / args.steps
+        cla.causal_dot_product_hip = timed
+        for _ in range(args.steps):
+            enc(x, attn_mask=mask)
+        torch.cuda.synchronize()
+        cla.causal_dot_product_hip = native
+    op_ms = sum(a.elapsed_time(b) for a, b in op_events) / args.steps
+    TH = N * 8 * L
+    print(json.dumps({
+        "metric": "causal-linear encoder eval forward Mtokens/s (8 layers, d_model 512); "
+                  "causal_dot_product share reported in config",
+        "value": round(N * L / (ms * 1e-3) / 1e6, 3), "unit": "Mtokens/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": "cfg4: 8-layer causal-linear TransformerEncoder eval forward, "
+                               "X=rand(10,4096,512), 8 heads, E=M=64, FFN 1024",
+                   "causal_dot_product_ms_per_forward": round(op_ms, 4),
+                   "causal_dot_product_share": round(op_ms / ms, 4),
+                   "causal_dot_product_fwd_alg_GBps":
+                       round(8 * 1024 * TH / (op_ms * 1e-3) / 1e9, 1)},
+    }))
 
 
 def cpu_baseline(N, H, L, E, M, seed, workload):
