@@ -74,7 +74,7 @@ int generic_scan(const Operand &a, const Operand &b, const Operand &v, const Ope
                  size_t workspace_bytes, hipStream_t stream);
 
 // ---------------------------------------------------------------------------
-// MFMA scan ((D, F) in {(64,64), (32,128), (128,32)}, 16-byte aligned rows; all-fp32 operands
+// MFMA scan (D, F multiples of 32 with D * F <= 4096, 16-byte aligned rows; all-fp32 operands
 // or the bf16 combinations of a forward / backward call): ftc_mfma.hip + ftc_mfma_kernel.h.
 // ---------------------------------------------------------------------------
 struct ScanDesc {

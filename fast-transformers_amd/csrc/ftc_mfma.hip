@@ -87,7 +87,8 @@ bool mfma_scan_supported(const ScanDesc &sd, int64_t L) {
     const Operand &a = sd.a, &b = sd.b, &v = sd.v;
     const OperandOut &out = sd.out;
     const int D = a.width, F = v.width;
-    const bool shape_ok = (D == 64 && F == 64) || (D == 32 && F == 128) || (D == 128 && F == 32);
+    const bool shape_ok = (D == 64 && F == 64) || (D == 32 && F == 128) || (D == 128 && F == 32) ||
+                          (D == 32 && F == 32) || (D == 32 && F == 64) || (D == 64 && F == 32);
     if (!shape_ok) return false;
     if (combo_of(sd) == kNone) return false;
     if (L > 1 && !(stride_ok(a.stride_l, D) && stride_ok(b.stride_l, D) &&

@@ -1,5 +1,6 @@
-// MFMA causal scan for gfx950, (D, F) in {(64,64), (32,128), (128,32)}; every operand is fp32
-// or bf16 rows (chosen per operand at compile time), the state and all sums are fp32.
+// MFMA causal scan for gfx950, row widths D, F multiples of 32 with D * F <= 4096; every
+// operand is fp32 or bf16 rows (chosen per operand at compile time), the state and all
+// sums are fp32.
 //
 //   out[c, l, f] = sum_{j <= l} (a[c,l,:] . b[c,j,:]) * v[c,j,f]      (REV: j >= l)
 //
@@ -778,15 +779,16 @@ __global__ __launch_bounds__(kWave) void scan_mfma_kernel(uint32_t *__restrict__
 template <typename TA, typename TB, typename TV, typename TO>
 void launch_scan(int D, int F, void *workspace, const ScanArgs &args, hipStream_t stream) {
     const dim3 grid((unsigned)args.total_waves), block(kWave);
-    if (D == 64 && F == 64)
-        hipLaunchKernelGGL((scan_mfma_kernel<64, 64, TA, TB, TV, TO>), grid, block, 0, stream,
-                           (uint32_t *)workspace, args);
-    else if (D == 32 && F == 128)
-        hipLaunchKernelGGL((scan_mfma_kernel<32, 128, TA, TB, TV, TO>), grid, block, 0, stream,
-                           (uint32_t *)workspace, args);
-    else
-        hipLaunchKernelGGL((scan_mfma_kernel<128, 32, TA, TB, TV, TO>), grid, block, 0, stream,
-                           (uint32_t *)workspace, args);
+#define FTC_LAUNCH(DD, FF)                                                                      \
+    hipLaunchKernelGGL((scan_mfma_kernel<DD, FF, TA, TB, TV, TO>), grid, block, 0, stream,      \
+                       (uint32_t *)workspace, args)
+    if (D == 64 && F == 64) FTC_LAUNCH(64, 64);
+    else if (D == 32 && F == 128) FTC_LAUNCH(32, 128);
+    else if (D == 128 && F == 32) FTC_LAUNCH(128, 32);
+    else if (D == 32 && F == 32) FTC_LAUNCH(32, 32);
+    else if (D == 32 && F == 64) FTC_LAUNCH(32, 64);
+    else FTC_LAUNCH(64, 32);
+#undef FTC_LAUNCH
 }
 
 // One function per element-type combination, each compiled in its own file.

@@ -102,6 +102,12 @@ CONFIG_SHAPES = {
     "e128_m128": (2, 2, 300, 128, 128, 7),
     "e25_m64": (10, 4, 100, 25, 64, 8),
     "l1": (2, 3, 1, 16, 16, 9),
+    # further MFMA shapes
+    "e32_m32": (3, 4, 700, 32, 32, 13),
+    "e32_m64": (2, 4, 500, 32, 64, 14),
+    "e64_m32": (2, 4, 500, 64, 32, 15),
+    # many chains: one segment per chain, no state exchange
+    "many_chains": (40, 32, 96, 64, 64, 16),
 }
 
 
