@@ -33,8 +33,8 @@ MFMA_FP32_PEAK_TFLOPS = 157.3   # MI355X dense fp32 matrix, published
 # HBM bytes per scan-kernel launch (mean of the forward and the backward launch) from
 # rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script, scaled by what the same
 # counters read for the 256 MiB copy of --calibrate-copy; the runs are summarised in
-# profiles/scan_mfma_kernel_cfg2_traffic.md.  None = not measured for that workload.
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {"cfg2": 245216602}
+# profiles/scan_mfma_kernel_<workload>_traffic.md.  None = not measured for that workload.
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {"cfg2": 249753678, "cfg3": 3169514478}
 
 WORKLOADS = {
     # name: (N, H, L, E, M, dtype, seed)
