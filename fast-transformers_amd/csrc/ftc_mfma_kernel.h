@@ -86,19 +86,36 @@ __device__ __forceinline__ f32x16 mfma(const Frag &a, const Frag &b, f32x16 c) {
 __device__ __forceinline__ uint32_t pack_hi16(float x0, float x1) {
     return __builtin_amdgcn_perm(__float_as_uint(x1), __float_as_uint(x0), 0x07060302u);
 }
-__device__ __forceinline__ float drop_hi_piece(float x) {
-    return x - __uint_as_float(__float_as_uint(x) & 0xffff0000u);
+// x minus the bf16 that sits in the low (even) or high (odd) half of `pair`, exactly: one
+// v_dot2c_f32_bf16 with a (-1, 0) or (0, -1) selector instead of a mask and a subtraction.
+// The selectors live in scalar registers behind an asm so that they are not folded into an
+// inline constant (which this instruction would read as a 32-bit pattern).
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t minus_one_even() {
+    uint32_t s;
+    asm("s_mov_b32 %0, 0xbf80" : "=s"(s));
+    return s;
+}
+__device__ __forceinline__ uint32_t minus_one_odd() {
+    uint32_t s;
+    asm("s_mov_b32 %0, 0xbf800000" : "=s"(s));
+    return s;
+}
+__device__ __forceinline__ float minus_piece(float x, uint32_t pair, uint32_t selector) {
+    return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, pair),
+                                           __builtin_bit_cast(bf16x2, selector), x, false);
 }
 
-// Cut two fp32 values into NS bf16 pieces each; out[p] packs piece p of (x0, x1).
+// Cut two fp32 values into NS bf16 pieces each (by truncation, so the pieces add up to the
+// value exactly); out[p] packs piece p of (x0, x1).
 template <int NS>
 __device__ __forceinline__ void split_pair(float x0, float x1, uint32_t (&out)[NS]) {
 #pragma unroll
     for (int p = 0; p < NS; p++) {
         out[p] = pack_hi16(x0, x1);
         if (p + 1 < NS) {
-            x0 = drop_hi_piece(x0);
-            x1 = drop_hi_piece(x1);
+            x0 = minus_piece(x0, out[p], minus_one_even());
+            x1 = minus_piece(x1, out[p], minus_one_odd());
         }
     }
 }
