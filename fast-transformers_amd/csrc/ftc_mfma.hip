@@ -142,13 +142,15 @@ int mfma_scan(const ScanDesc *scans, int nscans, int64_t N, int64_t H, int64_t L
     args.nseg = pl.nseg;
     args.waves_per_scan = (int32_t)pl.waves;
     args.total_waves = (int32_t)(pl.waves * nscans);
-    // short chains: one level (every step adds the sums of all steps before it); long
-    // chains: groups of about sqrt(nseg) steps
+    // very short chains: one level (every step adds the sums of all steps before it);
+    // otherwise groups of about sqrt(nseg) steps, which moves fewer states per step
     args.group = pl.nseg;
-    if (pl.nseg > 16) {
+    if (pl.nseg > 5) {
         args.group = 1;
         while (args.group * args.group < pl.nseg) args.group++;
     }
+    // tuning aid: FTC_GROUP=<n> forces groups of n steps
+    if (const char *env = getenv("FTC_GROUP")) args.group = std::max(1, atoi(env));
 
     const Combo combo = combo_of(scans[0]);
     for (int i = 1; i < nscans; i++)
