@@ -69,35 +69,52 @@ int read_dims(const ftc_tensor4 *q, const ftc_tensor4 *v, Dims *d) {
     return FTC_OK;
 }
 
-// Runs a list of independent scans: consecutive scans that qualify for the MFMA path and
-// share their row widths go out in one launch, the rest through the generic path.
+// Runs a list of independent scans.  A scan whose shape the MFMA kernels cover is cut into
+// column slices; consecutive slices (of any of the scans) that share widths and element
+// types go out in one launch.  Everything else takes the generic path.
 int run_scans(const ScanDesc *scans, int n, int64_t N, int64_t H, int64_t L, void *workspace,
               size_t workspace_bytes, hipStream_t stream) {
-    int i = 0;
-    while (i < n) {
-        if (mfma_scan_supported(scans[i], L)) {
-            int k = 1;
-            while (i + k < n && k < kMfmaMaxScans && mfma_scan_supported(scans[i + k], L) &&
-                   mfma_scan_same_launch(scans[i], scans[i + k]))
-                k++;
-            int rc = mfma_scan(scans + i, k, N, H, L, workspace, workspace_bytes, stream);
+    ScanDesc batch[kMfmaMaxScans];
+    int nbatch = 0;
+    auto flush = [&]() -> int {
+        if (nbatch == 0) return FTC_OK;
+        const int rc = mfma_scan(batch, nbatch, N, H, L, workspace, workspace_bytes, stream);
+        nbatch = 0;
+        return rc;
+    };
+    for (int i = 0; i < n; i++) {
+        int widths[kMfmaMaxSlices];
+        int nslices = mfma_slice_widths(scans[i].a.width, scans[i].v.width, widths);
+        for (int j = 0, col = 0; j < nslices; col += widths[j], j++)
+            if (!mfma_scan_supported(mfma_slice(scans[i], col, widths[j]), L)) nslices = 0;
+        if (nslices == 0) {
+            int rc = flush();
             if (rc) return rc;
-            i += k;
-        } else {
-            int rc = generic_scan(scans[i].a, scans[i].b, scans[i].v, scans[i].out, N, H, L,
-                                  scans[i].reverse, workspace, workspace_bytes, stream);
+            rc = generic_scan(scans[i].a, scans[i].b, scans[i].v, scans[i].out, N, H, L,
+                              scans[i].reverse, workspace, workspace_bytes, stream);
             if (rc) return rc;
-            i++;
+            continue;
+        }
+        for (int j = 0, col = 0; j < nslices; col += widths[j], j++) {
+            const ScanDesc slice = mfma_slice(scans[i], col, widths[j]);
+            if (nbatch == kMfmaMaxScans || (nbatch > 0 && !mfma_scan_same_launch(batch[0], slice))) {
+                const int rc = flush();
+                if (rc) return rc;
+            }
+            batch[nbatch++] = slice;
         }
     }
-    return FTC_OK;
+    return flush();
 }
 
-// Upper bound over every way run_scans may group scans of these widths.
+// Upper bound over every way run_scans may slice and group scans of these widths.
 int64_t scan_workspace_bytes(int64_t N, int64_t H, int64_t L, int64_t D, int64_t F) {
     int64_t need = generic_scan_workspace_bytes(N, H, L, D, F);
-    for (int k = 1; k <= kMfmaMaxScans; k++)
-        need = std::max(need, mfma_scan_workspace_bytes(N, H, L, D, F, k));
+    int widths[kMfmaMaxSlices];
+    const int nslices = mfma_slice_widths(D, F, widths);
+    for (int j = 0; j < nslices; j++)
+        for (int k = 1; k <= kMfmaMaxScans; k++)
+            need = std::max(need, mfma_scan_workspace_bytes(N, H, L, D, widths[j], k));
     return need;
 }
 

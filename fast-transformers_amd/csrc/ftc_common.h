@@ -74,16 +74,25 @@ int generic_scan(const Operand &a, const Operand &b, const Operand &v, const Ope
                  size_t workspace_bytes, hipStream_t stream);
 
 // ---------------------------------------------------------------------------
-// MFMA scan (D, F multiples of 32 with D * F <= 4096, 16-byte aligned rows; all-fp32 operands
-// or the bf16 combinations of a forward / backward call): ftc_mfma.hip + ftc_mfma_kernel.h.
+// MFMA scan: ftc_mfma.hip + ftc_mfma_kernel.h.  One wavefront keeps a D x F state with
+// (D, F) in {32, 64, 128} x multiples of 32 and D * F <= 4096; wider outputs are cut into
+// column slices of such widths, each slice a scan of its own over the same a and b rows.
+// Rows must be 16-byte aligned; all-fp32 operands or the bf16 combinations of a forward /
+// backward call.
 // ---------------------------------------------------------------------------
 struct ScanDesc {
     Operand a, b, v;
     OperandOut out;
     bool reverse;
 };
-constexpr int kMfmaMaxScans = 3;
+constexpr int kMfmaMaxScans = 4;   // scans per launch
+constexpr int kMfmaMaxSlices = 16;  // column slices per scan
 
+// Widths of the column slices that cover F output columns for state rows of width D;
+// returns their number (0: this shape does not go to the MFMA path).
+int mfma_slice_widths(int64_t D, int64_t F, int (&widths)[kMfmaMaxSlices]);
+// Column slice [col0, col0 + width) of a scan: same a and b rows, offset v and out rows.
+ScanDesc mfma_slice(const ScanDesc &scan, int col0, int width);
 bool mfma_scan_supported(const ScanDesc &scan, int64_t L);
 // true when two supported scans can share a launch (same widths, same element types)
 bool mfma_scan_same_launch(const ScanDesc &x, const ScanDesc &y);

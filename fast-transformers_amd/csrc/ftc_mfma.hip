@@ -79,6 +79,31 @@ bool stride_ok(int64_t stride_l, int width) { return stride_l >= width && stride
 
 }  // namespace
 
+int mfma_slice_widths(int64_t D, int64_t F, int (&widths)[kMfmaMaxSlices]) {
+    // the widest state a wavefront holds is 4096 values
+    const int widest = D == 32 ? 128 : D == 64 ? 64 : D == 128 ? 32 : 0;
+    if (widest == 0 || F < 32 || F % 32 != 0) return 0;
+    int n = 0;
+    for (int64_t left = F; left > 0;) {
+        int w = widest;
+        while (w > left) w /= 2;
+        if (n == kMfmaMaxSlices) return 0;
+        widths[n++] = w;
+        left -= w;
+    }
+    return n;
+}
+
+ScanDesc mfma_slice(const ScanDesc &scan, int col0, int width) {
+    ScanDesc s = scan;
+    const int vb = scan.v.dtype == FTC_F32 ? 4 : 2, ob = scan.out.dtype == FTC_F32 ? 4 : 2;
+    s.v.ptr = (const char *)scan.v.ptr + (int64_t)col0 * vb;
+    s.v.width = width;
+    s.out.ptr = (char *)scan.out.ptr + (int64_t)col0 * ob;
+    s.out.width = width;
+    return s;
+}
+
 bool mfma_scan_same_launch(const ScanDesc &x, const ScanDesc &y) {
     return combo_of(x) == combo_of(y) && x.a.width == y.a.width && x.v.width == y.v.width;
 }

@@ -396,8 +396,8 @@ struct StateExchange {
 };
 
 // One scan of a launch.  A launch runs up to kMaxScans independent scans of the same
-// (D, F, N, H, L) side by side (the three gradients of a backward call), so that their
-// launch gaps and wait times overlap.
+// (D, F, N, H, L) side by side (the three gradients of a backward call, the column slices
+// of a wide output), so that their launch gaps and wait times overlap.
 struct ScanOperands {
     const void *a, *b, *v;
     void *out;
@@ -408,7 +408,7 @@ struct ScanOperands {
     int32_t rev;  // 0: j <= l, walk up; 1: j >= l, walk down
     int32_t pad;
 };
-constexpr int kMaxScans = 3;
+constexpr int kMaxScans = kMfmaMaxScans;
 
 struct ScanArgs {
     ScanOperands scan[kMaxScans];
@@ -737,15 +737,18 @@ __global__ __launch_bounds__(kWave) void scan_mfma_kernel(uint32_t *__restrict__
 #pragma unroll
             for (int hh = 0; hh < 2; hh++) vt_frags(buf, ft, hh, v_frag[ft][hh]);
 
-        // (2b) + (2a) per output tile, then store
+        // (2b) + (2a): the output tiles advance side by side so that their MFMA chains are
+        // independent of each other, then store
         const uint32_t o_off = o_lane + (uint32_t)row0 * o_slb;
+        f32x16 O[FT];
 #pragma unroll
-        for (int ft = 0; ft < FT; ft++) {
-            f32x16 O;
+        for (int ft = 0; ft < FT; ft++)
 #pragma unroll
-            for (int r = 0; r < 16; r++) O[r] = 0.f;
+            for (int r = 0; r < 16; r++) O[ft][r] = 0.f;
 #pragma unroll
-            for (int ks = 0; ks < KD; ks++) {
+        for (int ks = 0; ks < KD; ks++) {
+#pragma unroll
+            for (int ft = 0; ft < FT; ft++) {
                 const int o8 = 8 * (ks % 2);
                 const float x[8] = {S[ks / 2][ft][o8 + 0], S[ks / 2][ft][o8 + 1],
                                     S[ks / 2][ft][o8 + 2], S[ks / 2][ft][o8 + 3],
@@ -753,16 +756,22 @@ __global__ __launch_bounds__(kWave) void scan_mfma_kernel(uint32_t *__restrict__
                                     S[ks / 2][ft][o8 + 6], S[ks / 2][ft][o8 + 7]};
                 Frag s_frag[NS];
                 split8<NS>(x, s_frag);
-                O = mfma_split<NS, NSA>(s_frag, a_frag[ks], O);
+                O[ft] = mfma_split<NS, NSA>(s_frag, a_frag[ks], O[ft]);
             }
+        }
 #pragma unroll
-            for (int hh = 0; hh < 2; hh++) O = mfma_split<NSV, NS>(v_frag[ft][hh], p_frag[hh], O);
-            // lane (i = ln, g) holds f = 32*ft + 8*q + 4*g + 0..3 in registers 4q..4q+3
+        for (int hh = 0; hh < 2; hh++)
+#pragma unroll
+            for (int ft = 0; ft < FT; ft++)
+                O[ft] = mfma_split<NSV, NS>(v_frag[ft][hh], p_frag[hh], O[ft]);
+        // lane (i = ln, g) holds f = 32*ft + 8*q + 4*g + 0..3 in registers 4q..4q+3
+#pragma unroll
+        for (int ft = 0; ft < FT; ft++)
 #pragma unroll
             for (int q = 0; q < 4; q++)
-                buffer_store_out(o_rs, o_off + (uint32_t)(BO * (32 * ft + 8 * q)), O[4 * q + 0],
-                                 O[4 * q + 1], O[4 * q + 2], O[4 * q + 3], (TO *)nullptr);
-        }
+                buffer_store_out(o_rs, o_off + (uint32_t)(BO * (32 * ft + 8 * q)), O[ft][4 * q + 0],
+                                 O[ft][4 * q + 1], O[ft][4 * q + 2], O[ft][4 * q + 3],
+                                 (TO *)nullptr);
 
         Frag bt_frag[DT][2][NSB];
 #pragma unroll

@@ -108,6 +108,12 @@ CONFIG_SHAPES = {
     "e64_m32": (2, 4, 500, 64, 32, 15),
     # many chains: one segment per chain, no state exchange
     "many_chains": (40, 32, 96, 64, 64, 16),
+    # outputs wider than one wavefront's state: column slices on the MFMA path
+    "e64_m128": (2, 3, 600, 64, 128, 17),
+    "e128_m64": (2, 3, 600, 128, 64, 18),
+    "e32_m256": (1, 4, 520, 32, 256, 19),
+    "e64_m96": (2, 2, 450, 64, 96, 20),      # slices of 64 and 32; dQ, dK have 96-wide states
+    "e128_m256": (1, 2, 300, 128, 256, 21),  # eight slices: more than one launch
 }
 
 
@@ -222,6 +228,8 @@ BF16_SHAPES = {
     "e64_m64": (2, 3, 1000, 64, 64, 11),
     # an odd shape: generic path
     "e40_m24": (2, 2, 300, 40, 24, 12),
+    # column slices
+    "e128_m128": (1, 3, 700, 128, 128, 22),
 }
 
 
