@@ -75,7 +75,7 @@ int generic_scan(const Operand &a, const Operand &b, const Operand &v, const Ope
 
 // ---------------------------------------------------------------------------
 // MFMA scan: ftc_mfma.hip + ftc_mfma_kernel.h.  One wavefront keeps a D x F state with
-// (D, F) in {32, 64, 128} x multiples of 32 and D * F <= 4096; wider outputs are cut into
+// (D, F) in {32, 64, 96, 128} x multiples of 32 and D * F <= 4096; wider outputs are cut into
 // column slices of such widths, each slice a scan of its own over the same a and b rows.
 // Rows must be 16-byte aligned; all-fp32 operands or the bf16 combinations of a forward /
 // backward call.

@@ -81,7 +81,7 @@ bool stride_ok(int64_t stride_l, int width) { return stride_l >= width && stride
 
 int mfma_slice_widths(int64_t D, int64_t F, int (&widths)[kMfmaMaxSlices]) {
     // the widest state a wavefront holds is 4096 values
-    const int widest = D == 32 ? 128 : D == 64 ? 64 : D == 128 ? 32 : 0;
+    const int widest = D == 32 ? 128 : D == 64 ? 64 : (D == 96 || D == 128) ? 32 : 0;
     if (widest == 0 || F < 32 || F % 32 != 0) return 0;
     int n = 0;
     for (int64_t left = F; left > 0;) {
@@ -113,7 +113,8 @@ bool mfma_scan_supported(const ScanDesc &sd, int64_t L) {
     const OperandOut &out = sd.out;
     const int D = a.width, F = v.width;
     const bool shape_ok = (D == 64 && F == 64) || (D == 32 && F == 128) || (D == 128 && F == 32) ||
-                          (D == 32 && F == 32) || (D == 32 && F == 64) || (D == 64 && F == 32);
+                          (D == 32 && F == 32) || (D == 32 && F == 64) || (D == 64 && F == 32) ||
+                          (D == 96 && F == 32);
     if (!shape_ok) return false;
     if (combo_of(sd) == kNone) return false;
     if (L > 1 && !(stride_ok(a.stride_l, D) && stride_ok(b.stride_l, D) &&

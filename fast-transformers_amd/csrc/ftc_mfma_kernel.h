@@ -813,6 +813,7 @@ void launch_scan(int D, int F, void *workspace, const ScanArgs &args, hipStream_
     else if (D == 128 && F == 32) FTC_LAUNCH(128, 32);
     else if (D == 32 && F == 32) FTC_LAUNCH(32, 32);
     else if (D == 32 && F == 64) FTC_LAUNCH(32, 64);
+    else if (D == 96 && F == 32) FTC_LAUNCH(96, 32);
     else FTC_LAUNCH(64, 32);
 #undef FTC_LAUNCH
 }

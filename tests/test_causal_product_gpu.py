@@ -114,6 +114,7 @@ CONFIG_SHAPES = {
     "e32_m256": (1, 4, 520, 32, 256, 19),
     "e64_m96": (2, 2, 450, 64, 96, 20),      # slices of 64 and 32; dQ, dK have 96-wide states
     "e128_m256": (1, 2, 300, 128, 256, 21),  # eight slices: more than one launch
+    "e96_m96": (2, 3, 500, 96, 96, 23),
 }
 
 
