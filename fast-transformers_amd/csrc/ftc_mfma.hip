@@ -3,7 +3,7 @@
 #include <algorithm>
 #include <cstdlib>
 
-#include "ftc_mfma_kernel.h"
+#include "ftc_mfma_dma_kernel.h"
 
 namespace ftc {
 using namespace mfma;
@@ -182,7 +182,11 @@ int mfma_scan(const ScanDesc *scans, int nscans, int64_t N, int64_t H, int64_t L
     for (int i = 1; i < nscans; i++)
         if (combo_of(scans[i]) != combo || scans[i].a.width != D || scans[i].v.width != F)
             return fail(FTC_ERR_INVALID, "scans of one launch must share widths and dtypes");
-    switch (combo) {
+    bool dma = D <= 64 && combo == kFFFF;
+    if (const char *env = getenv("FTC_DMA")) dma = dma && atoi(env) != 0;  // tuning aid
+    if (dma) {
+        launch_scan_dma_ffff(D, F, workspace, args, stream);
+    } else switch (combo) {
         case kFFFF: launch_scan_ffff(D, F, workspace, args, stream); break;
         case kBBBF: launch_scan_bbbf(D, F, workspace, args, stream); break;
         case kFBBB: launch_scan_fbbb(D, F, workspace, args, stream); break;
