@@ -182,6 +182,7 @@ int mfma_scan(const ScanDesc *scans, int nscans, int64_t N, int64_t H, int64_t L
     for (int i = 1; i < nscans; i++)
         if (combo_of(scans[i]) != combo || scans[i].a.width != D || scans[i].v.width != F)
             return fail(FTC_ERR_INVALID, "scans of one launch must share widths and dtypes");
+    // fp32 states of up to 64 rows: the kernel that feeds its fragments from LDS tiles
     bool dma = D <= 64 && combo == kFFFF;
     if (const char *env = getenv("FTC_DMA")) dma = dma && atoi(env) != 0;  // tuning aid
     if (dma) {

@@ -1,12 +1,11 @@
-// Instantiations of the LDS-fed MFMA scan kernel for (a, b, v, out) = (fp32, fp32, fp32,
-// fp32); see ftc_mfma_dma_kernel.h.
+// Instantiations of the LDS-fed MFMA scan kernel for (a, b, v, out) = (fp32, fp32, fp32, fp32);
+// see ftc_mfma_dma_kernel.h.
 #include "ftc_mfma_dma_kernel.h"
 
 namespace ftc {
 namespace mfma {
-#define FTC_INSTANTIATE(DD, FF)                                                                  \
-    template __global__ void scan_dma_kernel<DD, FF, float, float, float, float>(uint32_t *,     \
-                                                                                 ScanArgs)
+#define FTC_INSTANTIATE(DD, FF) \
+    template __global__ void scan_dma_kernel<DD, FF, float, float, float, float>(uint32_t *, ScanArgs)
 FTC_INSTANTIATE(64, 64);
 FTC_INSTANTIATE(32, 128);
 FTC_INSTANTIATE(32, 32);

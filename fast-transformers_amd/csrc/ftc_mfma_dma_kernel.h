@@ -140,68 +140,15 @@ __global__ __launch_bounds__(kWave) void scan_dma_kernel(uint32_t *__restrict__ 
     const uint32_t vblock = scan_id * wps + wave_in_scan;
     const ScanOperands &op = p.scan[scan_id];
     const bool REV = op.rev != 0;
-    uint32_t ticket = 0;
-    if (p.nseg > 1) {
-        const uint32_t my_chain = vblock / (uint32_t)p.nseg;
-        uint32_t order = 0;
-        if (lane == 0)
-            order = __hip_atomic_fetch_add(flags + kMaxWaves + my_chain, 1u, __ATOMIC_RELAXED,
-                                           __HIP_MEMORY_SCOPE_AGENT);
-        order = __builtin_amdgcn_readfirstlane(order);
-        ticket = my_chain * (uint32_t)p.nseg + order;
-        if (order >= (uint32_t)p.nseg) {
-            if (lane == 0)
-                __hip_atomic_store(hdr + kHdrError, 2u, __ATOMIC_RELAXED,
-                                   __HIP_MEMORY_SCOPE_AGENT);
-            return;
-        }
-    } else {
-        ticket = vblock;
-    }
-    const int64_t chain = (ticket - scan_id * wps) / (uint32_t)p.nseg;
-    const int step = (int)(ticket % (uint32_t)p.nseg);
-    const int seg = REV ? p.nseg - 1 - step : step;
-    const int n = (int)(chain / p.H), h = (int)(chain % p.H);
-    const int64_t lo = (int64_t)seg * p.seg_len;
-    const int64_t hi = min(p.L, lo + (int64_t)p.seg_len);
-    const int rows = (int)(hi - lo);
-    const int nchunks = (rows + kChunk - 1) / kChunk;
-
-    const char *a_seg =
-        (const char *)op.a + ((int64_t)n * op.a_sn + (int64_t)h * op.a_sh + lo * op.a_sl) * BA;
-    const char *b_seg =
-        (const char *)op.b + ((int64_t)n * op.b_sn + (int64_t)h * op.b_sh + lo * op.b_sl) * BB;
-    const char *v_seg =
-        (const char *)op.v + ((int64_t)n * op.v_sn + (int64_t)h * op.v_sh + lo * op.v_sl) * BV;
-    char *o_seg = (char *)op.out + ((int64_t)n * op.o_sn + (int64_t)h * op.o_sh + lo * op.o_sl) * BO;
+    // the ticket is asked for here and looked at only after the per-lane address tables,
+    // which do not depend on it, have been set up
+    const uint32_t my_chain = vblock / (uint32_t)p.nseg;
+    uint32_t order = 0;
+    if (p.nseg > 1 && lane == 0)
+        order = __hip_atomic_fetch_add(flags + kMaxWaves + my_chain, 1u, __ATOMIC_RELAXED,
+                                       __HIP_MEMORY_SCOPE_AGENT);
     const uint32_t a_slb = (uint32_t)op.a_sl * BA, b_slb = (uint32_t)op.b_sl * BB,
                    v_slb = (uint32_t)op.v_sl * BV, o_slb = (uint32_t)op.o_sl * BO;
-    const __amdgpu_buffer_rsrc_t a_rs = __builtin_amdgcn_make_buffer_rsrc(
-        (void *)a_seg, 0, (rows - 1) * a_slb + RBA, kRsrcFlags);
-    const __amdgpu_buffer_rsrc_t b_rs = __builtin_amdgcn_make_buffer_rsrc(
-        (void *)b_seg, 0, (rows - 1) * b_slb + RBB, kRsrcFlags);
-    const __amdgpu_buffer_rsrc_t v_rs = __builtin_amdgcn_make_buffer_rsrc(
-        (void *)v_seg, 0, (rows - 1) * v_slb + RBV, kRsrcFlags);
-    const __amdgpu_buffer_rsrc_t o_rs = __builtin_amdgcn_make_buffer_rsrc(
-        (void *)o_seg, 0, (rows - 1) * o_slb + F * BO, kRsrcFlags);
-    const uint32_t o_lane = ln * o_slb + 4u * BO * g;
-
-    auto chunk_row0 = [&](int c) -> int { return REV ? rows - kChunk * (c + 1) : kChunk * c; };
-    auto pass1_row0 = [&](int c) -> int { return c < 0 ? -2 * kChunk : chunk_row0(c); };
-
-    // ---- LDS tiles (separate arrays: the compiler then waits per tile, not for all) ----
-    __shared__ __align__(16) char a_tile_mem[kChunk * RBA];
-    __shared__ __align__(16) char b_tile0_mem[kChunk * RBB];
-    __shared__ __align__(16) char b_tile1_mem[kChunk * RBB];
-    __shared__ __align__(16) char v_tile_mem[kChunk * RBV];
-    // pass 1 alternates v between v_tile and a second tile: a's, when it is large enough
-    constexpr bool kVinA = RBA >= RBV;
-    constexpr bool kVSecond = kVinA || (kChunk * (RBA + 2 * RBB + 2 * RBV) <= 40960);
-    __shared__ __align__(16) char v_tile_extra_mem[(kVSecond && !kVinA) ? kChunk * RBV : 16];
-    lds_char *const a_tile = (lds_char *)a_tile_mem, *const b_tile0 = (lds_char *)b_tile0_mem,
-                    *const b_tile1 = (lds_char *)b_tile1_mem, *const v_tile = (lds_char *)v_tile_mem;
-    lds_char *const v_second = kVinA ? a_tile : (lds_char *)v_tile_extra_mem;
-
     TileRequest<RBA> a_req;
     TileRequest<RBB> b_req;
     TileRequest<RBV> v_req;
@@ -232,6 +179,73 @@ __global__ __launch_bounds__(kWave) void scan_dma_kernel(uint32_t *__restrict__ 
         for (int ft = 0; ft < FT; ft++)
             v_col_addr[ft][t] = Swizzle<RBV>::addr(row, (32 * ft + ln) * BV);
     }
+    // causal mask inside a chunk as bit masks (all ones: keep): accumulator register r of
+    // lane (i = ln, g) holds row j = 8*(r/4) + 4*g + r%4 of Pt
+    uint32_t keep[16];
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+        const int j = 8 * (r / 4) + 4 * g + (r % 4);
+        keep[r] = (REV ? (j >= ln) : (j <= ln)) ? 0xffffffffu : 0u;
+        // kept in a vector register: as 16 lane masks in scalar registers they would push
+        // other scalars out
+        asm volatile("" : "+v"(keep[r]));
+    }
+
+    uint32_t ticket = 0;
+    if (p.nseg > 1) {
+        order = __builtin_amdgcn_readfirstlane(order);
+        ticket = my_chain * (uint32_t)p.nseg + order;
+        if (order >= (uint32_t)p.nseg) {
+            if (lane == 0)
+                __hip_atomic_store(hdr + kHdrError, 2u, __ATOMIC_RELAXED,
+                                   __HIP_MEMORY_SCOPE_AGENT);
+            return;
+        }
+    } else {
+        ticket = vblock;
+    }
+    const int64_t chain = (ticket - scan_id * wps) / (uint32_t)p.nseg;
+    const int step = (int)(ticket % (uint32_t)p.nseg);
+    const int seg = REV ? p.nseg - 1 - step : step;
+    const int n = (int)(chain / p.H), h = (int)(chain % p.H);
+    const int64_t lo = (int64_t)seg * p.seg_len;
+    const int64_t hi = min(p.L, lo + (int64_t)p.seg_len);
+    const int rows = (int)(hi - lo);
+    const int nchunks = (rows + kChunk - 1) / kChunk;
+
+    const char *a_seg =
+        (const char *)op.a + ((int64_t)n * op.a_sn + (int64_t)h * op.a_sh + lo * op.a_sl) * BA;
+    const char *b_seg =
+        (const char *)op.b + ((int64_t)n * op.b_sn + (int64_t)h * op.b_sh + lo * op.b_sl) * BB;
+    const char *v_seg =
+        (const char *)op.v + ((int64_t)n * op.v_sn + (int64_t)h * op.v_sh + lo * op.v_sl) * BV;
+    char *o_seg = (char *)op.out + ((int64_t)n * op.o_sn + (int64_t)h * op.o_sh + lo * op.o_sl) * BO;
+    const __amdgpu_buffer_rsrc_t a_rs = __builtin_amdgcn_make_buffer_rsrc(
+        (void *)a_seg, 0, (rows - 1) * a_slb + RBA, kRsrcFlags);
+    const __amdgpu_buffer_rsrc_t b_rs = __builtin_amdgcn_make_buffer_rsrc(
+        (void *)b_seg, 0, (rows - 1) * b_slb + RBB, kRsrcFlags);
+    const __amdgpu_buffer_rsrc_t v_rs = __builtin_amdgcn_make_buffer_rsrc(
+        (void *)v_seg, 0, (rows - 1) * v_slb + RBV, kRsrcFlags);
+    const __amdgpu_buffer_rsrc_t o_rs = __builtin_amdgcn_make_buffer_rsrc(
+        (void *)o_seg, 0, (rows - 1) * o_slb + F * BO, kRsrcFlags);
+    const uint32_t o_lane = ln * o_slb + 4u * BO * g;
+
+    auto chunk_row0 = [&](int c) -> int { return REV ? rows - kChunk * (c + 1) : kChunk * c; };
+    auto pass1_row0 = [&](int c) -> int { return c < 0 ? -2 * kChunk : chunk_row0(c); };
+
+    // ---- LDS tiles (separate arrays: the compiler then waits per tile, not for all) ----
+    __shared__ __align__(16) char a_tile_mem[kChunk * RBA];
+    __shared__ __align__(16) char b_tile0_mem[kChunk * RBB];
+    __shared__ __align__(16) char b_tile1_mem[kChunk * RBB];
+    __shared__ __align__(16) char v_tile_mem[kChunk * RBV];
+    // pass 1 alternates v between v_tile and a second tile: a's, when it is large enough
+    constexpr bool kVinA = RBA >= RBV;
+    constexpr bool kVSecond = kVinA || (kChunk * (RBA + 2 * RBB + 2 * RBV) <= 40960);
+    __shared__ __align__(16) char v_tile_extra_mem[(kVSecond && !kVinA) ? kChunk * RBV : 16];
+    lds_char *const a_tile = (lds_char *)a_tile_mem, *const b_tile0 = (lds_char *)b_tile0_mem,
+                    *const b_tile1 = (lds_char *)b_tile1_mem, *const v_tile = (lds_char *)v_tile_mem;
+    lds_char *const v_second = kVinA ? a_tile : (lds_char *)v_tile_extra_mem;
+
     auto bt_frags = [&](const lds_char *tile, int dt, int hh, Frag (&frag)[NSB]) {
         lds_column_to_frags(tile, b_col_addr[dt], hh * 16 * RBB, frag, (TB *)nullptr);
     };
@@ -303,18 +317,6 @@ __global__ __launch_bounds__(kWave) void scan_dma_kernel(uint32_t *__restrict__ 
         for (int dt = 0; dt < DT; dt++)
 #pragma unroll
             for (int ft = 0; ft < FT; ft++) S[dt][ft] = X[dt][ft];
-    }
-
-    // causal mask inside a chunk as bit masks (all ones: keep): accumulator register r of
-    // lane (i = ln, g) holds row j = 8*(r/4) + 4*g + r%4 of Pt
-    uint32_t keep[16];
-#pragma unroll
-    for (int r = 0; r < 16; r++) {
-        const int j = 8 * (r / 4) + 4 * g + (r % 4);
-        keep[r] = (REV ? (j >= ln) : (j <= ln)) ? 0xffffffffu : 0u;
-        // kept in a vector register: as 16 lane masks in scalar registers they would push
-        // other scalars out
-        asm volatile("" : "+v"(keep[r]));
     }
 
     // ---- pass 2: outputs.  b alternates between its two tiles, hence the chunk pairs. ----
@@ -444,6 +446,8 @@ void launch_scan_dma(int D, int F, void *workspace, const ScanArgs &args, hipStr
 #undef FTC_LAUNCH
 }
 
+// Instantiated for all-fp32 scans (ftc_mfma_dma_ffff.hip); with bf16 rows, which need no
+// piece split, the register-fed kernel measured as fast or faster.
 void launch_scan_dma_ffff(int D, int F, void *ws, const ScanArgs &args, hipStream_t stream);
 
 }  // namespace mfma
