@@ -123,30 +123,13 @@ __global__ __launch_bounds__(kWave) void scan_dma_kernel(uint32_t *__restrict__ 
     gu32 *flags = hdr + kHdrWords;
     gfloat *sums = (gfloat *)(hdr + kControlBytes / 4);
 
-    // ---- which segment (same numbering and tickets as scan_mfma_kernel) ----
-    const uint32_t wps = (uint32_t)p.waves_per_scan;
-    const uint32_t nscans = (uint32_t)p.total_waves / wps;
-    const uint32_t full = (wps / 8u) * 8u;
-    uint32_t scan_id, wave_in_scan;
-    if (blockIdx.x < full * nscans) {
-        const uint32_t grp = blockIdx.x / (8u * nscans), r = blockIdx.x % (8u * nscans);
-        scan_id = r / 8u;
-        wave_in_scan = grp * 8u + r % 8u;
-    } else {
-        const uint32_t t = blockIdx.x - full * nscans;
-        scan_id = t / (wps - full);
-        wave_in_scan = full + t % (wps - full);
-    }
-    const uint32_t vblock = scan_id * wps + wave_in_scan;
-    const ScanOperands &op = p.scan[scan_id];
-    const bool REV = op.rev != 0;
     // the ticket is asked for here and looked at only after the per-lane address tables,
     // which do not depend on it, have been set up
-    const uint32_t my_chain = vblock / (uint32_t)p.nseg;
-    uint32_t order = 0;
-    if (p.nseg > 1 && lane == 0)
-        order = __hip_atomic_fetch_add(flags + kMaxWaves + my_chain, 1u, __ATOMIC_RELAXED,
-                                       __HIP_MEMORY_SCOPE_AGENT);
+    Segment sg;
+    uint32_t order;
+    segment_request(p, flags, lane, sg, order);
+    const ScanOperands &op = p.scan[sg.scan_id];
+    const bool REV = sg.rev;
     const uint32_t a_slb = (uint32_t)op.a_sl * BA, b_slb = (uint32_t)op.b_sl * BB,
                    v_slb = (uint32_t)op.v_sl * BV, o_slb = (uint32_t)op.o_sl * BO;
     TileRequest<RBA> a_req;
@@ -191,27 +174,10 @@ __global__ __launch_bounds__(kWave) void scan_dma_kernel(uint32_t *__restrict__ 
         asm volatile("" : "+v"(keep[r]));
     }
 
-    uint32_t ticket = 0;
-    if (p.nseg > 1) {
-        order = __builtin_amdgcn_readfirstlane(order);
-        ticket = my_chain * (uint32_t)p.nseg + order;
-        if (order >= (uint32_t)p.nseg) {
-            if (lane == 0)
-                __hip_atomic_store(hdr + kHdrError, 2u, __ATOMIC_RELAXED,
-                                   __HIP_MEMORY_SCOPE_AGENT);
-            return;
-        }
-    } else {
-        ticket = vblock;
-    }
-    const int64_t chain = (ticket - scan_id * wps) / (uint32_t)p.nseg;
-    const int step = (int)(ticket % (uint32_t)p.nseg);
-    const int seg = REV ? p.nseg - 1 - step : step;
-    const int n = (int)(chain / p.H), h = (int)(chain % p.H);
-    const int64_t lo = (int64_t)seg * p.seg_len;
-    const int64_t hi = min(p.L, lo + (int64_t)p.seg_len);
-    const int rows = (int)(hi - lo);
-    const int nchunks = (rows + kChunk - 1) / kChunk;
+    if (!segment_locate(p, hdr, lane, order, sg)) return;
+    const uint32_t ticket = sg.ticket;
+    const int step = sg.step, n = sg.n, h = sg.h, rows = sg.rows, nchunks = sg.nchunks;
+    const int64_t lo = sg.lo;
 
     const char *a_seg =
         (const char *)op.a + ((int64_t)n * op.a_sn + (int64_t)h * op.a_sh + lo * op.a_sl) * BA;
@@ -411,24 +377,7 @@ __global__ __launch_bounds__(kWave) void scan_dma_kernel(uint32_t *__restrict__ 
     // nothing may still be on its way into LDS when the wavefront ends
     wait_for_stores();
 
-    // ---- the last wavefront to finish leaves the workspace zeroed for the next launch ----
-    if (p.nseg > 1) {
-        uint32_t done = 0;
-        if (lane == 0)
-            done = __hip_atomic_fetch_add(hdr + kHdrDone, 1u, __ATOMIC_RELAXED,
-                                          __HIP_MEMORY_SCOPE_AGENT);
-        done = __builtin_amdgcn_readfirstlane(done);
-        if (done == (uint32_t)p.total_waves - 1) {
-            for (int i = lane; i < p.total_waves; i += kWave)
-                __hip_atomic_store(flags + i, kFlagEmpty, __ATOMIC_RELAXED,
-                                   __HIP_MEMORY_SCOPE_AGENT);
-            for (int i = lane; i < p.total_waves / p.nseg; i += kWave)
-                __hip_atomic_store(flags + kMaxWaves + i, 0u, __ATOMIC_RELAXED,
-                                   __HIP_MEMORY_SCOPE_AGENT);
-            if (lane == 0)
-                __hip_atomic_store(hdr + kHdrDone, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        }
-    }
+    release_control_block(p, hdr, flags, lane);
 }
 
 // Host-side launcher of one element-type combination; (D, F) with D <= 64.

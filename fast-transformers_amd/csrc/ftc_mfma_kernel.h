@@ -419,6 +419,96 @@ struct ScanArgs {
     int32_t group;        // steps per group of the two-level state sum
 };
 
+// Which (scan, chain, L-segment) a wavefront works on.
+//
+// Workgroups are dispatched round-robin over the 8 XCDs.  Blocks are numbered so that
+// wavefront w of every scan of the launch lands on the same XCD at about the same time
+// (groups of 8 consecutive blocks per scan): scans that read the same rows find each other's
+// lines in that XCD's L2.  Chains of all scans are numbered consecutively
+// (scan * chains + chain), and the wavefronts launched for a chain take that chain's steps in
+// the order in which they start running (a ticket per chain), so a step only ever waits for
+// steps that are already running.
+struct Segment {
+    uint32_t scan_id, chain_slot0;  // chain_slot0: slot of step 0 of this chain
+    uint32_t ticket;                // this wavefront's flag / state slot
+    int step, seg;                  // position in dependency order, position along L
+    int n, h;
+    int64_t lo;                     // first row of the segment
+    int rows, nchunks;
+    bool rev;
+};
+
+// First half: block number -> scan and chain, and the request for a ticket (answer pending
+// in `order`, valid in lane 0).
+__device__ __forceinline__ void segment_request(const ScanArgs &p, gu32 *flags, int lane,
+                                                Segment &s, uint32_t &order) {
+    const uint32_t wps = (uint32_t)p.waves_per_scan;
+    const uint32_t nscans = (uint32_t)p.total_waves / wps;
+    const uint32_t full = (wps / 8u) * 8u;
+    uint32_t wave_in_scan;
+    if (blockIdx.x < full * nscans) {
+        const uint32_t grp = blockIdx.x / (8u * nscans), r = blockIdx.x % (8u * nscans);
+        s.scan_id = r / 8u;
+        wave_in_scan = grp * 8u + r % 8u;
+    } else {
+        const uint32_t t = blockIdx.x - full * nscans;
+        s.scan_id = t / (wps - full);
+        wave_in_scan = full + t % (wps - full);
+    }
+    const uint32_t vblock = s.scan_id * wps + wave_in_scan;  // block id in scan-major order
+    const uint32_t my_chain = vblock / (uint32_t)p.nseg;
+    s.chain_slot0 = my_chain * (uint32_t)p.nseg;
+    s.rev = p.scan[s.scan_id].rev != 0;
+    order = vblock - s.chain_slot0;  // a single segment per chain needs no ticket
+    if (p.nseg > 1 && lane == 0)
+        order = __hip_atomic_fetch_add(flags + kMaxWaves + my_chain, 1u, __ATOMIC_RELAXED,
+                                       __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// Second half: waits for the ticket.  Returns false when the control block was not zero at
+// the start of the launch (the wavefront must then stop; the error word says so).
+__device__ __forceinline__ bool segment_locate(const ScanArgs &p, gu32 *hdr, int lane,
+                                               uint32_t order, Segment &s) {
+    order = __builtin_amdgcn_readfirstlane(order);
+    if (order >= (uint32_t)p.nseg) {
+        if (lane == 0)
+            __hip_atomic_store(hdr + kHdrError, 2u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        return false;
+    }
+    s.ticket = s.chain_slot0 + order;
+    s.step = (int)order;
+    s.seg = s.rev ? p.nseg - 1 - s.step : s.step;
+    const int64_t chain =
+        (s.chain_slot0 - s.scan_id * (uint32_t)p.waves_per_scan) / (uint32_t)p.nseg;
+    s.n = (int)(chain / p.H);
+    s.h = (int)(chain % p.H);
+    s.lo = (int64_t)s.seg * p.seg_len;
+    const int64_t hi = min(p.L, s.lo + (int64_t)p.seg_len);
+    s.rows = (int)(hi - s.lo);
+    s.nchunks = (s.rows + kChunk - 1) / kChunk;
+    return true;
+}
+
+// The last wavefront of a launch to get here leaves the control block zeroed for the next
+// launch (flags, ticket counters, the counter used here).
+__device__ __forceinline__ void release_control_block(const ScanArgs &p, gu32 *hdr, gu32 *flags,
+                                                      int lane) {
+    if (p.nseg <= 1) return;
+    uint32_t done = 0;
+    if (lane == 0)
+        done = __hip_atomic_fetch_add(hdr + kHdrDone, 1u, __ATOMIC_RELAXED,
+                                      __HIP_MEMORY_SCOPE_AGENT);
+    done = __builtin_amdgcn_readfirstlane(done);
+    if (done != (uint32_t)p.total_waves - 1) return;
+    for (int i = lane; i < p.total_waves; i += kWave)
+        __hip_atomic_store(flags + i, kFlagEmpty, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    for (int i = lane; i < p.total_waves / p.nseg; i += kWave)
+        __hip_atomic_store(flags + kMaxWaves + i, 0u, __ATOMIC_RELAXED,
+                           __HIP_MEMORY_SCOPE_AGENT);
+    if (lane == 0)
+        __hip_atomic_store(hdr + kHdrDone, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
 // TA, TB, TV, TO: element types (float or bf16_t) of the a, b, v rows and of the output rows.
 template <int D, int F, typename TA, typename TB, typename TV, typename TO>
 __global__ __launch_bounds__(kWave) void scan_mfma_kernel(uint32_t *__restrict__ ws_ptr,
@@ -438,60 +528,18 @@ __global__ __launch_bounds__(kWave) void scan_mfma_kernel(uint32_t *__restrict__
     gu32 *flags = hdr + kHdrWords;
     gfloat *sums = (gfloat *)(hdr + kControlBytes / 4);
 
-    // ---- which segment: the wavefronts launched for a chain take that chain's steps in
-    // the order in which they start running, so a step only ever waits for steps that are
-    // already running ----
-    // chains of all scans are numbered consecutively: global chain = scan * chains + chain
-    // Workgroups are dispatched round-robin over the 8 XCDs.  Blocks are numbered so that
-    // wavefront w of every scan of the launch lands on the same XCD at about the same time
-    // (groups of 8 consecutive blocks per scan): scans that read the same rows in the same
-    // direction (dK and dV) then find each other's lines in that XCD's L2.
-    const uint32_t wps = (uint32_t)p.waves_per_scan;
-    const uint32_t nscans = (uint32_t)p.total_waves / wps;
-    const uint32_t full = (wps / 8u) * 8u;
-    uint32_t scan_id, wave_in_scan;
-    if (blockIdx.x < full * nscans) {
-        const uint32_t grp = blockIdx.x / (8u * nscans), r = blockIdx.x % (8u * nscans);
-        scan_id = r / 8u;
-        wave_in_scan = grp * 8u + r % 8u;
-    } else {
-        const uint32_t t = blockIdx.x - full * nscans;
-        scan_id = t / (wps - full);
-        wave_in_scan = full + t % (wps - full);
-    }
-    const uint32_t vblock = scan_id * wps + wave_in_scan;  // block id in scan-major order
-    const ScanOperands &op = p.scan[scan_id];
-    const bool REV = op.rev != 0;
+    Segment sg;
+    uint32_t order;
+    segment_request(p, flags, lane, sg, order);
+    if (!segment_locate(p, hdr, lane, order, sg)) return;
+    const ScanOperands &op = p.scan[sg.scan_id];
+    const bool REV = sg.rev;
     const char *a_ptr = (const char *)op.a, *b_ptr = (const char *)op.b,
                *v_ptr = (const char *)op.v;
     char *out_ptr = (char *)op.out;
-    uint32_t ticket = 0;
-    if (p.nseg > 1) {
-        const uint32_t my_chain = vblock / (uint32_t)p.nseg;
-        uint32_t order = 0;
-        if (lane == 0)
-            order = __hip_atomic_fetch_add(flags + kMaxWaves + my_chain, 1u, __ATOMIC_RELAXED,
-                                           __HIP_MEMORY_SCOPE_AGENT);
-        order = __builtin_amdgcn_readfirstlane(order);
-        ticket = my_chain * (uint32_t)p.nseg + order;
-        if (order >= (uint32_t)p.nseg) {
-            // the control block was not zero when the launch started: refuse to run on it
-            if (lane == 0)
-                __hip_atomic_store(hdr + kHdrError, 2u, __ATOMIC_RELAXED,
-                                   __HIP_MEMORY_SCOPE_AGENT);
-            return;
-        }
-    } else {
-        ticket = vblock;
-    }
-    const int64_t chain = (ticket - scan_id * (uint32_t)p.waves_per_scan) / (uint32_t)p.nseg;
-    const int step = (int)(ticket % (uint32_t)p.nseg);      // position in dependency order
-    const int seg = REV ? p.nseg - 1 - step : step;
-    const int n = (int)(chain / p.H), h = (int)(chain % p.H);
-    const int64_t lo = (int64_t)seg * p.seg_len;
-    const int64_t hi = min(p.L, lo + (int64_t)p.seg_len);
-    const int rows = (int)(hi - lo);
-    const int nchunks = (rows + kChunk - 1) / kChunk;
+    const uint32_t ticket = sg.ticket;
+    const int step = sg.step, n = sg.n, h = sg.h, rows = sg.rows, nchunks = sg.nchunks;
+    const int64_t lo = sg.lo;
 
     // descriptors based at the segment's first row and ending with its last row
     const char *a_seg = a_ptr + ((int64_t)n * op.a_sn + (int64_t)h * op.a_sh + lo * op.a_sl) * BA;
@@ -781,24 +829,7 @@ __global__ __launch_bounds__(kWave) void scan_mfma_kernel(uint32_t *__restrict__
         update_state(bt_frag, v_frag);
     }
 
-    // ---- the last wavefront to finish leaves the workspace zeroed for the next launch ----
-    if (p.nseg > 1) {
-        uint32_t done = 0;
-        if (lane == 0)
-            done = __hip_atomic_fetch_add(hdr + kHdrDone, 1u, __ATOMIC_RELAXED,
-                                          __HIP_MEMORY_SCOPE_AGENT);
-        done = __builtin_amdgcn_readfirstlane(done);
-        if (done == (uint32_t)p.total_waves - 1) {
-            for (int i = lane; i < p.total_waves; i += kWave)
-                __hip_atomic_store(flags + i, kFlagEmpty, __ATOMIC_RELAXED,
-                                   __HIP_MEMORY_SCOPE_AGENT);
-            for (int i = lane; i < p.total_waves / p.nseg; i += kWave)
-                __hip_atomic_store(flags + kMaxWaves + i, 0u, __ATOMIC_RELAXED,
-                                   __HIP_MEMORY_SCOPE_AGENT);
-            if (lane == 0)
-                __hip_atomic_store(hdr + kHdrDone, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        }
-    }
+    release_control_block(p, hdr, flags, lane);
 }
 
 // Host-side launcher of one element-type combination; D, F picked at run time.
