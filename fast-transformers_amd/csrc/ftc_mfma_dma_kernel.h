@@ -286,10 +286,9 @@ __global__ __launch_bounds__(kWave) void scan_dma_kernel(uint32_t *__restrict__ 
     }
 
     // ---- pass 2: outputs.  b alternates between its two tiles, hence the chunk pairs. ----
-    auto output_chunk = [&](int c, lds_char *b_tile) {
-        const int row0 = chunk_row0(c);
-        // row-major fragments of a and b; a's tile is then free for the next chunk
-        Frag a_frag[KD][NSA], b_frag[KD][NSB];
+    // row-major fragments of a chunk's a and b rows; a's tile is free afterwards
+    Frag a_frag[KD][NSA], b_frag[KD][NSB];
+    auto row_frags = [&](lds_char *b_tile) {
 #pragma unroll
         for (int ks = 0; ks < KD; ks++) {
             Quad<TA> a0, a1;
@@ -301,14 +300,26 @@ __global__ __launch_bounds__(kWave) void scan_dma_kernel(uint32_t *__restrict__ 
             lds_read_quad(b_tile + b_row_addr[ks][1], b1);
             quads_to_frags(b0, b1, b_frag[ks]);
         }
-        a_req.issue(a_rs, a_tile, chunk_row0(c + 1), a_slb);
+    };
+    row_frags(b_tile0);
+    a_req.issue(a_rs, a_tile, chunk_row0(1), a_slb);
+
+    // On entry a_frag, b_frag hold chunk c; on exit they hold chunk c + 1, cut while the
+    // matrix cores are busy with the state update.
+    auto output_chunk = [&](int c, lds_char *b_tile, lds_char *b_next) {
+        const int row0 = chunk_row0(c);
+        Frag a_cur[KD][NSA];
+#pragma unroll
+        for (int ks = 0; ks < KD; ks++)
+#pragma unroll
+            for (int pc = 0; pc < NSA; pc++) a_cur[ks][pc] = a_frag[ks][pc];
 
         // (1) Pt = b a^T
         f32x16 P;
 #pragma unroll
         for (int r = 0; r < 16; r++) P[r] = 0.f;
 #pragma unroll
-        for (int ks = 0; ks < KD; ks++) P = mfma_split<NSB, NSA>(b_frag[ks], a_frag[ks], P);
+        for (int ks = 0; ks < KD; ks++) P = mfma_split<NSB, NSA>(b_frag[ks], a_cur[ks], P);
 #pragma unroll
         for (int r = 0; r < 16; r++) P[r] = __uint_as_float(__float_as_uint(P[r]) & keep[r]);
         Frag p_frag[2][NS];
@@ -345,7 +356,7 @@ __global__ __launch_bounds__(kWave) void scan_dma_kernel(uint32_t *__restrict__ 
                                     S[ks / 2][ft][o8 + 6], S[ks / 2][ft][o8 + 7]};
                 Frag s_frag[NS];
                 split8<NS>(x, s_frag);
-                O[ft] = mfma_split<NS, NSA>(s_frag, a_frag[ks], O[ft]);
+                O[ft] = mfma_split<NS, NSA>(s_frag, a_cur[ks], O[ft]);
             }
         }
 #pragma unroll
@@ -368,11 +379,13 @@ __global__ __launch_bounds__(kWave) void scan_dma_kernel(uint32_t *__restrict__ 
 #pragma unroll
             for (int hh = 0; hh < 2; hh++) bt_frags(b_tile, dt, hh, bt_frag[dt][hh]);
         b_req.issue(b_rs, b_tile, chunk_row0(c + 2), b_slb);
+        row_frags(b_next);
+        a_req.issue(a_rs, a_tile, chunk_row0(c + 2), a_slb);
         update_state(bt_frag, v_frag);
     };
     for (int c = 0; c < nchunks; c += 2) {
-        output_chunk(c, b_tile0);
-        if (c + 1 < nchunks) output_chunk(c + 1, b_tile1);
+        output_chunk(c, b_tile0, b_tile1);
+        if (c + 1 < nchunks) output_chunk(c + 1, b_tile1, b_tile0);
     }
     // nothing may still be on its way into LDS when the wavefront ends
     wait_for_stores();
