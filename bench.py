@@ -33,8 +33,8 @@ MFMA_FP32_PEAK_TFLOPS = 157.3   # MI355X dense fp32 matrix, published
 # HBM bytes per scan-kernel launch (mean of the forward and the backward launch) from
 # rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script, scaled by what the same
 # counters read for the 256 MiB copy of --calibrate-copy; the runs are summarised in
-# profiles/scan_mfma_kernel_<workload>_traffic.md.  None = not measured for that workload.
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {"cfg2": 249753678, "cfg3": 3169514478}
+# profiles/scan_dma_kernel_<workload>_traffic.md.  None = not measured for that workload.
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {"cfg2": 233148585, "cfg3": 3190003296}
 
 WORKLOADS = {
     # name: (N, H, L, E, M, dtype, seed)
@@ -221,8 +221,9 @@ def main():
                    "fwdbwd_frac_of_hbm_roofline":
                        round((fb + bb) * TH / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)},
         "roofline": {"bound": "hbm",
-                     "kernel": "scan_mfma_kernel (mean of its forward and backward launch)"
-                               if dtype == "f32" else "generic_scan_kernel launches",
+                     "kernel": ("scan_dma_kernel" if dtype == "f32" and max(E, M) <= 64
+                                else "scan_mfma_kernel")
+                               + " (mean over the forward and the backward call)",
                      "achieved": round(launch_gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(launch_gbps / HBM_PEAK_GBPS, 4),
                      "launch_ms_avg": round(launch_ms, 5),

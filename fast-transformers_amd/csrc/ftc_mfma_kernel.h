@@ -1,6 +1,6 @@
-// MFMA causal scan for gfx950, row widths D, F multiples of 32 with D * F <= 4096; every
-// operand is fp32 or bf16 rows (chosen per operand at compile time), the state and all
-// sums are fp32.
+// MFMA causal scan for gfx950, state shapes D x F with D, F multiples of 32 and
+// D * F <= 4096; every operand is fp32 or bf16 rows (chosen per operand at compile time),
+// the state and all sums are fp32.
 //
 //   out[c, l, f] = sum_{j <= l} (a[c,l,:] . b[c,j,:]) * v[c,j,f]      (REV: j >= l)
 //
@@ -25,14 +25,13 @@
 // of the contraction index for k-step h, provided the other operand uses the same order:
 // k-slot (g, t) of a 16-wide k-step carries logical index 8*(t/4) + 4*g + (t%4).
 //
-// No LDS: every operand fragment is loaded from global memory directly in the register
-// layout its MFMA wants.  Row-major fragments (a, and b for (1)) are two 16-byte loads per
-// k-step; position-major fragments (b for (3), v) are 4-byte loads in which the 32 lanes
-// of a half-wave read 32 consecutive floats of one row, so every load instruction still
-// covers whole 128-byte lines.  b is read in both layouts; the second read hits L1/L2.
-// (An earlier version transposed b and v through LDS: bank conflicts took 79 % of its LDS
-// cycles and the write -> wait -> read round trip per chunk could not be hidden with the
-// one wavefront per SIMD that the register budget allows.)
+// Operand paths of scan_mfma_kernel (this file; ftc_mfma_dma_kernel.h feeds everything
+// through LDS instead): row-major fragments (a, and b for (1)) are two 16-byte global loads
+// per k-step, straight into the register layout the MFMA wants.  Position-major fragments
+// (b for (3), v) are fetched as whole rows with 16-byte loads, parked in a double-buffered
+// LDS tile in their own element type, and read back by column with element-wide reads
+// (consecutive lanes, consecutive banks).  b is read in both layouts; the second read hits
+// L1/L2.
 //
 // One launch per scan.  A wavefront first sums its segment's own state (reading b and v
 // only), publishes it, obtains the state that precedes its segment from the published
