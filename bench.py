@@ -56,8 +56,9 @@ def alg_bytes_per_position(E, M, dtype):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--steps", type=int, default=None, help="timed steps (default: 1000; 50 for cfg4)")
+    ap.add_argument("--warmup", type=int, default=None,
+                    help="untimed steps first (default: 200, past the clock ramp; 5 for cfg4)")
     ap.add_argument("--workload", default="cfg2", choices=sorted(WORKLOADS) + ["cfg4"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--sets", type=int, default=0, help="input sets to rotate over (0 = auto)")
@@ -65,6 +66,10 @@ def main():
                     help="also run one 256 MiB device copy (a known-size kernel for scaling "
                          "the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)")
     args = ap.parse_args()
+    if args.steps is None:
+        args.steps = 50 if args.workload == "cfg4" else 1000
+    if args.warmup is None:
+        args.warmup = 5 if args.workload == "cfg4" else 200
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU (the path shards over N*H with no "
               "communication; no multi-GPU figure is produced). Use --gpus 1.", file=sys.stderr)
