@@ -91,7 +91,8 @@ int run_scans(const ScanDesc *scans, int n, int64_t N, int64_t H, int64_t L, voi
             int rc = flush();
             if (rc) return rc;
             rc = generic_scan(scans[i].a, scans[i].b, scans[i].v, scans[i].out, N, H, L,
-                              scans[i].reverse, workspace, workspace_bytes, stream);
+                              scans[i].reverse, scans[i].initial, scans[i].final_, workspace,
+                              workspace_bytes, stream);
             if (rc) return rc;
             continue;
         }
@@ -156,6 +157,44 @@ int ftc_causal_dot_product(const ftc_tensor4 *queries, const ftc_tensor4 *keys,
         return zero_rows(as_operand_out(product), d.N, d.H, d.L, s);
     const ScanDesc fwd = {as_operand(queries), as_operand(keys), as_operand(values),
                           as_operand_out(product), false};
+    return run_scans(&fwd, 1, d.N, d.H, d.L, workspace, workspace_bytes, s);
+}
+
+int ftc_causal_dot_product_state(const ftc_tensor4 *queries, const ftc_tensor4 *keys,
+                                 const ftc_tensor4 *values, const ftc_tensor4 *initial_state,
+                                 const ftc_tensor4 *product, const ftc_tensor4 *final_state,
+                                 void *workspace, size_t workspace_bytes, void *stream) {
+    Dims d;
+    int rc = read_dims(queries, values, &d);
+    if (rc) return rc;
+    const int dt = queries->dtype;
+    if ((rc = check_tensor(queries, "queries", d.N, d.H, d.L, d.E, dt, dt))) return rc;
+    if ((rc = check_tensor(keys, "keys", d.N, d.H, d.L, d.E, dt, dt))) return rc;
+    if ((rc = check_tensor(values, "values", d.N, d.H, d.L, d.M, dt, dt))) return rc;
+    if ((rc = check_tensor(product, "product", d.N, d.H, d.L, d.M, FTC_F32, FTC_F32))) return rc;
+    if (initial_state && (rc = check_tensor(initial_state, "initial_state", d.N, d.H, d.E, d.M,
+                                            FTC_F32, FTC_F32)))
+        return rc;
+    if (final_state &&
+        (rc = check_tensor(final_state, "final_state", d.N, d.H, d.E, d.M, FTC_F32, FTC_F32)))
+        return rc;
+    hipStream_t s = (hipStream_t)stream;
+    auto state_ref = [](const ftc_tensor4 *t) {
+        StateRef r = {nullptr, 0, 0, 0};
+        if (t) r = StateRef{(float *)t->ptr, t->stride[0], t->stride[1], t->stride[2]};
+        return r;
+    };
+    if (d.N * d.H * d.L * d.M == 0 || d.E == 0) {
+        // no position adds to a state; a state of E x M values with nothing to go through
+        // is not handed over
+        if (final_state && d.N * d.H * d.E * d.M > 0)
+            return fail(FTC_ERR_UNSUPPORTED, "a state hand-over needs at least one position");
+        if (d.N * d.H * d.L * d.M > 0) return zero_rows(as_operand_out(product), d.N, d.H, d.L, s);
+        return FTC_OK;
+    }
+    ScanDesc fwd = {as_operand(queries), as_operand(keys), as_operand(values),
+                    as_operand_out(product), false, state_ref(initial_state),
+                    state_ref(final_state)};
     return run_scans(&fwd, 1, d.N, d.H, d.L, workspace, workspace_bytes, s);
 }
 

@@ -25,6 +25,13 @@ struct OperandOut {
     int32_t width;
 };
 
+// A D x F fp32 state per chain: element (n, h, d, f) at ptr[n*stride_n + h*stride_h +
+// d*stride_d + f].  ptr == nullptr: absent.
+struct StateRef {
+    float *ptr;
+    int64_t stride_n, stride_h, stride_d;
+};
+
 inline Operand as_operand(const ftc_tensor4 *t) {
     return Operand{t->ptr, t->stride[0], t->stride[1], t->stride[2], t->dtype, (int32_t)t->size[3]};
 }
@@ -70,8 +77,9 @@ constexpr int kGenericMaxDim = 512;
 int64_t generic_scan_workspace_bytes(int64_t N, int64_t H, int64_t L, int64_t D, int64_t F);
 
 int generic_scan(const Operand &a, const Operand &b, const Operand &v, const OperandOut &out,
-                 int64_t N, int64_t H, int64_t L, bool reverse, void *workspace,
-                 size_t workspace_bytes, hipStream_t stream);
+                 int64_t N, int64_t H, int64_t L, bool reverse, const StateRef &initial,
+                 const StateRef &final_, void *workspace, size_t workspace_bytes,
+                 hipStream_t stream);
 
 // ---------------------------------------------------------------------------
 // MFMA scan: ftc_mfma.hip + ftc_mfma_kernel.h.  One wavefront keeps a D x F state with
@@ -84,6 +92,8 @@ struct ScanDesc {
     Operand a, b, v;
     OperandOut out;
     bool reverse;
+    StateRef initial;  // optional: the state the scan starts from (read)
+    StateRef final_;   // optional: where the state after the last position goes (written)
 };
 constexpr int kMfmaMaxScans = 4;   // scans per launch
 constexpr int kMfmaMaxSlices = 16;  // column slices per scan

@@ -35,6 +35,8 @@ struct GenericArgs {
     int32_t seg_len, nseg, nslice;
     int32_t reverse;
     int32_t state_only;  // 1: write the segment's state sum; 0: write output rows
+    StateRef initial;    // optional state before the first position (single segment: read here)
+    StateRef final_;     // optional state after the last position
 };
 
 __device__ __forceinline__ int64_t row_offset(int64_t sn, int64_t sh, int64_t sl, int n, int h,
@@ -74,6 +76,15 @@ __global__ __launch_bounds__(kThreads) void generic_scan_kernel(GenericArgs p) {
         for (int i = 0; i < DREG; i++) {
             const int d = g * DREG + i;
             S[i] = (d < p.D && f_ok) ? my_state[(int64_t)d * p.F + f0 + f_local] : 0.f;
+        }
+    } else if (!p.state_only && p.initial.ptr) {
+        // single segment: start from the caller's state
+        const float *s0 = p.initial.ptr + (int64_t)n * p.initial.stride_n +
+                          (int64_t)h * p.initial.stride_h;
+#pragma unroll
+        for (int i = 0; i < DREG; i++) {
+            const int d = g * DREG + i;
+            S[i] = (d < p.D && f_ok) ? s0[(int64_t)d * p.initial.stride_d + f0 + f_local] : 0.f;
         }
     } else {
 #pragma unroll
@@ -172,19 +183,32 @@ __global__ __launch_bounds__(kThreads) void generic_scan_kernel(GenericArgs p) {
             const int d = g * DREG + i;
             if (d < p.D && f_ok) my_state[(int64_t)d * p.F + f0 + f_local] = S[i];
         }
+    } else if (p.final_.ptr && seg == (p.reverse ? 0 : p.nseg - 1)) {
+        // the segment walked last ends on the state after the whole sequence
+        float *so = p.final_.ptr + (int64_t)n * p.final_.stride_n + (int64_t)h * p.final_.stride_h;
+#pragma unroll
+        for (int i = 0; i < DREG; i++) {
+            const int d = g * DREG + i;
+            if (d < p.D && f_ok) so[(int64_t)d * p.final_.stride_d + f0 + f_local] = S[i];
+        }
     }
 }
 
 // In place: states[chain][s] <- sum of states[chain][s'] over s' < s (s' > s when reversed).
+// The running sum starts from the caller's initial state when there is one.
 __global__ __launch_bounds__(kThreads) void generic_state_scan_kernel(float *states, int nseg,
-                                                                      int64_t elems,
-                                                                      int reverse) {
+                                                                      int64_t elems, int reverse,
+                                                                      StateRef initial, int H,
+                                                                      int F) {
     const int64_t blocks_per_chain = (elems + kThreads - 1) / kThreads;
     const int64_t chain = blockIdx.x / blocks_per_chain;
     const int64_t e = (blockIdx.x % blocks_per_chain) * kThreads + threadIdx.x;
     if (e >= elems) return;
     float *base = states + chain * nseg * elems + e;
     float run = 0.f;
+    if (initial.ptr)
+        run = initial.ptr[(chain / H) * initial.stride_n + (chain % H) * initial.stride_h +
+                          (e / F) * initial.stride_d + e % F];
     for (int i = 0; i < nseg; i++) {
         const int s = reverse ? nseg - 1 - i : i;
         const float x = base[(int64_t)s * elems];
@@ -271,8 +295,9 @@ int64_t generic_scan_workspace_bytes(int64_t N, int64_t H, int64_t L, int64_t D,
 }
 
 int generic_scan(const Operand &a, const Operand &b, const Operand &v, const OperandOut &out,
-                 int64_t N, int64_t H, int64_t L, bool reverse, void *workspace,
-                 size_t workspace_bytes, hipStream_t stream) {
+                 int64_t N, int64_t H, int64_t L, bool reverse, const StateRef &initial,
+                 const StateRef &final_, void *workspace, size_t workspace_bytes,
+                 hipStream_t stream) {
     const int64_t D = a.width, F = v.width;
     if (D < 1 || F < 1 || D > kGenericMaxDim || F > kGenericMaxDim)
         return fail(FTC_ERR_UNSUPPORTED, "row widths must be in [1, %d] (got %lld and %lld)",
@@ -301,6 +326,8 @@ int generic_scan(const Operand &a, const Operand &b, const Operand &v, const Ope
     args.nseg = pl.nseg;
     args.nslice = pl.nslice;
     args.reverse = reverse ? 1 : 0;
+    args.initial = initial;
+    args.final_ = final_;
 
     if (pl.nseg > 1) {
         args.state_only = 1;
@@ -309,7 +336,8 @@ int generic_scan(const Operand &a, const Operand &b, const Operand &v, const Ope
         const int64_t scan_wgs = (elems + kThreads - 1) / kThreads * chains;
         if (scan_wgs > 0x7fffffffLL) return fail(FTC_ERR_UNSUPPORTED, "too many workgroups");
         hipLaunchKernelGGL(generic_state_scan_kernel, dim3((unsigned)scan_wgs), dim3(kThreads), 0,
-                           stream, args.states, pl.nseg, elems, args.reverse);
+                           stream, args.states, pl.nseg, elems, args.reverse, initial, (int)H,
+                           (int)F);
     }
     args.state_only = 0;
     launch_by_width(args, wgs, stream);

@@ -101,6 +101,8 @@ ScanDesc mfma_slice(const ScanDesc &scan, int col0, int width) {
     s.v.width = width;
     s.out.ptr = (char *)scan.out.ptr + (int64_t)col0 * ob;
     s.out.width = width;
+    if (s.initial.ptr) s.initial.ptr += col0;
+    if (s.final_.ptr) s.final_.ptr += col0;
     return s;
 }
 
@@ -156,6 +158,10 @@ int mfma_scan(const ScanDesc *scans, int nscans, int64_t N, int64_t H, int64_t L
         o.o_sn = sd.out.stride_n, o.o_sh = sd.out.stride_h, o.o_sl = sd.out.stride_l;
         o.rev = sd.reverse ? 1 : 0;
         o.pad = 0;
+        o.s0 = sd.initial.ptr;
+        o.s0_sn = sd.initial.stride_n, o.s0_sh = sd.initial.stride_h, o.s0_sd = sd.initial.stride_d;
+        o.s_out = sd.final_.ptr;
+        o.so_sn = sd.final_.stride_n, o.so_sh = sd.final_.stride_h, o.so_sd = sd.final_.stride_d;
         max_stride = std::max(max_stride, std::max(std::max(sd.a.stride_l, sd.b.stride_l),
                                                    std::max(sd.v.stride_l, sd.out.stride_l)));
     }

@@ -284,6 +284,11 @@ __global__ __launch_bounds__(kWave) void scan_dma_kernel(uint32_t *__restrict__ 
 #pragma unroll
             for (int ft = 0; ft < FT; ft++) S[dt][ft] = X[dt][ft];
     }
+    // every segment starts from (the caller's initial state) + (the sums of the segments
+    // before it)
+    if (op.s0)
+        add_caller_state<DT, FT>(op.s0 + (int64_t)n * op.s0_sn + (int64_t)h * op.s0_sh, op.s0_sd,
+                                 ln, g, S);
 
     // ---- pass 2: outputs.  b alternates between its two tiles, hence the chunk pairs. ----
     // row-major fragments of a chunk's a and b rows; a's tile is free afterwards
@@ -387,6 +392,10 @@ __global__ __launch_bounds__(kWave) void scan_dma_kernel(uint32_t *__restrict__ 
         output_chunk(c, b_tile0, b_tile1);
         if (c + 1 < nchunks) output_chunk(c + 1, b_tile1, b_tile0);
     }
+    // the segment walked last ends on the state after the whole sequence
+    if (op.s_out && step == p.nseg - 1)
+        store_caller_state<DT, FT>(op.s_out + (int64_t)n * op.so_sn + (int64_t)h * op.so_sh,
+                                   op.so_sd, ln, g, S);
     // nothing may still be on its way into LDS when the wavefront ends
     wait_for_stores();
 

@@ -406,7 +406,43 @@ struct ScanOperands {
     int64_t o_sn, o_sh, o_sl;
     int32_t rev;  // 0: j <= l, walk up; 1: j >= l, walk down
     int32_t pad;
+    // optional D x F fp32 states per chain (null: none): the state the scan starts from and
+    // the state after its last position; strides in elements, unit stride along F
+    const float *s0;
+    float *s_out;
+    int64_t s0_sn, s0_sh, s0_sd;
+    int64_t so_sn, so_sh, so_sd;
 };
+
+// The caller's state in accumulator layout: register r of tile (dt, ft) in lane (ln, g) is
+// element (d = 32*dt + 8*(r/4) + 4*g + r%4, f = 32*ft + ln), so the 32 lanes of a half-wave
+// touch 128 consecutive bytes.
+template <int DT, int FT>
+__device__ __forceinline__ void add_caller_state(const float *base, int64_t row_stride, int ln,
+                                                 int g, f32x16 (&S)[DT][FT]) {
+#pragma unroll
+    for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+        for (int ft = 0; ft < FT; ft++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int d = 32 * dt + 8 * (r / 4) + 4 * g + (r % 4);
+                S[dt][ft][r] += base[(int64_t)d * row_stride + 32 * ft + ln];
+            }
+}
+template <int DT, int FT>
+__device__ __forceinline__ void store_caller_state(float *base, int64_t row_stride, int ln, int g,
+                                                   const f32x16 (&S)[DT][FT]) {
+#pragma unroll
+    for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+        for (int ft = 0; ft < FT; ft++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int d = 32 * dt + 8 * (r / 4) + 4 * g + (r % 4);
+                base[(int64_t)d * row_stride + 32 * ft + ln] = S[dt][ft][r];
+            }
+}
 constexpr int kMaxScans = kMfmaMaxScans;
 
 struct ScanArgs {
@@ -732,6 +768,11 @@ __global__ __launch_bounds__(kWave) void scan_mfma_kernel(uint32_t *__restrict__
         fetch_vt(chunk_row0(0));
         fetch_bt(chunk_row0(0));
     }
+    // every segment starts from (the caller's initial state) + (the sums of the segments
+    // before it)
+    if (op.s0)
+        add_caller_state<DT, FT>(op.s0 + (int64_t)n * op.s0_sn + (int64_t)h * op.s0_sh, op.s0_sd,
+                                 ln, g, S);
 
     // ---- pass 2: outputs ----
     for (int c = 0; c < nchunks; c++) {
@@ -828,6 +869,10 @@ __global__ __launch_bounds__(kWave) void scan_mfma_kernel(uint32_t *__restrict__
         update_state(bt_frag, v_frag);
     }
 
+    // the segment walked last ends on the state after the whole sequence
+    if (op.s_out && step == p.nseg - 1)
+        store_caller_state<DT, FT>(op.s_out + (int64_t)n * op.so_sn + (int64_t)h * op.so_sh,
+                                   op.so_sd, ln, g, S);
     release_control_block(p, hdr, flags, lane);
 }
 

@@ -88,6 +88,45 @@ def causal_dot_product_hip(queries, keys, values, product):
     _native.check(rc, "ftc_causal_dot_product")
 
 
+def causal_dot_product_with_state(queries, keys, values, initial_state=None,
+                                  return_state=True):
+    """The product of a piece of a sequence, started from ``initial_state`` (``(N, H, E, M)``
+    float32, or ``None`` for zeros) and returning ``(product, final_state)``:
+
+        S_l = initial_state + sum_{j<=l} keys_j values_j^T ;  product_l = S_l^T queries_l
+
+    ``final_state`` is the ``S_i`` that the reference's step-wise attention keeps
+    (``recurrent/attention/self_attention/linear_attention.py:63-90``), so a prompt processed
+    here can be continued there, or by another call on the next piece.  Forward only (no
+    autograd); enqueued on the current stream."""
+    lib = _native.load()
+    q, k, v = (_prepare(t, n) for t, n in
+               ((queries, "queries"), (keys, "keys"), (values, "values")))
+    N, H, L, E = q.shape
+    M = v.shape[3]
+    s0 = None
+    if initial_state is not None:
+        s0 = _prepare(initial_state, "initial_state")
+        if s0.dtype != torch.float32 or tuple(s0.shape) != (N, H, E, M):
+            raise RuntimeError("causal_dot_product_with_state: initial_state must be a float32 "
+                               "tensor of shape (N, H, E, M)")
+    out = torch.empty((N, H, L, M), dtype=torch.float32, device=q.device)
+    s1 = torch.empty((N, H, E, M), dtype=torch.float32, device=q.device) if return_state else None
+    with torch.cuda.device(q.device):
+        nbytes = _native.check(
+            lib.ftc_causal_dot_product_workspace_bytes(N, H, L, E, M, _native.dtype_code(q.dtype)),
+            "ftc_causal_dot_product_workspace_bytes")
+        ws, nbytes = _workspace(nbytes, q.device)
+        dq, dk, dv, do = (_native.describe(t) for t in (q, k, v, out))
+        d0 = _native.describe(s0) if s0 is not None else None
+        d1 = _native.describe(s1) if s1 is not None else None
+        rc = lib.ftc_causal_dot_product_state(dq, dk, dv, d0, do, d1,
+                                              ws.data_ptr() if ws is not None else None, nbytes,
+                                              torch.cuda.current_stream().cuda_stream)
+    _native.check(rc, "ftc_causal_dot_product_state")
+    return out, s1
+
+
 def causal_dot_backward_hip(queries, keys, values, grad_out, grad_queries, grad_keys,
                             grad_values):
     """In-place backward; replaces the reference's native ``causal_dot_backward``

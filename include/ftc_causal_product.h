@@ -85,6 +85,24 @@ int ftc_causal_dot_product(const ftc_tensor4 *queries, const ftc_tensor4 *keys,
                            const ftc_tensor4 *values, const ftc_tensor4 *product,
                            void *workspace, size_t workspace_bytes, void *stream);
 
+/*
+ * The product with the running state handed in and out, for processing a sequence in
+ * pieces and for passing a prompt's state on to step-wise decoding:
+ *   S_l = initial_state + sum_{j<=l} keys[n,h,j,:] values[n,h,j,:]^T        (E x M per chain)
+ *   product[n,h,l,:] = S_l^T queries[n,h,l,:] ;  final_state = S_{L-1}
+ * The state is the S_i of the reference's step-wise module
+ * (recurrent/attention/self_attention/linear_attention.py:63-90: "Si = Si + einsum(K, V)",
+ * then the read-out), which the reference can only reach one position at a time; its
+ * batched native op (causal_product_cpu.cpp:82-124) starts from zero and drops the state.
+ * initial_state, final_state: (N,H,E,M), FTC_F32, unit stride along M; either may be NULL
+ * (start from zero / do not return the state); they must not overlap.  Needs L >= 1 when
+ * final_state is given.  Workspace: ftc_causal_dot_product_workspace_bytes.
+ */
+int ftc_causal_dot_product_state(const ftc_tensor4 *queries, const ftc_tensor4 *keys,
+                                 const ftc_tensor4 *values, const ftc_tensor4 *initial_state,
+                                 const ftc_tensor4 *product, const ftc_tensor4 *final_state,
+                                 void *workspace, size_t workspace_bytes, void *stream);
+
 /* Scratch bytes ftc_causal_dot_backward needs (>= 0), or a negative ftc_status. */
 int64_t ftc_causal_dot_backward_workspace_bytes(int64_t N, int64_t H, int64_t L, int64_t E,
                                                 int64_t M, int32_t dtype);

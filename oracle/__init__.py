@@ -13,6 +13,8 @@ Contents
 * ``dense_forward`` / ``dense_backward``: the closed forms ``tril(Q K^T) V`` and
   their gradients, i.e. what the reference's own tests compare against
   (``tests/causal_product/test_causal_product_cpu.py:45-47,65-70``).
+* ``forward_with_state``: the forward with the running state handed in and out
+  (the ``Si`` of the reference's step-wise module).
 * ``recurrent_forward``: the step-wise einsum form of
   ``fast_transformers/recurrent/attention/self_attention/linear_attention.py:79-88``
   without the feature map and normaliser.
@@ -55,6 +57,10 @@ def _load():
             f = getattr(_lib, "oracle_causal_dot_product_" + sfx)
             f.restype = ctypes.c_int
             f.argtypes = [ctypes.c_void_p, i64p] * 4 + [ctypes.c_int] * 5
+            st = getattr(_lib, "oracle_causal_dot_product_state_" + sfx)
+            st.restype = ctypes.c_int
+            st.argtypes = ([ctypes.c_void_p, i64p] * 3 + [ctypes.c_void_p] +
+                           [ctypes.c_void_p, i64p] + [ctypes.c_void_p] + [ctypes.c_int] * 5)
             b = getattr(_lib, "oracle_causal_dot_backward_" + sfx)
             b.restype = ctypes.c_int
             b.argtypes = [ctypes.c_void_p, i64p] * 7 + [ctypes.c_int] * 5
@@ -109,6 +115,30 @@ def causal_dot_backward(queries, keys, values, grad_out, grad_queries, grad_keys
     rc = getattr(lib, "oracle_causal_dot_backward_" + sfx)(*args, N, H, L, E, M)
     if rc != 0:
         raise RuntimeError("oracle backward failed (%d)" % rc)
+
+
+def forward_with_state(Q, K, V, initial_state=None):
+    """(product, final_state) with the running state handed in and out; the state is the
+    ``Si`` of recurrent/attention/self_attention/linear_attention.py:63-66,79-80."""
+    lib = _load()
+    sfx = _suffix(Q, K, V)
+    N, H, L, E = Q.shape
+    M = V.shape[3]
+    out = torch.empty(N, H, L, M, dtype=Q.dtype)
+    s1 = torch.empty(N, H, E, M, dtype=Q.dtype)
+    s0p = None
+    if initial_state is not None:
+        s0 = initial_state.to(Q.dtype).contiguous()
+        assert s0.shape == (N, H, E, M)
+        s0p = ctypes.c_void_p(s0.data_ptr())
+    args = []
+    for t in (Q, K, V):
+        args.extend(_arg(t))
+    rc = getattr(lib, "oracle_causal_dot_product_state_" + sfx)(
+        *args, s0p, *_arg(out), ctypes.c_void_p(s1.data_ptr()), N, H, L, E, M)
+    if rc != 0:
+        raise RuntimeError("oracle stateful forward failed (%d)" % rc)
+    return out, s1
 
 
 def forward(Q, K, V):

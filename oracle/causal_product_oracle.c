@@ -121,6 +121,48 @@ int FN(oracle_causal_dot_product)(
     return failed ? -1 : 0;
 }
 
+/*
+ * The forward with the running state handed in and out: S starts from s0 (contiguous
+ * (N,H,E,M), or NULL for zeros) and is copied to s_out (or NULL) after the last position.
+ * The state and its update are the Si of the reference's step-wise module
+ * (fast_transformers/recurrent/attention/self_attention/linear_attention.py:63-66,79-80:
+ * "Si = Si + einsum('nhd,nhm->nhdm', K, value)", read out at :86 without the normaliser);
+ * the loop is the forward's above.  Pinned by tests/test_oracle.py: two pieces with the
+ * state handed over equal one pass of the (pinned) forward, the final state equals the
+ * dense K^T V, and a non-zero s0 adds Q s0 to every row.
+ */
+int FN(oracle_causal_dot_product_state)(
+    const REAL *q, const int64_t *q_stride, const REAL *k, const int64_t *k_stride,
+    const REAL *v, const int64_t *v_stride, const REAL *s0, REAL *out, const int64_t *o_stride,
+    REAL *s_out, int N, int H, int L, int E, int M) {
+    const view4 Q = {(REAL *)q, q_stride[0], q_stride[1], q_stride[2], q_stride[3]};
+    const view4 K = {(REAL *)k, k_stride[0], k_stride[1], k_stride[2], k_stride[3]};
+    const view4 V = {(REAL *)v, v_stride[0], v_stride[1], v_stride[2], v_stride[3]};
+    const view4 O = {out, o_stride[0], o_stride[1], o_stride[2], o_stride[3]};
+    int failed = 0;
+#pragma omp parallel for collapse(2)
+    for (int n = 0; n < N; n++) {
+        for (int h = 0; h < H; h++) {
+            REAL *S = (REAL *)calloc((size_t)E * M + M, sizeof(REAL));
+            if (!S) {
+#pragma omp atomic write
+                failed = 1;
+                continue;
+            }
+            REAL *tmp = S + (size_t)E * M;
+            const size_t chain = ((size_t)n * H + h) * E * M;
+            if (s0) memcpy(S, s0 + chain, (size_t)E * M * sizeof(REAL));
+            for (int l = 0; l < L; l++) {
+                rank1_add(row(&K, n, h, l), K.sx, row(&V, n, h, l), V.sx, S, E, M);
+                vec_mat(row(&Q, n, h, l), Q.sx, S, row(&O, n, h, l), O.sx, E, M, tmp);
+            }
+            if (s_out) memcpy(s_out + chain, S, (size_t)E * M * sizeof(REAL));
+            free(S);
+        }
+    }
+    return failed ? -1 : 0;
+}
+
 /* g: (N,H,L,M); dq,dk: (N,H,L,E); dv: (N,H,L,M). */
 int FN(oracle_causal_dot_backward)(
     const REAL *q, const int64_t *q_stride, const REAL *k, const int64_t *k_stride,

@@ -266,6 +266,101 @@ def test_bf16_inputs_fp32_accumulate(cp, name):
     assert scale_error(Qg.grad.float().cpu(), refs[0]) <= 2e-2
 
 
+STATE_SHAPES = {
+    # (N, H, L, E, M, seed, dtype): LDS-fed kernel with several segments per chain
+    "e64_m64": (2, 4, 1000, 64, 64, 51, torch.float32),
+    # one segment per chain (no exchange)
+    "many_chains": (40, 32, 64, 64, 64, 52, torch.float32),
+    "e32_m128": (2, 3, 700, 32, 128, 53, torch.float32),
+    # register-fed kernel, column slices
+    "e128_m128": (1, 3, 500, 128, 128, 54, torch.float32),
+    "e96_m64": (2, 2, 300, 96, 64, 55, torch.float32),
+    # generic path, several segments and a single one
+    "e25_m70": (2, 4, 600, 25, 70, 56, torch.float32),
+    "e10_m3": (3, 2, 40, 10, 3, 57, torch.float32),
+    # bf16 rows
+    "bf16_e64_m64": (2, 3, 800, 64, 64, 58, torch.bfloat16),
+}
+
+
+@pytest.mark.parametrize("name", sorted(STATE_SHAPES))
+def test_state_handed_in_and_out(cp, name):
+    """ftc_causal_dot_product_state against the CPU checker: from zero, from a given state,
+    and a sequence cut in two with the state passed on."""
+    N, H, L, E, M, seed, dtype = STATE_SHAPES[name]
+    print("state", name, (N, H, L, E, M), dtype, flush=True)
+    Q, K, V, _ = oracle.make_inputs(N, H, L, E, M, seed)
+    Q, K, V = (t.to(dtype) for t in (Q, K, V))
+    Qf, Kf, Vf = (t.float() for t in (Q, K, V))
+    S0 = torch.randn(N, H, E, M, generator=torch.Generator().manual_seed(seed + 100)) * 3
+    tol = 1e-4
+
+    def close(got, want, what):
+        err = (got.cpu().double() - want.double()).abs().amax(dim=(-2, -1)) / \
+            want.double().abs().amax(dim=(-2, -1)).clamp_min(1e-30)
+        print("    %s: max scale error %.3e" % (what, err.max().item()), flush=True)
+        assert torch.isfinite(got).all(), what
+        assert err.max().item() <= tol, what
+
+    # from zero: the plain product, and the state after the last position
+    want, want_state = oracle.forward_with_state(Qf, Kf, Vf)
+    out, state = cp.causal_dot_product_with_state(Q.cuda(), K.cuda(), V.cuda())
+    close(out, want, "product from zero")
+    close(state, want_state, "final state from zero")
+    plain = torch.empty_like(out)
+    cp.causal_dot_product_hip(Q.cuda(), K.cuda(), V.cuda(), plain)
+    assert torch.equal(out, plain), "a zero start must not change the product"
+
+    # from a given state
+    want, want_state = oracle.forward_with_state(Qf, Kf, Vf, S0)
+    out, state = cp.causal_dot_product_with_state(Q.cuda(), K.cuda(), V.cuda(), S0.cuda())
+    close(out, want, "product from S0")
+    close(state, want_state, "final state from S0")
+    whole, whole_state = out, state
+
+    # cut in two, odd cut, state passed on; no state asked for at the end of a third call
+    cut = max(1, (L * 5) // 11)
+    o1, s1 = cp.causal_dot_product_with_state(Q[:, :, :cut].cuda(), K[:, :, :cut].cuda(),
+                                              V[:, :, :cut].cuda(), S0.cuda())
+    o2, s2 = cp.causal_dot_product_with_state(Q[:, :, cut:].cuda(), K[:, :, cut:].cuda(),
+                                              V[:, :, cut:].cuda(), s1)
+    close(torch.cat([o1, o2], dim=2), want, "two pieces")
+    close(s2, want_state, "state after two pieces")
+    o3, none = cp.causal_dot_product_with_state(Q[:, :, cut:].cuda(), K[:, :, cut:].cuda(),
+                                                V[:, :, cut:].cuda(), s1, return_state=False)
+    assert none is None and torch.equal(o3, o2)
+    del whole, whole_state
+
+
+def test_state_continues_into_stepwise_decoding(cp):
+    """Prefill on the GPU, then the reference's step-wise update and read-out
+    (recurrent/attention/self_attention/linear_attention.py:79-88) on the returned state:
+    the rows must be the ones a single batched pass gives."""
+    N, H, L, E, M = 2, 4, 400, 64, 64
+    Q, K, V, _ = oracle.make_inputs(N, H, L, E, M, seed=61)
+    cut = 389
+    _, S = cp.causal_dot_product_with_state(Q[:, :, :cut].cuda(), K[:, :, :cut].cuda(),
+                                            V[:, :, :cut].cuda())
+    S = S.cpu().double()
+    whole = oracle.forward(Q.double(), K.double(), V.double())
+    for l in range(cut, L):
+        S = S + torch.einsum("nhd,nhm->nhdm", K[:, :, l].double(), V[:, :, l].double())
+        row = torch.einsum("nhd,nhdm->nhm", Q[:, :, l].double(), S)
+        err = (row - whole[:, :, l]).abs().max() / whole[:, :, l].abs().max()
+        assert err < 1e-5, (l, err)
+
+
+def test_state_errors(cp):
+    Q, K, V, _ = (t.cuda() for t in oracle.make_inputs(1, 2, 40, 16, 16, seed=62))
+    with pytest.raises(RuntimeError):
+        cp.causal_dot_product_with_state(Q, K, V, torch.zeros(1, 2, 16, 8, device="cuda"))
+    with pytest.raises(RuntimeError):
+        cp.causal_dot_product_with_state(Q, K, V, torch.zeros(1, 2, 16, 16, device="cuda",
+                                                             dtype=torch.bfloat16))
+    with pytest.raises(RuntimeError):  # nothing to hand over without a position
+        cp.causal_dot_product_with_state(Q[:, :, :0], K[:, :, :0], V[:, :, :0])
+
+
 def test_graph_replay_matches_direct_launches(cp):
     """The entry points only enqueue kernels (the control block is cleared by the kernels
     themselves), so a forward + backward pair can be captured in a HIP graph.  Every replay,

@@ -228,3 +228,50 @@ def test_outputs_need_not_be_zeroed():
     out = torch.full((1, 1, 10, 4), 7.0)
     oracle.causal_dot_product(Q, K, V, out)
     assert torch.equal(out, oracle.forward(Q, K, V))
+
+
+# ---------------------------------------------------------------------------
+# the forward with the running state handed in and out
+# ---------------------------------------------------------------------------
+def test_stateful_forward_from_zero_is_the_forward_and_ends_on_kt_v():
+    Q, K, V, _ = oracle.make_inputs(2, 3, 70, 9, 6, seed=41)
+    out, state = oracle.forward_with_state(Q, K, V)
+    assert torch.equal(out, oracle.forward(Q, K, V))
+    exact = torch.einsum("nhle,nhlm->nhem", K.double(), V.double())
+    # V has zero mean, so single entries cancel; the yardstick is the size of the state
+    assert (state.double() - exact).abs().max() / exact.abs().max() < 1e-6
+
+
+def test_stateful_forward_hands_the_state_over_between_pieces():
+    """Two pieces with the state passed on are one pass: the running state after position
+    l is the same sequence of operations either way, so the match is exact."""
+    Q, K, V, _ = oracle.make_inputs(2, 2, 90, 7, 5, seed=42)
+    whole, end = oracle.forward_with_state(Q, K, V)
+    for cut in (1, 33, 89):
+        o1, s1 = oracle.forward_with_state(Q[:, :, :cut], K[:, :, :cut], V[:, :, :cut])
+        o2, s2 = oracle.forward_with_state(Q[:, :, cut:], K[:, :, cut:], V[:, :, cut:], s1)
+        assert torch.equal(torch.cat([o1, o2], dim=2), whole)
+        assert torch.equal(s2, end)
+
+
+def test_stateful_forward_initial_state_adds_q_times_state():
+    Q, K, V, _ = oracle.make_inputs(1, 3, 40, 6, 8, seed=43, dtype=torch.float64)
+    s0 = torch.randn(1, 3, 6, 8, dtype=torch.float64, generator=torch.Generator().manual_seed(7))
+    out, end = oracle.forward_with_state(Q, K, V, s0)
+    want = oracle.dense_forward(Q, K, V) + torch.einsum("nhle,nhem->nhlm", Q, s0)
+    assert max_relative_error(out, want) < 1e-12
+    assert max_relative_error(end, s0 + torch.einsum("nhle,nhlm->nhem", K, V)) < 1e-12
+
+
+def test_stateful_forward_continues_into_the_stepwise_form():
+    """The final state is the Si of the reference's step-wise module
+    (recurrent/attention/self_attention/linear_attention.py:79-88): stepping on from it with
+    the einsum form gives the rows the batched pass gives."""
+    Q, K, V, _ = oracle.make_inputs(2, 2, 30, 5, 4, seed=44, dtype=torch.float64)
+    cut = 21
+    _, S = oracle.forward_with_state(Q[:, :, :cut], K[:, :, :cut], V[:, :, :cut])
+    whole = oracle.forward(Q, K, V)
+    for l in range(cut, 30):
+        S = S + torch.einsum("nhd,nhm->nhdm", K[:, :, l], V[:, :, l])
+        row = torch.einsum("nhd,nhdm->nhm", Q[:, :, l], S)
+        assert max_relative_error(row, whole[:, :, l]) < 1e-12
