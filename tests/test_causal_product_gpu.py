@@ -266,6 +266,54 @@ def test_bf16_inputs_fp32_accumulate(cp, name):
     assert scale_error(Qg.grad.float().cpu(), refs[0]) <= 2e-2
 
 
+def _random_case(rng):
+    widths = [32, 64, 96, 128, 256, 17, 40, 100]
+    E = widths[int(rng.integers(len(widths)))]
+    M = widths[int(rng.integers(len(widths)))]
+    N, H = int(rng.integers(1, 4)), int(rng.integers(1, 6))
+    L = int(rng.choice([1, 31, 32, 33, 95, 200, 777, 1500, 2600]))
+    if E * M * N * H * L > 6e8:  # keep the CPU checker quick
+        L = min(L, 200)
+    layout = str(rng.choice(["nhle", "nlhe", "padded"]))
+    return N, H, L, E, M, layout
+
+
+def _lay_out(t, layout):
+    """The same values in a tensor with other strides (device side)."""
+    t = t.cuda()
+    N, H, L, X = t.shape
+    if layout == "nlhe":  # the projections' layout, seen as (N, H, L, X)
+        return t.permute(0, 2, 1, 3).contiguous().permute(0, 2, 1, 3)
+    if layout == "padded":  # rows with a gap behind them; keeps 16-byte alignment
+        wide = torch.zeros(N, H, L, X + 8, device="cuda", dtype=t.dtype)
+        wide[..., :X] = t
+        return wide[..., :X]
+    return t
+
+
+def test_random_shapes_and_layouts_against_cpu_checker(cp):
+    """Forty seeded draws over widths (MFMA shapes, sliced shapes, odd shapes), lengths around
+    the chunk size and beyond, batch sizes and memory layouts; forward and backward."""
+    rng = np.random.default_rng(2024)
+    for case in range(40):
+        N, H, L, E, M, layout = _random_case(rng)
+        print("random case", case, (N, H, L, E, M), layout, flush=True)
+        Q, K, V, G = oracle.make_inputs(N, H, L, E, M, seed=1000 + case)
+        want = oracle.forward(Q, K, V)
+        refs = oracle.backward(Q, K, V, G)
+        Qd, Kd, Vd, Gd = (_lay_out(t, layout) for t in (Q, K, V, G))
+        out = _lay_out(torch.full((N, H, L, M), float("nan")), layout)
+        cp.causal_dot_product_hip(Qd, Kd, Vd, out)
+        grads = [_lay_out(torch.full(sh, float("nan")), layout)
+                 for sh in ((N, H, L, E), (N, H, L, E), (N, H, L, M))]
+        cp.causal_dot_backward_hip(Qd, Kd, Vd, Gd, *grads)
+        torch.cuda.synchronize()
+        for key, got, ref in zip(("product", "dQ", "dK", "dV"), [out] + grads, [want] + list(refs)):
+            got = got.cpu()
+            assert torch.isfinite(got).all(), (case, key)
+            assert scale_error(got, ref) <= 1e-4, (case, key, scale_error(got, ref))
+
+
 STATE_SHAPES = {
     # (N, H, L, E, M, seed, dtype): LDS-fed kernel with several segments per chain
     "e64_m64": (2, 4, 1000, 64, 64, 51, torch.float32),
