@@ -6,10 +6,13 @@ key_lengths)`` over ``(N, L, H, E)`` tensors, same equations (feature map ``elu(
 ``feature_maps/base.py:71-73``; key-length masking ``:83``; normaliser
 ``Z = 1 / (q . cumsum(k) + eps)`` ``:95``; result ``V' * Z`` ``:104``).
 
-One difference in mechanics: the reference makes four ``permute().contiguous()`` copies
-around the native call (``:19-24``).  The kernels here take any N/H/L strides, so the
+Two differences in mechanics.  The reference makes four ``permute().contiguous()`` copies
+around the native call (``:19-24``); the kernels here take any N/H/L strides, so the
 ``(N, L, H, X)`` tensors are handed over as permuted views and the product is written
-straight into ``(N, L, H, M)`` storage.
+straight into ``(N, L, H, M)`` storage.  And the normaliser's ``q_l . sum_{j<=l} k_j`` is
+the same causal product with a column of ones for values, so it is a second call of the
+operator instead of a cumulative sum over L followed by a batched dot product (which on
+this stack cost ten and fifty times the operator itself).
 """
 import torch
 from torch.nn import Module
@@ -44,6 +47,22 @@ class _CausalLinearNLH(torch.autograd.Function):
                                 gQ.permute(0, 2, 1, 3), gK.permute(0, 2, 1, 3),
                                 gV.permute(0, 2, 1, 3))
         return gQ, gK, gV
+
+
+_ONES_WIDTH = 32  # the narrowest value width the matrix-core kernels take
+_ones_rows = {}
+
+
+def _ones_column(N, L, H, device):
+    """An (N, L, H, 32) view whose column 0 is one and whose other columns are zero, backed
+    by a single (L, 32) buffer (zero strides over N and H)."""
+    key = (device, L)
+    rows = _ones_rows.get(key)
+    if rows is None:
+        rows = torch.zeros(L, _ONES_WIDTH, device=device, dtype=torch.float32)
+        rows[:, 0] = 1
+        _ones_rows[key] = rows
+    return rows[None, :, None, :].expand(N, L, H, _ONES_WIDTH)
 
 
 def causal_linear(Q, K, V):
@@ -86,6 +105,9 @@ class CausalLinearAttention(Module):
             raise RuntimeError("CausalLinearAttention only supports full lower triangular masks")
         K = K * key_lengths.float_matrix[:, :, None, None]
         K, values = self._make_sizes_compatible(Q, K, values)
-        Z = 1 / (torch.einsum("nlhi,nlhi->nlh", Q, K.cumsum(1)) + self.eps)
+        # q_l . cumsum(k)_l  ==  sum_{j<=l} (q_l . k_j) * 1
+        N, L, H, _ = Q.shape
+        denominator = causal_linear(Q, K, _ones_column(N, L, H, Q.device))[..., 0]
+        Z = 1 / (denominator + self.eps)
         V = causal_linear(Q, K, values)
         return V * Z[:, :, :, None]

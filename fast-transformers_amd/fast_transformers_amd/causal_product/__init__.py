@@ -30,7 +30,9 @@ def _prepare(t, name):
                            % (name, t.device))
     if t.shape[3] > 1 and t.stride(3) != 1:
         return t.contiguous()
-    if any(s == 0 and n > 1 for s, n in zip(t.stride()[:3], t.shape[:3])):
+    # rows that overlap (an expanded L dimension) would take the slow general path; zero
+    # strides over N or H (one sequence shared by chains) are read as they are
+    if t.shape[2] > 1 and t.stride(2) < t.shape[3]:
         return t.contiguous()
     return t
 
