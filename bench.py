@@ -34,7 +34,7 @@ MFMA_FP32_PEAK_TFLOPS = 157.3   # MI355X dense fp32 matrix, published
 # rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script, scaled by what the same
 # counters read for the 256 MiB copy of --calibrate-copy; the runs are summarised in
 # profiles/scan_dma_kernel_<workload>_traffic.md.  None = not measured for that workload.
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {"cfg2": 233148585, "cfg3": 3190003296}
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {"cfg2": 234721354, "cfg3": 3186430251}
 
 WORKLOADS = {
     # name: (N, H, L, E, M, dtype, seed)
