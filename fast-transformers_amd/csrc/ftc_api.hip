@@ -221,13 +221,19 @@ int ftc_causal_dot_backward(const ftc_tensor4 *queries, const ftc_tensor4 *keys,
     if ((rc = check_tensor(keys, "keys", d.N, d.H, d.L, d.E, dt, dt))) return rc;
     if ((rc = check_tensor(values, "values", d.N, d.H, d.L, d.M, dt, dt))) return rc;
     if ((rc = check_tensor(grad_out, "grad_out", d.N, d.H, d.L, d.M, FTC_F32, FTC_F32))) return rc;
-    if ((rc = check_tensor(grad_queries, "grad_queries", d.N, d.H, d.L, d.E, dt, dt))) return rc;
-    if ((rc = check_tensor(grad_keys, "grad_keys", d.N, d.H, d.L, d.E, dt, dt))) return rc;
-    if ((rc = check_tensor(grad_values, "grad_values", d.N, d.H, d.L, d.M, dt, dt))) return rc;
+    // a gradient that is not wanted may be passed as NULL
+    if (grad_queries &&
+        (rc = check_tensor(grad_queries, "grad_queries", d.N, d.H, d.L, d.E, dt, dt)))
+        return rc;
+    if (grad_keys && (rc = check_tensor(grad_keys, "grad_keys", d.N, d.H, d.L, d.E, dt, dt)))
+        return rc;
+    if (grad_values && (rc = check_tensor(grad_values, "grad_values", d.N, d.H, d.L, d.M, dt, dt)))
+        return rc;
     if (d.N * d.H * d.L == 0 || d.E == 0 || d.M == 0) {
         // A zero row width: whichever gradient is non-empty is a sum over an empty index set.
         const ftc_tensor4 *outs[3] = {grad_queries, grad_keys, grad_values};
         for (const ftc_tensor4 *t : outs) {
+            if (!t) continue;
             if (t->size[0] * t->size[1] * t->size[2] * t->size[3] == 0) continue;
             if ((rc = zero_rows(as_operand_out(t), d.N, d.H, d.L, (hipStream_t)stream))) return rc;
         }
@@ -236,12 +242,15 @@ int ftc_causal_dot_backward(const ftc_tensor4 *queries, const ftc_tensor4 *keys,
     hipStream_t s = (hipStream_t)stream;
     const Operand Q = as_operand(queries), K = as_operand(keys), V = as_operand(values),
                   G = as_operand(grad_out);
-    const ScanDesc scans[3] = {
-        {G, V, K, as_operand_out(grad_queries), false},  // dQ: state M x E, walks up
-        {V, G, Q, as_operand_out(grad_keys), true},      // dK: state M x E, walks down
-        {K, Q, G, as_operand_out(grad_values), true},    // dV: state E x M, walks down
-    };
-    return run_scans(scans, 3, d.N, d.H, d.L, workspace, workspace_bytes, s);
+    ScanDesc scans[3];
+    int n = 0;
+    if (grad_queries)  // dQ: state M x E, walks up
+        scans[n++] = ScanDesc{G, V, K, as_operand_out(grad_queries), false};
+    if (grad_keys)  // dK: state M x E, walks down
+        scans[n++] = ScanDesc{V, G, Q, as_operand_out(grad_keys), true};
+    if (grad_values)  // dV: state E x M, walks down
+        scans[n++] = ScanDesc{K, Q, G, as_operand_out(grad_values), true};
+    return run_scans(scans, n, d.N, d.H, d.L, workspace, workspace_bytes, s);
 }
 
 }  // extern "C"

@@ -40,12 +40,14 @@ class _CausalLinearNLH(torch.autograd.Function):
     @staticmethod
     def backward(ctx, grad_out):
         Q, K, V = ctx.saved_tensors
-        gQ, gK, gV = (torch.empty(t.shape, device=t.device, dtype=t.dtype) for t in (Q, K, V))
+        # gradients nobody asked for (the normaliser's column of ones) are not computed
+        gQ, gK, gV = (torch.empty(t.shape, device=t.device, dtype=t.dtype) if need else None
+                      for t, need in zip((Q, K, V), ctx.needs_input_grad))
         G = grad_out if grad_out.dtype == torch.float32 else grad_out.float()
         causal_dot_backward_hip(Q.permute(0, 2, 1, 3), K.permute(0, 2, 1, 3),
                                 V.permute(0, 2, 1, 3), G.contiguous().permute(0, 2, 1, 3),
-                                gQ.permute(0, 2, 1, 3), gK.permute(0, 2, 1, 3),
-                                gV.permute(0, 2, 1, 3))
+                                *(t.permute(0, 2, 1, 3) if t is not None else None
+                                  for t in (gQ, gK, gV)))
         return gQ, gK, gV
 
 

@@ -132,14 +132,15 @@ def causal_dot_product_with_state(queries, keys, values, initial_state=None,
 def causal_dot_backward_hip(queries, keys, values, grad_out, grad_queries, grad_keys,
                             grad_values):
     """In-place backward; replaces the reference's native ``causal_dot_backward``
-    (``causal_product_cuda.cu:1438-1467``).  Enqueued on the current stream."""
+    (``causal_product_cuda.cu:1438-1467``).  A gradient passed as ``None`` is skipped.
+    Enqueued on the current stream."""
     lib = _native.load()
     q, k, v, g = (_prepare(t, n) for t, n in
                   ((queries, "queries"), (keys, "keys"), (values, "values"),
                    (grad_out, "grad_out")))
     if g.dtype != torch.float32:
         g = g.float()
-    gq, gk, gv = (_check_out(t, n) for t, n in
+    gq, gk, gv = (_check_out(t, n) if t is not None else None for t, n in
                   ((grad_queries, "grad_queries"), (grad_keys, "grad_keys"),
                    (grad_values, "grad_values")))
     N, H, L, E = q.shape
@@ -150,7 +151,7 @@ def causal_dot_backward_hip(queries, keys, values, grad_out, grad_queries, grad_
                                                         _native.dtype_code(q.dtype)),
             "ftc_causal_dot_backward_workspace_bytes")
         ws, nbytes = _workspace(nbytes, q.device)
-        descs = [_native.describe(t) for t in (q, k, v, g, gq, gk, gv)]
+        descs = [_native.describe(t) if t is not None else None for t in (q, k, v, g, gq, gk, gv)]
         rc = lib.ftc_causal_dot_backward(*descs, ws.data_ptr() if ws is not None else None,
                                          nbytes, torch.cuda.current_stream().cuda_stream)
     _native.check(rc, "ftc_causal_dot_backward")

@@ -112,7 +112,8 @@ int64_t ftc_causal_dot_backward_workspace_bytes(int64_t N, int64_t H, int64_t L,
  * grad_out = d loss / d product.  Replaces causal_dot_backward(queries, keys,
  * values, grad_out, grad_queries, grad_keys, grad_values)
  * (causal_product_cpu.cpp:133-209, causal_product_cuda.cu:1438-1467).
- * All three gradients are always computed, as in the reference.
+ * The reference always computes all three gradients; here a gradient that is not wanted
+ * may be passed as NULL and is then skipped.
  */
 int ftc_causal_dot_backward(const ftc_tensor4 *queries, const ftc_tensor4 *keys,
                             const ftc_tensor4 *values, const ftc_tensor4 *grad_out,
