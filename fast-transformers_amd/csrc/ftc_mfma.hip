@@ -18,7 +18,7 @@ MfmaPlan make_plan(int64_t N, int64_t H, int64_t L, int64_t D, int64_t F, int ns
     MfmaPlan pl;
     const int64_t chains = std::max<int64_t>(1, N * H);
     const int64_t total_chunks = (L + kChunk - 1) / kChunk;
-    // One wavefront per SIMD is resident (LDS footprint): 1024 slots.  Pick the segment
+    // One wavefront per SIMD is resident (register footprint): 1024 slots.  Pick the segment
     // length (in chunks) that minimises an estimate of the makespan: rounds of resident
     // wavefronts times the work of one wavefront (pass 1 costs about half of pass 2, the
     // exchange of segment sums about three chunks).
