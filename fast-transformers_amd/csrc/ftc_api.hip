@@ -12,8 +12,14 @@
 #include <stdio.h>
 
 #include <algorithm>
+#include <mutex>
 
 #include "ftc_common.h"
+
+// Scratch memory of ftc_causal_dot_product_static: one array per GPU, part of the loaded
+// code object (zero when it is loaded).  Host code never uses this name as an address; it
+// asks the runtime for the array's device address once per device (scratch_of_device).
+static __device__ __align__(256) unsigned char scratch[FTC_STATIC_SCRATCH_BYTES];
 
 namespace ftc {
 
@@ -119,6 +125,36 @@ int64_t scan_workspace_bytes(int64_t N, int64_t H, int64_t L, int64_t D, int64_t
     return need;
 }
 
+// Zeroes `words` 32-bit words (a fill kernel, so that a caller may capture the call in a
+// HIP graph, where memset nodes are best avoided).
+__global__ __launch_bounds__(256) void zero_words_kernel(uint32_t *p, uint32_t words) {
+    for (uint32_t i = blockIdx.x * 256u + threadIdx.x; i < words; i += gridDim.x * 256u) p[i] = 0u;
+}
+
+// Device address of `scratch` on the current device, looked up on the first call per device.
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void *g_scratch_ptr[kMaxDevices];
+
+int scratch_of_device(void **ptr) {
+    int dev = -1;
+    hipError_t err = hipGetDevice(&dev);
+    if (err != hipSuccess) return fail(FTC_ERR_HIP, "hipGetDevice: %s", hipGetErrorString(err));
+    if (dev < 0 || dev >= kMaxDevices)
+        return fail(FTC_ERR_UNSUPPORTED, "device ordinal %d outside [0, %d)", dev, kMaxDevices);
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void *p = nullptr;
+        err = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (err != hipSuccess || !p)
+            return fail(FTC_ERR_HIP, "hipGetSymbolAddress(scratch) on device %d: %s", dev,
+                        hipGetErrorString(err));
+        g_scratch_ptr[dev] = p;
+    }
+    *ptr = g_scratch_ptr[dev];
+    return FTC_OK;
+}
+
 }  // namespace
 }  // namespace ftc
 
@@ -158,6 +194,35 @@ int ftc_causal_dot_product(const ftc_tensor4 *queries, const ftc_tensor4 *keys,
     const ScanDesc fwd = {as_operand(queries), as_operand(keys), as_operand(values),
                           as_operand_out(product), false};
     return run_scans(&fwd, 1, d.N, d.H, d.L, workspace, workspace_bytes, s);
+}
+
+int ftc_causal_dot_product_static(const ftc_tensor4 *queries, const ftc_tensor4 *keys,
+                                  const ftc_tensor4 *values, const ftc_tensor4 *product,
+                                  void *stream) {
+    Dims d;
+    int rc = read_dims(queries, values, &d);
+    if (rc) return rc;
+    int64_t need = 0;
+    if (d.N * d.H * d.L * d.M > 0 && d.E > 0) {
+        need = ftc_causal_dot_product_workspace_bytes(d.N, d.H, d.L, d.E, d.M, queries->dtype);
+        if (need < 0) return (int)need;
+    }
+    if (need > (int64_t)FTC_STATIC_SCRATCH_BYTES)
+        return fail(FTC_ERR_WORKSPACE,
+                    "ftc_causal_dot_product_static: these sizes need %lld bytes of scratch, the "
+                    "built-in array holds %lld; use ftc_causal_dot_product with a workspace",
+                    (long long)need, (long long)FTC_STATIC_SCRATCH_BYTES);
+    void *ws = nullptr;
+    if (need > 0) {
+        if ((rc = scratch_of_device(&ws))) return rc;
+        // The array keeps what the last call left.  The states behind the control block are
+        // written before they are read; the control block must start at zero, and although
+        // every completed call leaves it so, it is cleared here as well so that a call that
+        // was cut short cannot spoil the next one.
+        hipLaunchKernelGGL(zero_words_kernel, dim3(16), dim3(256), 0, (hipStream_t)stream,
+                           (uint32_t *)ws, (uint32_t)(FTC_WORKSPACE_CONTROL_BYTES / 4));
+    }
+    return ftc_causal_dot_product(queries, keys, values, product, ws, (size_t)need, stream);
 }
 
 int ftc_causal_dot_product_state(const ftc_tensor4 *queries, const ftc_tensor4 *keys,

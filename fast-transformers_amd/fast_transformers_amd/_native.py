@@ -23,6 +23,7 @@ EXPORTED_SYMBOLS = (
     "ftc_last_error",
     "ftc_causal_dot_product_workspace_bytes",
     "ftc_causal_dot_product",
+    "ftc_causal_dot_product_static",
     "ftc_causal_dot_product_state",
     "ftc_causal_dot_backward_workspace_bytes",
     "ftc_causal_dot_backward",
@@ -65,6 +66,8 @@ def load():
     lib.ftc_causal_dot_product.restype = ctypes.c_int
     lib.ftc_causal_dot_product.argtypes = [t4] * 4 + [ctypes.c_void_p, ctypes.c_size_t,
                                                       ctypes.c_void_p]
+    lib.ftc_causal_dot_product_static.restype = ctypes.c_int
+    lib.ftc_causal_dot_product_static.argtypes = [t4] * 4 + [ctypes.c_void_p]
     lib.ftc_causal_dot_product_state.restype = ctypes.c_int
     lib.ftc_causal_dot_product_state.argtypes = [t4] * 6 + [ctypes.c_void_p, ctypes.c_size_t,
                                                             ctypes.c_void_p]

@@ -47,6 +47,8 @@ extern "C" {
 #endif
 
 #define FTC_WORKSPACE_CONTROL_BYTES 65536
+/* size of the built-in scratch array of ftc_causal_dot_product_static (per GPU) */
+#define FTC_STATIC_SCRATCH_BYTES (48u << 20)
 
 enum ftc_dtype { FTC_F32 = 0, FTC_BF16 = 1 };
 
@@ -84,6 +86,23 @@ int64_t ftc_causal_dot_product_workspace_bytes(int64_t N, int64_t H, int64_t L, 
 int ftc_causal_dot_product(const ftc_tensor4 *queries, const ftc_tensor4 *keys,
                            const ftc_tensor4 *values, const ftc_tensor4 *product,
                            void *workspace, size_t workspace_bytes, void *stream);
+
+/*
+ * ftc_causal_dot_product for callers that cannot allocate device memory or hand in a
+ * workspace: code under HIP graph capture, tight serving loops, harnesses that forbid
+ * hipMalloc.  It has no counterpart in the reference.  Same arguments and result as
+ * ftc_causal_dot_product, without the workspace: the scratch memory is an array of
+ * FTC_STATIC_SCRATCH_BYTES that is part of the library's device code (each GPU the library
+ * runs on holds one until the process ends).  The call allocates and frees nothing and
+ * enqueues kernels only.  Sizes whose scratch need
+ * (ftc_causal_dot_product_workspace_bytes) exceeds the array are refused with
+ * FTC_ERR_WORKSPACE.  All calls on one GPU share that GPU's array: two calls whose work
+ * overlaps in time on one GPU (different streams, different threads) race; calls on one
+ * stream are safe.
+ */
+int ftc_causal_dot_product_static(const ftc_tensor4 *queries, const ftc_tensor4 *keys,
+                                  const ftc_tensor4 *values, const ftc_tensor4 *product,
+                                  void *stream);
 
 /*
  * The product with the running state handed in and out, for processing a sequence in
