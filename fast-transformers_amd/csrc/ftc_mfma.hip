@@ -3,7 +3,7 @@
 #include <algorithm>
 #include <cstdlib>
 
-#include "ftc_mfma_dma_kernel.h"
+#include "ftc_wg_kernel.h"
 
 namespace ftc {
 using namespace mfma;
@@ -14,8 +14,17 @@ struct MfmaPlan {
     int64_t waves, workspace_bytes;
 };
 
-MfmaPlan make_plan(int64_t N, int64_t H, int64_t L, int64_t D, int64_t F, int nscans) {
+// all-fp32 scans of these widths run as workgroups of F / 32 wavefronts (ftc_wg_kernel.h)
+bool use_wg_kernel(int64_t D, int64_t F, bool all_f32) {
+    if (!all_f32 || !scan_wg_covers((int)D, (int)F)) return false;
+    if (const char *env = getenv("FTC_WG")) return atoi(env) != 0;  // tuning aid
+    return false;
+}
+
+// `wg`: the plan is for workgroups of F / 32 wavefronts (each has its own flag words)
+MfmaPlan make_plan(int64_t N, int64_t H, int64_t L, int64_t D, int64_t F, int nscans, bool wg) {
     MfmaPlan pl;
+    const int64_t flags_per_unit = wg ? F / 32 : 1;
     const int64_t chains = std::max<int64_t>(1, N * H);
     const int64_t total_chunks = (L + kChunk - 1) / kChunk;
     // One wavefront per SIMD is resident (register footprint): 1024 slots.  Pick the segment
@@ -27,7 +36,7 @@ MfmaPlan make_plan(int64_t N, int64_t H, int64_t L, int64_t D, int64_t F, int ns
     for (int64_t c = 1; c < total_chunks && c <= 4096; c++) {
         const int64_t nseg = (total_chunks + c - 1) / c;
         const int64_t waves = chains * nseg;
-        if (waves * nscans > kMaxWaves || nseg > 4096) continue;  // <= 64 groups of 64 steps
+        if (waves * nscans * flags_per_unit > kMaxWaves || nseg > 4096) continue;  // <= 64 groups of 64 steps
         const double rounds = (double)((waves * nscans + 1023) / 1024);
         const double per_wave = nseg > 1 ? c * 1.5 + 3.0 : (double)c;
         const double cost = rounds * per_wave;
@@ -41,7 +50,7 @@ MfmaPlan make_plan(int64_t N, int64_t H, int64_t L, int64_t D, int64_t F, int ns
         const int64_t forced = atoll(env);
         if (forced >= 1 && forced <= total_chunks) {
             const int64_t nseg = (total_chunks + forced - 1) / forced;
-            if (chains * nseg * nscans <= kMaxWaves && nseg <= 4096) best_c = forced;
+            if (chains * nseg * nscans * flags_per_unit <= kMaxWaves && nseg <= 4096) best_c = forced;
         }
     }
     pl.seg_len = (int)(best_c * kChunk);
@@ -130,15 +139,18 @@ bool mfma_scan_supported(const ScanDesc &sd, int64_t L) {
 
 int64_t mfma_scan_workspace_bytes(int64_t N, int64_t H, int64_t L, int64_t D, int64_t F,
                                   int nscans) {
-    const MfmaPlan pl = make_plan(N, H, L, D, F, nscans);
-    return pl.workspace_bytes;
+    // whichever kernel the element types will select
+    return std::max(make_plan(N, H, L, D, F, nscans, false).workspace_bytes,
+                    make_plan(N, H, L, D, F, nscans, true).workspace_bytes);
 }
 
 int mfma_scan(const ScanDesc *scans, int nscans, int64_t N, int64_t H, int64_t L,
               void *workspace, size_t workspace_bytes, hipStream_t stream) {
     if (nscans < 1 || nscans > kMaxScans) return fail(FTC_ERR_INVALID, "bad scan count");
     const int D = scans[0].a.width, F = scans[0].v.width;
-    const MfmaPlan pl = make_plan(N, H, L, D, F, nscans);
+    const Combo combo = combo_of(scans[0]);
+    const bool wg = use_wg_kernel(D, F, combo == kFFFF);
+    const MfmaPlan pl = make_plan(N, H, L, D, F, nscans, wg);
     if (pl.workspace_bytes > 0 && (!workspace || workspace_bytes < (size_t)pl.workspace_bytes))
         return fail(FTC_ERR_WORKSPACE, "workspace of %lld bytes needed, %zu given",
                     (long long)pl.workspace_bytes, workspace_bytes);
@@ -184,14 +196,15 @@ int mfma_scan(const ScanDesc *scans, int nscans, int64_t N, int64_t H, int64_t L
     // tuning aid: FTC_GROUP=<n> forces groups of n steps
     if (const char *env = getenv("FTC_GROUP")) args.group = std::max(1, atoi(env));
 
-    const Combo combo = combo_of(scans[0]);
     for (int i = 1; i < nscans; i++)
         if (combo_of(scans[i]) != combo || scans[i].a.width != D || scans[i].v.width != F)
             return fail(FTC_ERR_INVALID, "scans of one launch must share widths and dtypes");
     // fp32 states of up to 64 rows: the kernel that feeds its fragments from LDS tiles
     bool dma = D <= 64 && combo == kFFFF;
     if (const char *env = getenv("FTC_DMA")) dma = dma && atoi(env) != 0;  // tuning aid
-    if (dma) {
+    if (wg) {
+        launch_scan_wg_ffff(D, F, workspace, args, stream);
+    } else if (dma) {
         launch_scan_dma_ffff(D, F, workspace, args, stream);
     } else switch (combo) {
         case kFFFF: launch_scan_ffff(D, F, workspace, args, stream); break;

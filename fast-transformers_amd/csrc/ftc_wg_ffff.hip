@@ -1,0 +1,28 @@
+// Workgroup scan, all-fp32 rows: instantiations and launcher.
+#include "ftc_wg_kernel.h"
+
+namespace ftc {
+namespace mfma {
+
+bool scan_wg_covers(int D, int F) {
+    return (D == 64 && (F == 64 || F == 32 || F == 128)) ||
+           (D == 32 && (F == 32 || F == 64 || F == 128));
+}
+
+void launch_scan_wg_ffff(int D, int F, void *workspace, const ScanArgs &args,
+                         hipStream_t stream) {
+    const dim3 grid((unsigned)args.total_waves), block(64 * (F / 32));
+#define FTC_LAUNCH(DD, FF)                                                                   \
+    hipLaunchKernelGGL((scan_wg_kernel<DD, FF>), grid, block, 0, stream, (uint32_t *)workspace, \
+                       args)
+    if (D == 64 && F == 64) FTC_LAUNCH(64, 64);
+    else if (D == 64 && F == 32) FTC_LAUNCH(64, 32);
+    else if (D == 64 && F == 128) FTC_LAUNCH(64, 128);
+    else if (D == 32 && F == 32) FTC_LAUNCH(32, 32);
+    else if (D == 32 && F == 64) FTC_LAUNCH(32, 64);
+    else FTC_LAUNCH(32, 128);
+#undef FTC_LAUNCH
+}
+
+}  // namespace mfma
+}  // namespace ftc
