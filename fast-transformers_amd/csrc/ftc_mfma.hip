@@ -27,17 +27,19 @@ MfmaPlan make_plan(int64_t N, int64_t H, int64_t L, int64_t D, int64_t F, int ns
     const int64_t flags_per_unit = wg ? F / 32 : 1;
     const int64_t chains = std::max<int64_t>(1, N * H);
     const int64_t total_chunks = (L + kChunk - 1) / kChunk;
-    // One wavefront per SIMD is resident (register footprint): 1024 slots.  Pick the segment
+    // Resident at a time: 1024 wavefronts (one per SIMD: register footprint), or one workgroup
+    // per CU with 4 / (F / 32) segments each.  Pick the segment
     // length (in chunks) that minimises an estimate of the makespan: rounds of resident
     // wavefronts times the work of one wavefront (pass 1 costs about half of pass 2, the
     // exchange of segment sums about three chunks).
+    const int64_t slots = wg ? 256 * scan_wg_units_per_block((int)F) : 1024;
     int64_t best_c = total_chunks;
-    double best_cost = (double)total_chunks * (double)((chains * nscans + 1023) / 1024);
+    double best_cost = (double)total_chunks * (double)((chains * nscans + slots - 1) / slots);
     for (int64_t c = 1; c < total_chunks && c <= 4096; c++) {
         const int64_t nseg = (total_chunks + c - 1) / c;
         const int64_t waves = chains * nseg;
         if (waves * nscans * flags_per_unit > kMaxWaves || nseg > 4096) continue;  // <= 64 groups of 64 steps
-        const double rounds = (double)((waves * nscans + 1023) / 1024);
+        const double rounds = (double)((waves * nscans + slots - 1) / slots);
         const double per_wave = nseg > 1 ? c * 1.5 + 3.0 : (double)c;
         const double cost = rounds * per_wave;
         if (cost < best_cost - 1e-9) {

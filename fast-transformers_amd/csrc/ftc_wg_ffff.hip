@@ -5,18 +5,20 @@ namespace ftc {
 namespace mfma {
 
 bool scan_wg_covers(int D, int F) {
-    return (D == 64 && (F == 64 || F == 32 || F == 128)) ||
-           (D == 32 && (F == 32 || F == 64 || F == 128));
+    return (D == 64 && (F == 64 || F == 128)) || (D == 32 && (F == 32 || F == 64 || F == 128));
 }
 
 void launch_scan_wg_ffff(int D, int F, void *workspace, const ScanArgs &args,
                          hipStream_t stream) {
-    const dim3 grid((unsigned)args.total_waves), block(64 * (F / 32));
+    // args.waves_per_scan / args.total_waves count units; a workgroup carries several
+    const unsigned ns = (unsigned)scan_wg_units_per_block(F);
+    const unsigned nscans = (unsigned)(args.total_waves / args.waves_per_scan);
+    const unsigned blocks_per_scan = ((unsigned)args.waves_per_scan + ns - 1) / ns;
+    const dim3 grid(nscans * blocks_per_scan), block(512);
 #define FTC_LAUNCH(DD, FF)                                                                   \
     hipLaunchKernelGGL((scan_wg_kernel<DD, FF>), grid, block, 0, stream, (uint32_t *)workspace, \
                        args)
     if (D == 64 && F == 64) FTC_LAUNCH(64, 64);
-    else if (D == 64 && F == 32) FTC_LAUNCH(64, 32);
     else if (D == 64 && F == 128) FTC_LAUNCH(64, 128);
     else if (D == 32 && F == 32) FTC_LAUNCH(32, 32);
     else if (D == 32 && F == 64) FTC_LAUNCH(32, 64);
