@@ -354,10 +354,15 @@ __global__ __launch_bounds__(512, 2) void scan_wg_kernel(uint32_t *__restrict__ 
             vt_addr[u] = kOffV + PieceSwizzle<RBV>::addr(row, 2 * (32 * w + 16 * (G % 2) + 4 * x));
         }
     }
-    // causal mask inside a chunk: accumulator register r of lane (i = ln, g) holds row
-    // j = 8 (r / 4) + 4 g + r % 4 of Pt, kept when j <= i (REV: j >= i), i.e. when
-    // mask_t = i - 4 g >= (<=) 8 (r / 4) + r % 4
-    const int mask_t = ln - 4 * g;
+    // causal mask inside a chunk as bit masks (all ones: keep): accumulator register r of
+    // lane (i = ln, g) holds row j = 8 (r / 4) + 4 g + r % 4 of Pt
+    uint32_t keep[16];
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+        const int j = 8 * (r / 4) + 4 * g + (r % 4);
+        keep[r] = (REV ? (j >= ln) : (j <= ln)) ? 0xffffffffu : 0u;
+        asm volatile("" : "+v"(keep[r]));
+    }
     f32x16 S[DT];
 #pragma unroll
     for (int dt = 0; dt < DT; dt++)
@@ -430,9 +435,10 @@ __global__ __launch_bounds__(512, 2) void scan_wg_kernel(uint32_t *__restrict__ 
                                 32 * w + ln, g, S);
 
     // ---- pass 2: outputs ----
-    // Every fragment of a chunk is requested from LDS well before the matrix instruction
-    // that consumes it: a consumer is alone on its SIMD with matrix work, so nothing else
-    // would fill the wait.
+    // A consumer is the only wavefront with matrix work on its SIMD, and a wavefront issues in
+    // order: its own vector ALU work (cutting S and Pt) and its LDS reads only overlap with
+    // its matrix instructions when they alternate in the instruction stream.  The body of a
+    // chunk is therefore one scheduling region whose instruction mix is prescribed at the end.
     wg_barrier();
     for (int c = 0; c < n2max; c++) {
         if (c < n2) {
@@ -445,20 +451,16 @@ __global__ __launch_bounds__(512, 2) void scan_wg_kernel(uint32_t *__restrict__ 
                     af[ks][k] = lds_frag16(pc + k * kTileA + row_addr[ks]);
                     bf[ks][k] = lds_frag16(pc + kOffB + k * kTileA + row_addr[ks]);
                 }
-            __builtin_amdgcn_sched_barrier(0);
-            // (1) Pt = b a^T (every consumer of the unit needs all of it)
-            f32x16 P;
-#pragma unroll
-            for (int r = 0; r < 16; r++) P[r] = 0.f;
-#pragma unroll
-            for (int ks = 0; ks < KD; ks++) P = mfma_split<3, 3>(bf[ks], af[ks], P);
             v_frags(pc, v_frag);
-            // (2b) Ot = S^T a^T while Pt is on its way
-            f32x16 O;
+            bt_frags(pc, bt);
+            // (1) Pt = b a^T (every consumer of the unit needs all of it) and
+            // (2b) Ot = S^T a^T, k-step by k-step
+            f32x16 P, O;
 #pragma unroll
-            for (int r = 0; r < 16; r++) O[r] = 0.f;
+            for (int r = 0; r < 16; r++) P[r] = 0.f, O[r] = 0.f;
 #pragma unroll
             for (int ks = 0; ks < KD; ks++) {
+                P = mfma_split<3, 3>(bf[ks], af[ks], P);
                 const int o8 = 8 * (ks % 2);
                 const float x[8] = {S[ks / 2][o8 + 0], S[ks / 2][o8 + 1], S[ks / 2][o8 + 2],
                                     S[ks / 2][o8 + 3], S[ks / 2][o8 + 4], S[ks / 2][o8 + 5],
@@ -467,15 +469,11 @@ __global__ __launch_bounds__(512, 2) void scan_wg_kernel(uint32_t *__restrict__ 
                 split8<3>(x, s_frag);
                 O = mfma_split<3, 3>(s_frag, af[ks], O);
             }
-            __builtin_amdgcn_sched_barrier(0);
-            bt_frags(pc, bt);
-            // mask and cut Pt
+            // (3) S += b^T v, with the masking and cutting of Pt underneath
+            update_state(bt, v_frag);
             Frag p_frag[2][3];
 #pragma unroll
-            for (int r = 0; r < 16; r++) {
-                const int j0 = 8 * (r / 4) + (r % 4);  // row j = j0 + 4 g of Pt
-                P[r] = (REV ? mask_t <= j0 : mask_t >= j0) ? P[r] : 0.f;
-            }
+            for (int r = 0; r < 16; r++) P[r] = __uint_as_float(__float_as_uint(P[r]) & keep[r]);
 #pragma unroll
             for (int hh = 0; hh < 2; hh++) {
                 const float x[8] = {P[8 * hh + 0], P[8 * hh + 1], P[8 * hh + 2], P[8 * hh + 3],
@@ -491,9 +489,22 @@ __global__ __launch_bounds__(512, 2) void scan_wg_kernel(uint32_t *__restrict__ 
             for (int q = 0; q < 4; q++)
                 buffer_store4(o_rs, o_off + (uint32_t)(4 * 8 * q), O[4 * q + 0], O[4 * q + 1],
                               O[4 * q + 2], O[4 * q + 3]);
-            __builtin_amdgcn_sched_barrier(0);
-            // (3) S += b^T v
-            update_state(bt, v_frag);
+            // instruction mix: row-major fragments first; then the 12 KD matrix instructions of
+            // (1) and (2b) with three vector instructions (cutting S) and one transposing read
+            // after each; then the 12 DT of (3) with three vector instructions (Pt) each
+            constexpr int kMfma = 0x008, kValu = 0x002, kDsRead = 0x100;
+            __builtin_amdgcn_sched_group_barrier(kDsRead, 6 * KD, 0);
+#pragma unroll
+            for (int i = 0; i < 12 * KD; i++) {
+                __builtin_amdgcn_sched_group_barrier(kMfma, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(kValu, 3, 0);
+                __builtin_amdgcn_sched_group_barrier(kDsRead, 1, 0);
+            }
+#pragma unroll
+            for (int i = 0; i < 12 * DT; i++) {
+                __builtin_amdgcn_sched_group_barrier(kMfma, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(kValu, 3, 0);
+            }
         }
         wg_barrier();
     }
