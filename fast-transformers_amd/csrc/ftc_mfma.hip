@@ -62,6 +62,9 @@ MfmaPlan make_plan(int64_t N, int64_t H, int64_t L, int64_t D, int64_t F, int ns
     if (pl.nseg > 1)
         pl.workspace_bytes =
             kControlBytes + 2 * nscans * pl.waves * D * F * (int64_t)sizeof(float);
+#ifdef FTC_TIMELINE
+    pl.workspace_bytes += nscans * pl.waves * 128;  // time stamps (ftc_wg_kernel.h)
+#endif
     return pl;
 }
 

@@ -78,6 +78,20 @@ __device__ __forceinline__ Frag lds_frag_tr(const lds_char *p0, const lds_char *
     return Frag{{lo.x, lo.y, hi.x, hi.y}};
 }
 
+// Tuning aid: with -DFTC_TIMELINE the first consumer of every unit records when it passes the
+// marked points (s_memrealtime ticks) behind the state slots of the workspace, 16 words per
+// unit; the host side then reserves that room.
+#ifdef FTC_TIMELINE
+#define FTC_STAMP(i)                                                                  \
+    do {                                                                              \
+        if (stamp_on) stamp_base[(i)] = __builtin_amdgcn_s_memrealtime();             \
+    } while (0)
+#else
+#define FTC_STAMP(i) \
+    do {             \
+    } while (0)
+#endif
+
 // Workgroup barrier that waits for this wavefront's LDS traffic only: rows requested from
 // memory for a later chunk stay in flight across it (__syncthreads would wait for them).
 __device__ __forceinline__ void wg_barrier() {
@@ -326,6 +340,14 @@ __global__ __launch_bounds__(512, 2) void scan_wg_kernel(uint32_t *__restrict__ 
     }
 
     // =========================== consumers ===========================
+#ifdef FTC_TIMELINE
+    typedef __attribute__((address_space(1))) uint64_t gu64;
+    const bool stamp_on = valid && p.nseg > 1 && w == 0 && lane == 0;
+    gu64 *const stamp_base =
+        (gu64 *)((__attribute__((address_space(1))) char *)ws_ptr + kControlBytes +
+                 (int64_t)2 * p.total_waves * (D * F * 4)) + (valid ? sg.ticket : 0) * 16;
+#endif
+    FTC_STAMP(0);
     const uint32_t vticket = (uint32_t)w * total_units + (valid ? sg.ticket : 0);
     const uint32_t o_slb = (uint32_t)op.o_sl * 4;
     char *o_seg = (char *)op.out + ((int64_t)n * op.o_sn + (int64_t)h * op.o_sh + lo * op.o_sl) * 4;
@@ -420,6 +442,7 @@ __global__ __launch_bounds__(512, 2) void scan_wg_kernel(uint32_t *__restrict__ 
             xch.publish_sum(Sx);
         }
     }
+    FTC_STAMP(1);
     if (exchange) {
         f32x16 X[DT][1];
 #pragma unroll
@@ -439,7 +462,9 @@ __global__ __launch_bounds__(512, 2) void scan_wg_kernel(uint32_t *__restrict__ 
     // order: its own vector ALU work (cutting S and Pt) and its LDS reads only overlap with
     // its matrix instructions when they alternate in the instruction stream.  The body of a
     // chunk is therefore one scheduling region whose instruction mix is prescribed at the end.
+    FTC_STAMP(2);
     wg_barrier();
+    FTC_STAMP(3);
     for (int c = 0; c < n2max; c++) {
         if (c < n2) {
             const lds_char *pc = unit_pc + (c & 1) * kBufBytes;
@@ -507,7 +532,9 @@ __global__ __launch_bounds__(512, 2) void scan_wg_kernel(uint32_t *__restrict__ 
             }
         }
         wg_barrier();
+        if (c < 8) FTC_STAMP(8 + c);
     }
+    FTC_STAMP(4);
     if (!valid) return;
     if (op.s_out && step == p.nseg - 1)
         wg_store_caller_state<DT>(op.s_out + (int64_t)n * op.so_sn + (int64_t)h * op.so_sh,
