@@ -98,12 +98,28 @@ __device__ __forceinline__ void wg_barrier() {
     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 }
 
+// split_pair<3> for a wavefront that also feeds the matrix cores.  v_dot2c_f32_bf16, which
+// split_pair uses to subtract a piece, does not issue while a matrix instruction of the same
+// wavefront is in flight (measured: each one adds its full 2.5 ns to a 14 ns MFMA), whereas
+// v_and_b32, v_sub_f32 and v_perm_b32 do (six of them cost 2.7 ns together).  Here the
+// remainder is x - (x & 0xffff0000): one more instruction per value and piece, all hidden.
+__device__ __forceinline__ void split_pair_under_mfma(float x0, float x1, uint32_t (&out)[3]) {
+#pragma unroll
+    for (int p = 0; p < 3; p++) {
+        out[p] = pack_hi16(x0, x1);
+        if (p + 1 < 3) {
+            x0 = x0 - __uint_as_float(__float_as_uint(x0) & 0xffff0000u);
+            x1 = x1 - __uint_as_float(__float_as_uint(x1) & 0xffff0000u);
+        }
+    }
+}
+
 // Four consecutive fp32 values of a row -> 8 bytes of each of the three piece tiles.
 __device__ __forceinline__ void split_quad_to_lds(const u32x4 raw, lds_char *tile, int piece_bytes,
                                                   int addr) {
     uint32_t lo[3], hi[3];
-    split_pair<3>(__uint_as_float(raw.x), __uint_as_float(raw.y), lo);
-    split_pair<3>(__uint_as_float(raw.z), __uint_as_float(raw.w), hi);
+    split_pair_under_mfma(__uint_as_float(raw.x), __uint_as_float(raw.y), lo);
+    split_pair_under_mfma(__uint_as_float(raw.z), __uint_as_float(raw.w), hi);
 #pragma unroll
     for (int pc = 0; pc < 3; pc++) {
         const u32x2 w = {lo[pc], hi[pc]};
@@ -281,58 +297,78 @@ __global__ __launch_bounds__(512, 2) void scan_wg_kernel(uint32_t *__restrict__ 
             v_goff[q] = (uint32_t)row * v_slb + 16u * c4;
             v_waddr[q] = PieceSwizzle<RBV>::addr(row, 8 * c4);
         }
-        u32x4 a_raw[LA], b_raw[LA], v_raw[LV];
-        auto fetch = [&](int row0, bool with_a) {
+        // Rows are requested two chunks ahead of the cut, into two sets of registers that
+        // take turns, so that a request has a whole chunk's time to be served.
+        struct Raw {
+            u32x4 a[LA], b[LA], v[LV];
+        };
+        Raw raw0, raw1;
+        auto fetch = [&](Raw &r, int row0, bool with_a) {
 #pragma unroll
             for (int q = 0; q < LA; q++) {
                 if (with_a)
-                    a_raw[q] = __builtin_amdgcn_raw_buffer_load_b128(
+                    r.a[q] = __builtin_amdgcn_raw_buffer_load_b128(
                         a_rs, a_goff[q] + (uint32_t)row0 * a_slb, 0, 0);
-                b_raw[q] = __builtin_amdgcn_raw_buffer_load_b128(
+                r.b[q] = __builtin_amdgcn_raw_buffer_load_b128(
                     b_rs, b_goff[q] + (uint32_t)row0 * b_slb, 0, 0);
             }
 #pragma unroll
             for (int q = 0; q < LV; q++)
-                v_raw[q] = __builtin_amdgcn_raw_buffer_load_b128(
+                r.v[q] = __builtin_amdgcn_raw_buffer_load_b128(
                     v_rs, v_goff[q] + (uint32_t)row0 * v_slb, 0, 0);
         };
-        auto cut = [&](int buf, bool with_a) {
+        auto cut = [&](const Raw &r, int buf, bool with_a) {
             lds_char *const pc = unit_pc + buf * kBufBytes;
 #pragma unroll
             for (int q = 0; q < LA; q++) {
-                if (with_a) split_quad_to_lds(a_raw[q], pc, kTileA, a_waddr[q]);
-                split_quad_to_lds(b_raw[q], pc + kOffB, kTileA, a_waddr[q]);
+                if (with_a) split_quad_to_lds(r.a[q], pc, kTileA, a_waddr[q]);
+                split_quad_to_lds(r.b[q], pc + kOffB, kTileA, a_waddr[q]);
             }
 #pragma unroll
-            for (int q = 0; q < LV; q++) split_quad_to_lds(v_raw[q], pc + kOffV, kTileV, v_waddr[q]);
+            for (int q = 0; q < LV; q++) split_quad_to_lds(r.v[q], pc + kOffV, kTileV, v_waddr[q]);
         };
         // rows of a chunk that does not exist lie outside the descriptor and read as zero
         auto pass1_row0 = [&](int i) -> int { return i < n1 ? chunk_row0(n1 - 1 - i) : -2 * kChunk; };
         auto pass2_row0 = [&](int c) -> int { return c < n2 ? chunk_row0(c) : -2 * kChunk; };
 
-        // ---- pass 1: chunk i of the walk (against the direction of pass 2) -> buffer i % 2 ----
+        // ---- pass 1: chunk i of the walk (against the direction of pass 2) -> buffer i % 2;
+        // even chunks travel through raw0, odd ones through raw1 ----
         if (n1max > 0) {
-            fetch(pass1_row0(0), false);
-            cut(0, false);
-            fetch(pass1_row0(1), false);
+            fetch(raw0, pass1_row0(0), false);
+            fetch(raw1, pass1_row0(1), false);
+            cut(raw0, 0, false);
+            fetch(raw0, pass1_row0(2), false);
             wg_barrier();
-            for (int i = 0; i < n1max; i++) {
+            for (int i = 0; i < n1max; i += 2) {
                 if (i + 1 < n1max) {
-                    cut((i + 1) & 1, false);
-                    fetch(pass1_row0(i + 2), false);
+                    cut(raw1, 1, false);
+                    fetch(raw1, pass1_row0(i + 3), false);
+                }
+                wg_barrier();
+                if (i + 1 >= n1max) break;
+                if (i + 2 < n1max) {
+                    cut(raw0, 0, false);
+                    fetch(raw0, pass1_row0(i + 4), false);
                 }
                 wg_barrier();
             }
         }
         // ---- pass 2 ----
-        fetch(pass2_row0(0), true);
-        cut(0, true);
-        fetch(pass2_row0(1), true);
+        fetch(raw0, pass2_row0(0), true);
+        fetch(raw1, pass2_row0(1), true);
+        cut(raw0, 0, true);
+        fetch(raw0, pass2_row0(2), true);
         wg_barrier();
-        for (int c = 0; c < n2max; c++) {
+        for (int c = 0; c < n2max; c += 2) {
             if (c + 1 < n2max) {
-                cut((c + 1) & 1, true);
-                fetch(pass2_row0(c + 2), true);
+                cut(raw1, 1, true);
+                fetch(raw1, pass2_row0(c + 3), true);
+            }
+            wg_barrier();
+            if (c + 1 >= n2max) break;
+            if (c + 2 < n2max) {
+                cut(raw0, 0, true);
+                fetch(raw0, pass2_row0(c + 4), true);
             }
             wg_barrier();
         }
@@ -459,16 +495,27 @@ __global__ __launch_bounds__(512, 2) void scan_wg_kernel(uint32_t *__restrict__ 
 
     // ---- pass 2: outputs ----
     // A consumer is the only wavefront with matrix work on its SIMD, and a wavefront issues in
-    // order: its own vector ALU work (cutting S and Pt) and its LDS reads only overlap with
-    // its matrix instructions when they alternate in the instruction stream.  The body of a
-    // chunk is therefore one scheduling region whose instruction mix is prescribed at the end.
+    // order: its own vector ALU work (cutting S and Pt) and its LDS reads overlap with its
+    // matrix instructions only when they alternate in the instruction stream.  The body of a
+    // chunk is therefore written out in that order, one matrix instruction and what goes
+    // under it at a time, with scheduling barriers that keep the compiler from regrouping it:
+    //
+    //   cut S(0) | (1)[0] + cut S(1) | (2b)[0] + reads | (1)[1] + cut S(2) | (2b)[1] + reads | ...
+    //   | (3) + mask and cut Pt | (2a) | store
+    //
+    // (1)[ks], (2b)[ks]: the six matrix instructions of k-step ks of Pt = b a^T and of
+    // Ot = S^T a^T; "reads": the transposing reads of v and b^T for (3) and (2a).
+    constexpr int kPa[6] = {0, 1, 2, 0, 1, 0}, kPb[6] = {2, 1, 0, 1, 0, 0};  // piece products
+    constexpr int kTrFrags = 6 + 6 * DT;  // position-major fragments of a chunk
+    constexpr int kM3 = 12 * DT;          // matrix instructions of (3)
     FTC_STAMP(2);
     wg_barrier();
     FTC_STAMP(3);
     for (int c = 0; c < n2max; c++) {
         if (c < n2) {
             const lds_char *pc = unit_pc + (c & 1) * kBufBytes;
-            Frag af[KD][3], bf[KD][3], v_frag[2][3], bt[2][DT][3];
+            Frag af[KD][3], bf[KD][3], v_frag[2][3], bt[2][DT][3], sf[2][3], p_frag[2][3];
+            f32x16 P, O;
 #pragma unroll
             for (int ks = 0; ks < KD; ks++)
 #pragma unroll
@@ -476,60 +523,75 @@ __global__ __launch_bounds__(512, 2) void scan_wg_kernel(uint32_t *__restrict__ 
                     af[ks][k] = lds_frag16(pc + k * kTileA + row_addr[ks]);
                     bf[ks][k] = lds_frag16(pc + kOffB + k * kTileA + row_addr[ks]);
                 }
-            v_frags(pc, v_frag);
-            bt_frags(pc, bt);
-            // (1) Pt = b a^T (every consumer of the unit needs all of it) and
-            // (2b) Ot = S^T a^T, k-step by k-step
-            f32x16 P, O;
+            // pair q of k-step ks of S -> sf[ks % 2]
+            auto cut_s = [&](int ks, int q) {
+                uint32_t o[3];
+                split_pair_under_mfma(S[ks / 2][8 * (ks % 2) + 2 * q],
+                                      S[ks / 2][8 * (ks % 2) + 2 * q + 1], o);
+#pragma unroll
+                for (int k = 0; k < 3; k++) sf[ks % 2][k].w[q] = o[k];
+            };
+            // position-major fragment number i in the order in which (3) and (2a) use them
+            auto tr_frag = [&](int i) {
+                const int hh = i / (3 + 3 * DT), j = i % (3 + 3 * DT);
+                if (j < 3)
+                    v_frag[hh][j] = lds_frag_tr(pc + j * kTileV + hh * 16 * RBV + vt_addr[0],
+                                                pc + j * kTileV + hh * 16 * RBV + vt_addr[1]);
+                else {
+                    const int dt = (j - 3) / 3, k = (j - 3) % 3;
+                    bt[hh][dt][k] = lds_frag_tr(pc + k * kTileA + hh * 16 * RBA + bt_addr[dt][0],
+                                                pc + k * kTileA + hh * 16 * RBA + bt_addr[dt][1]);
+                }
+            };
 #pragma unroll
             for (int r = 0; r < 16; r++) P[r] = 0.f, O[r] = 0.f;
 #pragma unroll
+            for (int q = 0; q < 4; q++) cut_s(0, q);
+            __builtin_amdgcn_sched_barrier(0);
+            int tr_next = 0;
+#pragma unroll
             for (int ks = 0; ks < KD; ks++) {
-                P = mfma_split<3, 3>(bf[ks], af[ks], P);
-                const int o8 = 8 * (ks % 2);
-                const float x[8] = {S[ks / 2][o8 + 0], S[ks / 2][o8 + 1], S[ks / 2][o8 + 2],
-                                    S[ks / 2][o8 + 3], S[ks / 2][o8 + 4], S[ks / 2][o8 + 5],
-                                    S[ks / 2][o8 + 6], S[ks / 2][o8 + 7]};
-                Frag s_frag[3];
-                split8<3>(x, s_frag);
-                O = mfma_split<3, 3>(s_frag, af[ks], O);
+#pragma unroll
+                for (int i = 0; i < 6; i++) {  // (1)[ks], with S(ks + 1) cut underneath
+                    P = mfma(bf[ks][kPa[i]], af[ks][kPb[i]], P);
+                    if (ks + 1 < KD && i < 4) cut_s(ks + 1, i);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+#pragma unroll
+                for (int i = 0; i < 6; i++) {  // (2b)[ks], with the transposing reads underneath
+                    O = mfma(sf[ks % 2][kPa[i]], af[ks][kPb[i]], O);
+                    if (tr_next < kTrFrags) tr_frag(tr_next++);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
             }
             // (3) S += b^T v, with the masking and cutting of Pt underneath
-            update_state(bt, v_frag);
-            Frag p_frag[2][3];
 #pragma unroll
-            for (int r = 0; r < 16; r++) P[r] = __uint_as_float(__float_as_uint(P[r]) & keep[r]);
+            for (int i = 0; i < kM3; i++) {
+                const int hh = i / (6 * DT), dt = (i / 6) % DT, m = i % 6;
+                S[dt] = mfma(bt[hh][dt][kPa[m]], v_frag[hh][kPb[m]], S[dt]);
 #pragma unroll
-            for (int hh = 0; hh < 2; hh++) {
-                const float x[8] = {P[8 * hh + 0], P[8 * hh + 1], P[8 * hh + 2], P[8 * hh + 3],
-                                    P[8 * hh + 4], P[8 * hh + 5], P[8 * hh + 6], P[8 * hh + 7]};
-                split8<3>(x, p_frag[hh]);
+                for (int u = 0; u < 8; u++)
+                    if ((u * kM3) / 8 == i) {  // pair u of Pt: registers 2 u, 2 u + 1
+                        uint32_t o[3];
+                        split_pair_under_mfma(
+                            __uint_as_float(__float_as_uint(P[2 * u]) & keep[2 * u]),
+                            __uint_as_float(__float_as_uint(P[2 * u + 1]) & keep[2 * u + 1]), o);
+#pragma unroll
+                        for (int k = 0; k < 3; k++) p_frag[u / 4][k].w[u % 4] = o[k];
+                    }
+                __builtin_amdgcn_sched_barrier(0);
             }
             // (2a) Ot += v^T Pt
 #pragma unroll
-            for (int hh = 0; hh < 2; hh++) O = mfma_split<3, 3>(v_frag[hh], p_frag[hh], O);
+            for (int hh = 0; hh < 2; hh++)
+#pragma unroll
+                for (int m = 0; m < 6; m++) O = mfma(v_frag[hh][kPa[m]], p_frag[hh][kPb[m]], O);
             // lane (i = ln, g) holds f = 32 w + 8 q + 4 g + 0..3 in registers 4 q .. 4 q + 3
             const uint32_t o_off = o_lane + (uint32_t)chunk_row0(c) * o_slb;
 #pragma unroll
             for (int q = 0; q < 4; q++)
                 buffer_store4(o_rs, o_off + (uint32_t)(4 * 8 * q), O[4 * q + 0], O[4 * q + 1],
                               O[4 * q + 2], O[4 * q + 3]);
-            // instruction mix: row-major fragments first; then the 12 KD matrix instructions of
-            // (1) and (2b) with three vector instructions (cutting S) and one transposing read
-            // after each; then the 12 DT of (3) with three vector instructions (Pt) each
-            constexpr int kMfma = 0x008, kValu = 0x002, kDsRead = 0x100;
-            __builtin_amdgcn_sched_group_barrier(kDsRead, 6 * KD, 0);
-#pragma unroll
-            for (int i = 0; i < 12 * KD; i++) {
-                __builtin_amdgcn_sched_group_barrier(kMfma, 1, 0);
-                __builtin_amdgcn_sched_group_barrier(kValu, 3, 0);
-                __builtin_amdgcn_sched_group_barrier(kDsRead, 1, 0);
-            }
-#pragma unroll
-            for (int i = 0; i < 12 * DT; i++) {
-                __builtin_amdgcn_sched_group_barrier(kMfma, 1, 0);
-                __builtin_amdgcn_sched_group_barrier(kValu, 3, 0);
-            }
         }
         wg_barrier();
         if (c < 8) FTC_STAMP(8 + c);
