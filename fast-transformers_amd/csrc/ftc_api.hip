@@ -196,6 +196,18 @@ int ftc_causal_dot_product(const ftc_tensor4 *queries, const ftc_tensor4 *keys,
     return run_scans(&fwd, 1, d.N, d.H, d.L, workspace, workspace_bytes, s);
 }
 
+int ftc_workspace_reset(void *workspace, size_t workspace_bytes, void *stream) {
+    if (!workspace || workspace_bytes < (size_t)FTC_WORKSPACE_CONTROL_BYTES)
+        return fail(FTC_ERR_WORKSPACE, "a workspace has at least %d bytes",
+                    (int)FTC_WORKSPACE_CONTROL_BYTES);
+    hipLaunchKernelGGL(zero_words_kernel, dim3(16), dim3(256), 0, (hipStream_t)stream,
+                       (uint32_t *)workspace, (uint32_t)(FTC_WORKSPACE_CONTROL_BYTES / 4));
+    const hipError_t err = hipGetLastError();
+    if (err != hipSuccess)
+        return fail(FTC_ERR_HIP, "workspace reset launch failed: %s", hipGetErrorString(err));
+    return FTC_OK;
+}
+
 int ftc_causal_dot_product_static(const ftc_tensor4 *queries, const ftc_tensor4 *keys,
                                   const ftc_tensor4 *values, const ftc_tensor4 *product,
                                   void *stream) {

@@ -169,10 +169,16 @@ int mfma_scan(const ScanDesc *scans, int nscans, int64_t N, int64_t H, int64_t L
         ScanOperands &o = args.scan[i];
         o.a = sd.a.ptr, o.b = sd.b.ptr, o.v = sd.v.ptr;
         o.out = sd.out.ptr;
-        o.a_sn = sd.a.stride_n, o.a_sh = sd.a.stride_h, o.a_sl = sd.a.stride_l;
-        o.b_sn = sd.b.stride_n, o.b_sh = sd.b.stride_h, o.b_sl = sd.b.stride_l;
-        o.v_sn = sd.v.stride_n, o.v_sh = sd.v.stride_h, o.v_sl = sd.v.stride_l;
-        o.o_sn = sd.out.stride_n, o.o_sh = sd.out.stride_h, o.o_sl = sd.out.stride_l;
+        // With a single position the row stride addresses nothing, but the kernels still
+        // step over the 31 absent rows of the chunk with it: those must fall outside the
+        // one-row descriptor, so a stride below the row width is replaced by the width.
+        auto row_stride = [L](int64_t stride_l, int width) {
+            return L == 1 ? std::max<int64_t>(stride_l, width) : stride_l;
+        };
+        o.a_sn = sd.a.stride_n, o.a_sh = sd.a.stride_h, o.a_sl = row_stride(sd.a.stride_l, D);
+        o.b_sn = sd.b.stride_n, o.b_sh = sd.b.stride_h, o.b_sl = row_stride(sd.b.stride_l, D);
+        o.v_sn = sd.v.stride_n, o.v_sh = sd.v.stride_h, o.v_sl = row_stride(sd.v.stride_l, F);
+        o.o_sn = sd.out.stride_n, o.o_sh = sd.out.stride_h, o.o_sl = row_stride(sd.out.stride_l, F);
         o.rev = sd.reverse ? 1 : 0;
         o.pad = 0;
         o.s0 = sd.initial.ptr;
@@ -200,6 +206,9 @@ int mfma_scan(const ScanDesc *scans, int nscans, int64_t N, int64_t H, int64_t L
     }
     // tuning aid: FTC_GROUP=<n> forces groups of n steps
     if (const char *env = getenv("FTC_GROUP")) args.group = std::max(1, atoi(env));
+    // a wavefront watches one flag per lane: at most 64 steps per group and 64 groups
+    args.group = std::min(args.group, 64);
+    while ((pl.nseg + args.group - 1) / args.group > 64) args.group++;
 
     for (int i = 1; i < nscans; i++)
         if (combo_of(scans[i]) != combo || scans[i].a.width != D || scans[i].v.width != F)

@@ -339,6 +339,9 @@ struct StateExchange {
             if (++spins > kSpinLimit) failed = true;
             __builtin_amdgcn_s_sleep(4);
         }
+        // the states behind these flags are read with plain buffer loads: keep the compiler
+        // from moving any of them above the wait
+        asm volatile("" ::: "memory");
     }
 
     // after pass 1: make this step's own sum visible to the later steps of its group

@@ -21,6 +21,7 @@ _DTYPE_CODE = {torch.float32: FTC_F32, torch.bfloat16: FTC_BF16}
 EXPORTED_SYMBOLS = (
     "ftc_version",
     "ftc_last_error",
+    "ftc_workspace_reset",
     "ftc_causal_dot_product_workspace_bytes",
     "ftc_causal_dot_product",
     "ftc_causal_dot_product_static",
@@ -63,6 +64,8 @@ def load():
         f = getattr(lib, name)
         f.restype = ctypes.c_int64
         f.argtypes = [ctypes.c_int64] * 5 + [ctypes.c_int32]
+    lib.ftc_workspace_reset.restype = ctypes.c_int
+    lib.ftc_workspace_reset.argtypes = [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]
     lib.ftc_causal_dot_product.restype = ctypes.c_int
     lib.ftc_causal_dot_product.argtypes = [t4] * 4 + [ctypes.c_void_p, ctypes.c_size_t,
                                                       ctypes.c_void_p]

@@ -70,6 +70,26 @@ def workspace_error_words():
     return {key: int(ws[8:12].view(torch.int32).item()) for key, ws in _workspaces.items()}
 
 
+def check_workspaces():
+    """Synchronise and raise if any cached workspace reports that a call was cut short.  The
+    control block of such a workspace is cleared first (``ftc_workspace_reset``), so calls
+    made after the exception start from a clean workspace again: a control block left
+    non-zero would make every later call on it stop early with its outputs unwritten."""
+    bad = {key: word for key, word in workspace_error_words().items() if word != 0}
+    if not bad:
+        return
+    lib = _native.load()
+    for (device_index, stream) in bad:
+        ws = _workspaces[(device_index, stream)]
+        with torch.cuda.device(device_index):
+            _native.check(lib.ftc_workspace_reset(ws.data_ptr(), ws.numel(), stream),
+                          "ftc_workspace_reset")
+    torch.cuda.synchronize()
+    raise RuntimeError("causal_dot_product: a call was cut short on workspace(s) %s "
+                       "(error words %s); its outputs are not valid.  The workspaces have "
+                       "been reset." % (sorted(bad), [bad[k] for k in sorted(bad)]))
+
+
 def causal_dot_product_hip(queries, keys, values, product):
     """In-place forward; replaces the reference's native ``causal_dot_product``
     (``causal_product_cuda.cu:1273-1285``).  Enqueued on the current stream."""

@@ -73,6 +73,15 @@ int ftc_version(void);
 /* Message of the last failing call on this thread ("" if none). */
 const char *ftc_last_error(void);
 
+/*
+ * Clears the control block of a workspace (a fill kernel enqueued on `stream`; no memset, so
+ * it may be captured in a graph).  No counterpart in the reference.  A workspace needs this
+ * once before its first use unless it was allocated zero-filled, and again after a call whose
+ * work was cut short (error word non-zero, see above): a control block that is not zero makes
+ * every later call on that workspace stop early.
+ */
+int ftc_workspace_reset(void *workspace, size_t workspace_bytes, void *stream);
+
 /* Scratch bytes ftc_causal_dot_product needs for these sizes (>= 0), or a negative ftc_status. */
 int64_t ftc_causal_dot_product_workspace_bytes(int64_t N, int64_t H, int64_t L, int64_t E,
                                                int64_t M, int32_t dtype);
@@ -93,8 +102,10 @@ int ftc_causal_dot_product(const ftc_tensor4 *queries, const ftc_tensor4 *keys,
  * hipMalloc.  It has no counterpart in the reference.  Same arguments and result as
  * ftc_causal_dot_product, without the workspace: the scratch memory is an array of
  * FTC_STATIC_SCRATCH_BYTES that is part of the library's device code (each GPU the library
- * runs on holds one until the process ends).  The call allocates and frees nothing and
- * enqueues kernels only.  Sizes whose scratch need
+ * runs on holds one until the process ends; the HIP runtime places it when the first call
+ * on a device loads that part of the library's device code, so make one call before
+ * starting a graph capture).  The call itself allocates and frees nothing and enqueues
+ * kernels only.  Sizes whose scratch need
  * (ftc_causal_dot_product_workspace_bytes) exceeds the array are refused with
  * FTC_ERR_WORKSPACE.  All calls on one GPU share that GPU's array: two calls whose work
  * overlaps in time on one GPU (different streams, different threads) race; calls on one

@@ -118,57 +118,202 @@ CONFIG_SHAPES = {
 }
 
 
+def _gate_against_float64(tag, got, want, exact):
+    """Two correct fp32 summation orders differ near the zero crossings of the output, so the
+    element-wise test 1e-5 + 1e-4 |b| cannot hold everywhere -- not even for the reference's
+    own order against float64.  The gate: per-chain scale error <= 1e-4; no further from
+    float64 than the checker is (factor 4 on the scale error); the fraction of elements
+    outside the element-wise bound, measured against float64, at most twice the checker's own
+    fraction on the same inputs; and the same fraction measured against the checker (where
+    both orders' errors add up) likewise; 0.06 % is added to both bounds for the near-empty
+    counts of short sequences (a few dozen elements)."""
+    s, v = report(tag, got, want)
+    v_ref, v_hip = violation_fraction(want, exact), violation_fraction(got, exact)
+    s_hip, s_cpu = scale_error(got, exact), scale_error(want, exact)
+    print("    vs float64: hip %.3e  cpu %.3e ; outside: hip-vs-cpu %.4f%%  hip-vs-float64 %.4f%%"
+          "  cpu-vs-float64 %.4f%%" % (s_hip, s_cpu, 100 * v, 100 * v_hip, 100 * v_ref), flush=True)
+    assert s <= 1e-4, tag
+    assert s_hip <= max(4 * s_cpu, 2e-6), tag
+    assert v_hip <= 2 * v_ref + 6e-4, tag
+    assert v <= 2 * v_ref + 6e-4, tag
+
+
 @pytest.mark.parametrize("name", sorted(CONFIG_SHAPES))
 def test_configs_against_cpu_checker(cp, name):
     N, H, L, E, M, seed = CONFIG_SHAPES[name]
     print("config", name, (N, H, L, E, M), flush=True)
     Q, K, V, G = oracle.make_inputs(N, H, L, E, M, seed)
+    Qd, Kd, Vd, Gd = (t.double() for t in (Q, K, V, G))
     want = oracle.forward(Q, K, V)
     out = hip_forward(cp, Q, K, V)
     assert torch.isfinite(out).all()
-    s, v = report(name + " product", out, want)
-    assert s <= 1e-4 and v <= 0.02
-    # neither fp32 order is exact: the HIP result must be as close to float64 as the checker
-    if N * H * L <= 200000:
-        exact = oracle.forward(Q.double(), K.double(), V.double())
-        s_hip, s_cpu = scale_error(out, exact), scale_error(want, exact)
-        print("    vs float64: hip %.3e  cpu %.3e" % (s_hip, s_cpu), flush=True)
-        assert s_hip <= max(4 * s_cpu, 2e-6)
+    _gate_against_float64(name + " product", out, want, oracle.forward(Qd, Kd, Vd))
     grads = hip_backward(cp, Q, K, V, G)
-    for key, got, ref in zip(("dQ", "dK", "dV"), grads, oracle.backward(Q, K, V, G)):
+    exact = oracle.backward(Qd, Kd, Vd, Gd)
+    for key, got, ref, ex in zip(("dQ", "dK", "dV"), grads, oracle.backward(Q, K, V, G), exact):
         assert torch.isfinite(got).all(), key
-        s, v = report(name + " " + key, got, ref)
-        assert s <= 1e-4 and v <= 0.02, key
+        _gate_against_float64(name + " " + key, got, ref, ex)
+
+
+def _linear_in(fn, X1, X2, coeff=0.37):
+    """fn(X1 + coeff X2) against fn(X1) + coeff fn(X2), as per-chain scale errors per output."""
+    combo = [t.cpu() for t in fn(X1 + coeff * X2)]
+    parts = [a.cpu() + coeff * b.cpu() for a, b in zip(fn(X1), fn(X2))]
+    return [scale_error(c, p) for c, p in zip(combo, parts)]
 
 
 def test_full_config3_size_properties(cp):
-    """N=1, H=16, L=65536 at full size: prefix property, linearity in V, and two heads
-    against the CPU checker."""
+    """N=1, H=16, L=65536 at full size.  Forward: prefix property, linearity in V, two heads
+    against the CPU checker.  Backward, over all 16 heads: linearity in G of all three
+    gradients (a combination that is not a power of two), the time-reversal identity
+    dK = flip(product(flip V, flip G, flip Q)) evaluated with the HIP forward, the prefix
+    property of dQ, and two heads against the checker."""
     N, H, L, E, M = 1, 16, 65536, 64, 64
     Q, K, V, G = oracle.make_inputs(N, H, L, E, M, seed=3)
-    Qd, Kd, Vd = Q.cuda(), K.cuda(), V.cuda()
-    out = torch.empty(N, H, L, M, device="cuda")
-    cp.causal_dot_product_hip(Qd, Kd, Vd, out)
+    Qd, Kd, Vd, Gd = Q.cuda(), K.cuda(), V.cuda(), G.cuda()
+
+    def fwd(q, k, v):
+        o = torch.empty(q.shape[:3] + (v.shape[3],), device="cuda")
+        cp.causal_dot_product_hip(q, k, v, o)
+        return o
+
+    def bwd(g, q=Qd, k=Kd, v=Vd):
+        outs = [torch.empty_like(t) for t in (q, k, v)]
+        cp.causal_dot_backward_hip(q, k, v, g, *outs)
+        return outs
+
+    out = fwd(Qd, Kd, Vd)
     # prefix property: a truncated sequence gives the same rows
     Lp = L // 2 + 13
-    outp = torch.empty(N, H, Lp, M, device="cuda")
-    cp.causal_dot_product_hip(Qd[:, :, :Lp], Kd[:, :, :Lp], Vd[:, :, :Lp], outp)
+    outp = fwd(Qd[:, :, :Lp], Kd[:, :, :Lp], Vd[:, :, :Lp])
     assert scale_error(outp.cpu(), out[:, :, :Lp].cpu()) <= 1e-5
     # linearity in V
-    out2 = torch.empty_like(out)
-    cp.causal_dot_product_hip(Qd, Kd, 2.0 * Vd, out2)
-    assert scale_error(out2.cpu(), (2.0 * out).cpu()) <= 1e-6
+    V2 = torch.randn(N, H, L, M, generator=torch.Generator().manual_seed(33)).cuda()
+    (err,) = _linear_in(lambda v: [fwd(Qd, Kd, v)], Vd, V2)
+    print("cfg3 product linear in V: %.3e" % err, flush=True)
+    assert err <= 2e-5
     want = oracle.forward(Q[:, 5:7].contiguous(), K[:, 5:7].contiguous(), V[:, 5:7].contiguous())
     s, _ = report("cfg3 heads 5-6", out[:, 5:7].cpu(), want)
     assert s <= 1e-4
-    # backward: dV is linear in G, and two heads against the checker
-    grads = [torch.empty_like(t) for t in (Qd, Kd, Vd)]
-    cp.causal_dot_backward_hip(Qd, Kd, Vd, G.cuda(), *grads)
+
+    grads = bwd(Gd)
+    # all three gradients are linear in G
+    G2 = torch.randn(N, H, L, M, generator=torch.Generator().manual_seed(34)).cuda()
+    errs = _linear_in(bwd, Gd, G2)
+    print("cfg3 dQ, dK, dV linear in G: %.3e %.3e %.3e" % tuple(errs), flush=True)
+    assert max(errs) <= 2e-5
+    # time reversal: dK_l = sum_{j>=l} (v_l . g_j) q_j is a forward product of the flipped rows
+    flip = lambda t: torch.flip(t, dims=[2]).contiguous()
+    dK_rev = flip(fwd(flip(Vd), flip(Gd), flip(Qd)))
+    s = scale_error(grads[1].cpu(), dK_rev.cpu())
+    print("cfg3 dK against flipped forward: %.3e" % s, flush=True)
+    assert s <= 2e-5
+    dV_rev = flip(fwd(flip(Kd), flip(Qd), flip(Gd)))
+    assert scale_error(grads[2].cpu(), dV_rev.cpu()) <= 2e-5
+    # dQ is itself a forward product, of (G, V, K)
+    assert scale_error(grads[0].cpu(), fwd(Gd, Vd, Kd).cpu()) <= 2e-5
+    # prefix property of dQ (dK and dV of a truncated sequence differ: they sum over j >= l)
+    gp = bwd(Gd[:, :, :Lp].contiguous(), Qd[:, :, :Lp], Kd[:, :, :Lp], Vd[:, :, :Lp])
+    assert scale_error(gp[0].cpu(), grads[0][:, :, :Lp].cpu()) <= 1e-5
     sl = slice(5, 7)
     refs = oracle.backward(Q[:, sl].contiguous(), K[:, sl].contiguous(), V[:, sl].contiguous(),
                            G[:, sl].contiguous())
     for key, got, ref in zip(("dQ", "dK", "dV"), grads, refs):
         s, _ = report("cfg3 heads 5-6 " + key, got[:, sl].cpu(), ref)
+        assert s <= 1e-4, key
+
+
+def test_full_config5_size_properties(cp):
+    """Config 5 at full size: bf16 Q, K, V, N=4, H=32, L=16384, E=32, M=128 (128 chains of 512
+    chunks, two-level state exchange, three backward launches).  Properties over all chains
+    plus two chains against the CPU checker on the same rounded inputs (2e-2 bar)."""
+    N, H, L, E, M = 4, 32, 16384, 32, 128
+    Q, K, V, G = oracle.make_inputs(N, H, L, E, M, seed=5)
+    Qb, Kb, Vb = (t.bfloat16().cuda() for t in (Q, K, V))
+    Gd = G.cuda()
+
+    def fwd(q, k, v):
+        o = torch.empty(q.shape[:3] + (v.shape[3],), device="cuda")
+        cp.causal_dot_product_hip(q, k, v, o)
+        return o
+
+    def bwd(g, q=Qb, k=Kb, v=Vb):
+        outs = [torch.empty_like(t) for t in (q, k, v)]
+        cp.causal_dot_backward_hip(q, k, v, g, *outs)
+        return [t.float() for t in outs]
+
+    out = fwd(Qb, Kb, Vb)
+    assert out.dtype == torch.float32 and torch.isfinite(out).all()
+    Lp = L // 2 + 13
+    outp = fwd(Qb[:, :, :Lp], Kb[:, :, :Lp], Vb[:, :, :Lp])
+    assert scale_error(outp.cpu(), out[:, :, :Lp].cpu()) <= 1e-5
+    # linearity in V: the combination is formed in float32 and rounded to bf16 once more, so
+    # the bar is bf16 rounding of the values (2^-8 relative to the largest product)
+    V2 = torch.randn(N, H, L, M, generator=torch.Generator().manual_seed(55)).bfloat16().cuda()
+    Vc = (Vb.float() + 0.5 * V2.float())  # exact in float32; 0.5 keeps bf16 sums exact enough
+    o12 = fwd(Qb, Kb, Vc.bfloat16())
+    o1, o2 = fwd(Qb, Kb, Vb), fwd(Qb, Kb, V2)
+    err = scale_error(o12.cpu(), (o1 + 0.5 * o2).cpu())
+    print("cfg5 product linear in V (bf16 values): %.3e" % err, flush=True)
+    assert err <= 2 ** -7
+    grads = bwd(Gd)
+    G2 = torch.randn(N, H, L, M, generator=torch.Generator().manual_seed(56)).cuda()
+    errs = _linear_in(bwd, Gd, G2)   # G is float32: exact combination, bf16-rounded results
+    print("cfg5 dQ, dK, dV linear in G: %.3e %.3e %.3e" % tuple(errs), flush=True)
+    assert max(errs) <= 2 ** -7
+    # two chains against the checker on the rounded inputs
+    sl = (slice(1, 2), slice(7, 9))
+    cut = lambda t: t[sl].float().cpu().contiguous()
+    want = oracle.forward(cut(Qb), cut(Kb), cut(Vb))
+    s, _ = report("cfg5 chains (1,7-8) product", out[sl].cpu(), want)
+    assert s <= 2e-2 and s <= 1e-5
+    refs = oracle.backward(cut(Qb), cut(Kb), cut(Vb), cut(Gd))
+    for key, got, ref in zip(("dQ", "dK", "dV"), grads, refs):
+        s, _ = report("cfg5 chains (1,7-8) " + key, got[sl].cpu(), ref)
+        assert s <= 2e-2, key
+
+
+def test_config4_operator_shape_through_nlhe_strides(cp):
+    """The operator as the config-4 encoder calls it: N=10, H=8, L=4096, E=M=64, with Q, K, V
+    and the product living in (N, L, H, X) storage and seen as (N, H, L, X) views.  Prefix
+    property and linearity over all chains, two chains against the CPU checker, forward and
+    backward."""
+    N, H, L, E, M = 10, 8, 4096, 64, 64
+    Q, K, V, G = oracle.make_inputs(N, H, L, E, M, seed=4)
+    nlhe = lambda t: t.cuda().permute(0, 2, 1, 3).contiguous().permute(0, 2, 1, 3)
+    Qd, Kd, Vd, Gd = (nlhe(t) for t in (Q, K, V, G))
+    assert not Qd.is_contiguous() and Qd.stride(2) == H * E
+
+    def fwd(q, k, v):
+        o = torch.empty(N, q.shape[2], H, M, device="cuda").permute(0, 2, 1, 3)
+        cp.causal_dot_product_hip(q, k, v, o)
+        return o
+
+    def bwd(g):
+        outs = [torch.empty(N, L, H, X, device="cuda").permute(0, 2, 1, 3) for X in (E, E, M)]
+        cp.causal_dot_backward_hip(Qd, Kd, Vd, g, *outs)
+        return outs
+
+    out = fwd(Qd, Kd, Vd)
+    Lp = L // 2 + 13
+    outp = fwd(Qd[:, :, :Lp], Kd[:, :, :Lp], Vd[:, :, :Lp])
+    assert scale_error(outp.cpu(), out[:, :, :Lp].cpu()) <= 1e-5
+    V2 = nlhe(torch.randn(N, H, L, M, generator=torch.Generator().manual_seed(44)))
+    (err,) = _linear_in(lambda v: [fwd(Qd, Kd, v)], Vd, V2)
+    assert err <= 2e-5
+    grads = bwd(Gd)
+    G2 = nlhe(torch.randn(N, H, L, M, generator=torch.Generator().manual_seed(45)))
+    errs = _linear_in(bwd, Gd, G2)
+    print("cfg4op dQ, dK, dV linear in G: %.3e %.3e %.3e" % tuple(errs), flush=True)
+    assert max(errs) <= 2e-5
+    sl = (slice(3, 4), slice(2, 4))
+    cut = lambda t: t[sl].cpu().contiguous()
+    want = oracle.forward(cut(Q), cut(K), cut(V))
+    s, _ = report("cfg4op chains (3,2-3) product", out[sl].cpu(), want)
+    assert s <= 1e-4
+    for key, got, ref in zip(("dQ", "dK", "dV"), grads,
+                             oracle.backward(cut(Q), cut(K), cut(V), cut(G))):
+        s, _ = report("cfg4op chains (3,2-3) " + key, got[sl].cpu(), ref)
         assert s <= 1e-4, key
 
 
@@ -477,6 +622,30 @@ def test_zz_no_wavefront_gave_up_waiting(cp):
     words = cp.workspace_error_words()
     assert words, "no workspace was used: the MFMA path did not run"
     assert all(w == 0 for w in words.values()), words
+
+
+def test_dirty_control_block_is_reported_and_healed(cp):
+    """A control block that is not zero when a call starts (here: a ticket counter set from
+    the host) makes the wavefronts of that chain stop early; every kernel still ends
+    normally.  check_workspaces() reports it and resets the workspace, after which calls work
+    again."""
+    N, H, L, E, M = 2, 2, 1500, 64, 64
+    Q, K, V, _ = oracle.make_inputs(N, H, L, E, M, seed=77)
+    want = oracle.forward(Q, K, V)
+    out = hip_forward(cp, Q, K, V)     # makes sure a workspace exists
+    assert scale_error(out, want) <= 1e-4
+    key, ws = next(iter(cp._workspaces.items()))
+    control_words = 65536 // 4
+    max_waves = (control_words - 64) // 2
+    ws.view(torch.int32)[64 + max_waves] = 1000   # ticket counter of the first chain
+    torch.cuda.synchronize()
+    hip_forward(cp, Q, K, V)
+    with pytest.raises(RuntimeError, match="cut short"):
+        cp.check_workspaces()
+    assert all(w == 0 for w in cp.workspace_error_words().values())
+    out = hip_forward(cp, Q, K, V)
+    assert scale_error(out, want) <= 1e-4
+    cp.check_workspaces()
 
 
 def test_errors_and_empty_inputs(cp):

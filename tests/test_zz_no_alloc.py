@@ -16,7 +16,7 @@ from parity import scale_error
 pytestmark = pytest.mark.gpu
 
 
-def _call_pair(lib, native, shape, seed, dtype=torch.float32):
+def _call_pair(lib, native, shape, seed, dtype=torch.float32, check_memory=True):
     N, H, L, E, M = shape
     Q, K, V, _ = oracle.make_inputs(N, H, L, E, M, seed)
     Qd, Kd, Vd = (t.to(dtype).cuda() for t in (Q, K, V))
@@ -35,11 +35,16 @@ def _call_pair(lib, native, shape, seed, dtype=torch.float32):
     # the entry point under test: outputs are allocated before the call, nothing inside it
     got = torch.full((N, H, L, M), float("nan"), device="cuda")
     torch.cuda.synchronize()
-    before = torch.cuda.memory_allocated()
+    # device memory as the driver sees it (not torch's cache): a hipMalloc inside the call,
+    # by the library or anything it uses, would lower the free amount
+    free_before, _ = torch.cuda.mem_get_info()
+    allocs_before = torch.cuda.memory_stats().get("allocation.all.allocated", 0)
     native.check(lib.ftc_causal_dot_product_static(*descs, native.describe(got), stream),
                  "ftc_causal_dot_product_static")
     torch.cuda.synchronize()
-    assert torch.cuda.memory_allocated() == before
+    if check_memory:
+        assert torch.cuda.mem_get_info()[0] >= free_before
+        assert torch.cuda.memory_stats().get("allocation.all.allocated", 0) == allocs_before
     return Q, K, V, got.cpu(), want.cpu(), nbytes
 
 
@@ -54,6 +59,9 @@ def test_static_scratch_entry_point_matches_workspace_entry_point():
               ((2, 3, 333, 64, 64), 32, torch.float32),
               ((2, 4, 2048, 32, 128), 33, torch.bfloat16),
               ((2, 2, 700, 25, 40), 34, torch.float32)]
+    # set-up: the first call on a device makes the HIP runtime load the part of the library's
+    # device code that holds the scratch array; later calls touch no allocator at all
+    _call_pair(lib, native, (1, 2, 200, 64, 64), 30, check_memory=False)
     for shape, seed, dtype in shapes:
         print("static scratch", shape, dtype, flush=True)
         Q, K, V, got, want, nbytes = _call_pair(lib, native, shape, seed, dtype)
