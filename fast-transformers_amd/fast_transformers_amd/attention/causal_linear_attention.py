@@ -1,7 +1,7 @@
 """Causally masked linear attention on top of the MI355X ``causal_dot_product``.
 
 Own counterpart of ``fast_transformers/attention/causal_linear_attention.py:19-104``: same
-constructor arguments, same ``forward(queries, keys, values, attn_mask, query_lengths,
+constructor arguments (feature-map factory, ``eps``, ``event_dispatcher``), same ``forward(queries, keys, values, attn_mask, query_lengths,
 key_lengths)`` over ``(N, L, H, E)`` tensors, same equations (feature map ``elu(x)+1``
 ``feature_maps/base.py:71-73``; key-length masking ``:83``; normaliser
 ``Z = 1 / (q . cumsum(k) + eps)`` ``:95``; result ``V' * Z`` ``:104``).
@@ -20,9 +20,42 @@ from torch.nn import Module
 from ..causal_product import causal_dot_product_hip, causal_dot_backward_hip
 
 
-def elu_feature_map(x):
-    """phi(x) = elu(x) + 1 (``feature_maps/base.py:71-73``)."""
+class ActivationFunctionFeatureMap(Module):
+    """An element-wise feature map behind the reference's feature-map protocol
+    (``feature_maps/base.py:19-73``): attention modules receive a *factory* that is called
+    with the query dimensions and returns an object with ``new_feature_map(device)``,
+    ``forward_queries(x)`` and ``forward_keys(x)``."""
+
+    def __init__(self, query_dims, activation_function):
+        super().__init__()
+        self.query_dims = query_dims
+        self.activation_function = activation_function
+
+    def new_feature_map(self, device):
+        return
+
+    def forward_queries(self, x):
+        return self(x)
+
+    def forward_keys(self, x):
+        return self(x)
+
+    def forward(self, x):
+        return self.activation_function(x)
+
+    @classmethod
+    def factory(cls, *args, **kwargs):
+        def inner(query_dims):
+            return cls(query_dims, *args, **kwargs)
+        return inner
+
+
+def _elu_plus_one(x):
     return torch.nn.functional.elu(x) + 1
+
+
+# phi(x) = elu(x) + 1 as a feature-map factory (``feature_maps/base.py:71-73``)
+elu_feature_map = ActivationFunctionFeatureMap.factory(_elu_plus_one)
 
 
 class _CausalLinearNLH(torch.autograd.Function):
@@ -75,15 +108,20 @@ def causal_linear(Q, K, V):
 class CausalLinearAttention(Module):
     """Causally masked attention with feature maps in O(L D^2) (reference ``:27-104``).
 
-    Arguments: ``query_dimensions`` (kept for signature compatibility), ``feature_map`` (a
-    callable applied to queries and keys, default ``elu(x)+1``), ``eps`` (default 1e-6).
+    Arguments as in the reference (``:47-55``): ``query_dimensions``; ``feature_map``, a
+    factory called with the query dimensions that returns a feature map object (default
+    ``elu_feature_map``; any factory of the reference's ``feature_maps`` package fits);
+    ``eps`` (default 1e-6); ``event_dispatcher``, accepted and kept for signature
+    compatibility (the reference stores a dispatcher here and never dispatches through it,
+    ``:55``).
     """
 
-    def __init__(self, query_dimensions, feature_map=None, eps=1e-6):
+    def __init__(self, query_dimensions, feature_map=None, eps=1e-6, event_dispatcher=""):
         super().__init__()
-        self.query_dimensions = query_dimensions
-        self.feature_map = feature_map or elu_feature_map
+        self.feature_map = (feature_map(query_dimensions) if feature_map
+                            else elu_feature_map(query_dimensions))
         self.eps = eps
+        self.event_dispatcher = event_dispatcher
 
     @staticmethod
     def _make_sizes_compatible(Q, K, V):
@@ -101,8 +139,9 @@ class CausalLinearAttention(Module):
                 torch.cat([V, V.new_zeros(N, L - S, H, M)], dim=1))
 
     def forward(self, queries, keys, values, attn_mask, query_lengths, key_lengths):
-        Q = self.feature_map(queries)
-        K = self.feature_map(keys)
+        self.feature_map.new_feature_map(queries.device)
+        Q = self.feature_map.forward_queries(queries)
+        K = self.feature_map.forward_keys(keys)
         if not attn_mask.lower_triangular:
             raise RuntimeError("CausalLinearAttention only supports full lower triangular masks")
         K = K * key_lengths.float_matrix[:, :, None, None]

@@ -4,9 +4,9 @@
 * ``CausalDotProduct`` is a ``torch.autograd.Function`` with the class-level
   dispatch tables ``dot`` / ``dot_backward`` keyed by ``device.type``
   (reference ``__init__.py:23-30``).  ROCm PyTorch reports ``"cuda"`` for an AMD
-  GPU, so the HIP kernels register under that key.  There is no ``"cpu"`` entry:
-  this package ships the GPU path only and a CPU tensor raises ``KeyError`` the
-  way an unknown device type does in the reference (``__init__.py:44``).
+  GPU, so the HIP kernels register under that key.  The ``"cpu"`` entry is a small
+  chunked implementation of its own for CPU tensors (plain torch matmuls); the GPU entry
+  never falls back to it: without the HIP library a GPU tensor raises.
 * The native functions keep the reference's in-place calling convention
   (``causal_product_cpu.cpp:82-87,133-141``): ``causal_dot_product(Q, K, V,
   product)`` and ``causal_dot_backward(Q, K, V, grad_out, grad_Q, grad_K,
@@ -177,13 +177,59 @@ def causal_dot_backward_hip(queries, keys, values, grad_out, grad_queries, grad_
     _native.check(rc, "ftc_causal_dot_backward")
 
 
+def _cpu_args(name, *tensors):
+    for t in tensors:
+        if t.dim() != 4 or t.device.type != "cpu":
+            raise RuntimeError("%s: expected 4-dimensional CPU tensors" % name)
+
+
+def _cpu_scan(a, b, v, out, reverse, chunk=128):
+    """out[l] = sum_{j<=l} (a_l . b_j) v_j on CPU tensors (reverse: j >= l), chunked along L:
+    a running (D, F) state plus the masked product inside a chunk, float32 accumulation,
+    written into ``out`` in place.  This is the package's own host path for CPU tensors (the
+    reference keeps a ``"cpu"`` entry next to ``"cuda"``, ``__init__.py:23-30``); it shares
+    nothing with the GPU path and is not a fallback for it."""
+    N, H, L, D = a.shape
+    state = a.new_zeros((N, H, D, v.shape[3]), dtype=torch.float32)
+    starts = list(range(0, L, chunk))
+    for lo in (reversed(starts) if reverse else starts):
+        hi = min(L, lo + chunk)
+        ac, bc, vc = (t[:, :, lo:hi].float() for t in (a, b, v))
+        p = torch.matmul(ac, bc.transpose(2, 3))
+        p = torch.triu(p) if reverse else torch.tril(p)
+        out[:, :, lo:hi] = (torch.matmul(p, vc) + torch.matmul(ac, state)).to(out.dtype)
+        state = state + torch.matmul(bc.transpose(2, 3), vc)
+
+
+def causal_dot_product_cpu(queries, keys, values, product):
+    """In-place forward for CPU tensors, the reference's native signature
+    (``causal_product_cpu.cpp:82-87``)."""
+    _cpu_args("causal_dot_product", queries, keys, values, product)
+    _cpu_scan(queries, keys, values, product, False)
+
+
+def causal_dot_backward_cpu(queries, keys, values, grad_out, grad_queries, grad_keys,
+                            grad_values):
+    """In-place backward for CPU tensors (``causal_product_cpu.cpp:133-141``): the three
+    gradients are the same scan under a change of roles."""
+    _cpu_args("causal_dot_backward", queries, keys, values, grad_out)
+    if grad_queries is not None:
+        _cpu_scan(grad_out, values, keys, grad_queries, False)
+    if grad_keys is not None:
+        _cpu_scan(values, grad_out, queries, grad_keys, True)
+    if grad_values is not None:
+        _cpu_scan(keys, queries, grad_out, grad_values, True)
+
+
 class CausalDotProduct(torch.autograd.Function):
     """Compute the weighted sum of values but attending only to previous values
     (reference ``__init__.py:20-74``)."""
     dot = {
+        "cpu": causal_dot_product_cpu,
         "cuda": causal_dot_product_hip,
     }
     dot_backward = {
+        "cpu": causal_dot_backward_cpu,
         "cuda": causal_dot_backward_hip,
     }
 

@@ -63,8 +63,22 @@ def test_python_surface_matches_reference_module():
     from fast_transformers_amd import causal_product as cp
     import torch
     assert issubclass(cp.CausalDotProduct, torch.autograd.Function)
-    assert set(cp.CausalDotProduct.dot) == set(cp.CausalDotProduct.dot_backward) == {"cuda"}
+    assert set(cp.CausalDotProduct.dot) == set(cp.CausalDotProduct.dot_backward) == {"cpu", "cuda"}
     assert callable(cp.causal_dot_product)
-    Q = torch.zeros(1, 1, 2, 2)
-    with pytest.raises(KeyError):  # no CPU path is shipped
-        cp.causal_dot_product(Q, Q, Q)
+
+
+def test_cpu_entry_matches_the_checker():
+    """CPU tensors take the package's own host implementation (the reference keeps a "cpu"
+    entry beside "cuda", causal_product/__init__.py:23-30); checked against the CPU checker
+    and through autograd."""
+    import torch
+    import oracle
+    from parity import scale_error
+    from fast_transformers_amd import causal_product as cp
+    Q, K, V, G = oracle.make_inputs(2, 3, 300, 20, 24, seed=5)
+    Qg, Kg, Vg = (t.clone().requires_grad_(True) for t in (Q, K, V))
+    out = cp.causal_dot_product(Qg, Kg, Vg)
+    (out * G).sum().backward()
+    assert scale_error(out.detach(), oracle.forward(Q, K, V)) <= 1e-5
+    for got, ref in zip((Qg.grad, Kg.grad, Vg.grad), oracle.backward(Q, K, V, G)):
+        assert scale_error(got, ref) <= 1e-5

@@ -5,8 +5,15 @@ Checked against (a) the CPU checker through the (N, L, H, X) entry without layou
 (tests/causal_product/test_causal_product.py:34-40), (c) the step-wise recurrent form the
 reference tests batch attention against
 (tests/recurrent/attention/self_attention/test_linear_attention.py:54-79, bound 1e-5), and
-(d) the same encoder with a dense pure-torch inner attention.
+(d) the same encoder with a dense pure-torch inner attention, and (e) the outputs of a
+builder-made reference encoder on its own weights (tests/golden/encoder_causal_linear.npz,
+written by tests/golden/make_encoder_golden.py from the reference's modules), which pins the
+block structure: projections, head split, residual and post-norm order, feed-forward, final
+norm, parameter names.
 """
+import os
+
+import numpy as np
 import pytest
 import torch
 
@@ -40,6 +47,11 @@ def test_causal_linear_on_nlh_layout_matches_checker(att):
         assert scale_error(got.cpu().permute(0, 2, 1, 3), ref) <= 1e-5
 
 
+def _phi(x):
+    """elu(x) + 1 (feature_maps/base.py:71-73)"""
+    return torch.nn.functional.elu(x) + 1
+
+
 def dense_attention(phi, q, k, v, key_lengths, eps):
     """phi(q) phi(k)^T masked to j <= i and to valid keys, row-normalised, times v; float64."""
     Q, K, V = phi(q.double()), phi(k.double()), v.double()
@@ -61,7 +73,7 @@ def test_module_against_dense_normalised_attention(att):
     layer = att.CausalLinearAttention(E)
     out = layer(q, k, v, m.TriangularCausalMask(L, device="cuda"), lengths, lengths)
     assert out.shape == (N, L, H, M) and out.is_contiguous()
-    want = dense_attention(att.elu_feature_map, q, k, v, lengths, 1e-6)
+    want = dense_attention(_phi, q, k, v, lengths, 1e-6)
     assert (out.double() - want).abs().max().item() < 1e-5
     with pytest.raises(RuntimeError):
         layer(q, k, v, m.FullMask(L, device="cuda"), lengths, lengths)
@@ -70,13 +82,13 @@ def test_module_against_dense_normalised_attention(att):
     klen = m.LengthMask(torch.full((N,), S).cuda(), max_len=S)
     sliced = layer(q[:, :70], k[:, :S], v[:, :S], m.TriangularCausalMask(70, device="cuda"),
                    klen, klen)
-    want70 = dense_attention(att.elu_feature_map, q[:, :70], k[:, :70], v[:, :70],
+    want70 = dense_attention(_phi, q[:, :70], k[:, :70], v[:, :70],
                              m.LengthMask(torch.full((N,), 70).cuda(), max_len=70), 1e-6)
     assert (sliced.double() - want70).abs().max().item() < 1e-5
     padded = layer(q, k[:, :S], v[:, :S], m.TriangularCausalMask(L, device="cuda"), klen, klen)
     assert padded.shape == (N, L, H, M)
     assert (padded[:, :S].double() - dense_attention(
-        att.elu_feature_map, q[:, :S], k[:, :S], v[:, :S], klen, 1e-6)).abs().max().item() < 1e-5
+        _phi, q[:, :S], k[:, :S], v[:, :S], klen, 1e-6)).abs().max().item() < 1e-5
 
 
 def test_batch_equals_recurrent_form(att):
@@ -90,7 +102,7 @@ def test_batch_equals_recurrent_form(att):
     layer = att.CausalLinearAttention(E)
     out = layer(q, k, v, m.TriangularCausalMask(L, device="cuda"), lengths, lengths)
     # recurrent form (recurrent/attention/self_attention/linear_attention.py:63-90)
-    Q, K = att.elu_feature_map(q.double()), att.elu_feature_map(k.double())
+    Q, K = _phi(q.double()), _phi(k.double())
     S = torch.zeros(N, H, E, M, dtype=torch.float64, device="cuda")
     Zs = torch.zeros(N, H, E, dtype=torch.float64, device="cuda")
     worst = 0.0
@@ -140,3 +152,68 @@ def test_encoder_against_dense_inner_attention(att):
     out = enc(x, attn_mask=mask)
     out.sum().backward()
     assert all(p.grad is not None and torch.isfinite(p.grad).all() for p in enc.parameters())
+
+
+def test_encoder_against_reference_golden_outputs(att):
+    """The reference's builder-made 2-layer causal-linear encoder (gelu, final norm, randomised
+    LayerNorm weights): its state_dict loads into the encoder here by name, and the outputs
+    for a full-length and a ragged batch must match.  Heads of 8 dimensions: the odd-shape
+    kernels run inside."""
+    m = att.masking
+    z = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden",
+                             "encoder_causal_linear.npz"))
+    n_layers, n_heads, qd, vd, ffn = (int(v) for v in z["config"])
+    enc = att.build_causal_linear_encoder(n_layers=n_layers, n_heads=n_heads,
+                                          query_dimensions=qd, value_dimensions=vd,
+                                          feed_forward_dimensions=ffn, activation="gelu",
+                                          final_normalization=True)
+    state = {k[len("param:"):]: torch.from_numpy(z[k]) for k in z.files if k.startswith("param:")}
+    assert set(state) == set(enc.state_dict()), "parameter names differ from the reference's"
+    enc.load_state_dict(state, strict=True)
+    enc = enc.cuda().eval()
+    x = torch.from_numpy(z["x"]).cuda()
+    L = x.shape[1]
+    mask = m.TriangularCausalMask(L, device="cuda")
+    with torch.no_grad():
+        y_full = enc(x, attn_mask=mask)
+        y_ragged = enc(x, attn_mask=mask,
+                       length_mask=m.LengthMask(torch.from_numpy(z["lengths"]).cuda(), max_len=L))
+    err_full = (y_full.cpu() - torch.from_numpy(z["y_full"])).abs().max().item()
+    err_ragged = (y_ragged.cpu() - torch.from_numpy(z["y_ragged"])).abs().max().item()
+    print("encoder vs reference outputs: full %.2e ragged %.2e" % (err_full, err_ragged),
+          flush=True)
+    assert err_full < 1e-4 and err_ragged < 1e-4
+
+
+def test_attention_takes_the_reference_constructor_arguments(att):
+    """feature_map is a factory called with the query dimensions (feature_maps/base.py:42-53),
+    event_dispatcher is accepted (attention/causal_linear_attention.py:47-55)."""
+    calls = []
+
+    class Squares(torch.nn.Module):           # an asymmetric map: queries and keys differ
+        def __init__(self, query_dims):
+            super().__init__()
+            calls.append(query_dims)
+
+        def new_feature_map(self, device):
+            calls.append(str(device))
+
+        def forward_queries(self, x):
+            return x * x + 0.5
+
+        def forward_keys(self, x):
+            return x.abs() + 0.25
+
+    m = att.masking
+    N, L, H, E, M = 2, 50, 2, 16, 16
+    gen = torch.Generator().manual_seed(8)
+    q, k, v = (torch.randn(N, L, H, X, generator=gen).cuda() for X in (E, E, M))
+    layer = att.CausalLinearAttention(E, feature_map=Squares, eps=1e-5, event_dispatcher="")
+    lengths = m.LengthMask(torch.full((N,), L).cuda(), max_len=L)
+    out = layer(q, k, v, m.TriangularCausalMask(L, device="cuda"), lengths, lengths)
+    assert calls[0] == E and calls[1].startswith("cuda")
+    Q, K = (q.double() ** 2 + 0.5), (k.double().abs() + 0.25)
+    A = torch.einsum("nlhe,nshe->nhls", Q, K) * torch.tril(
+        torch.ones(L, L, dtype=torch.float64, device="cuda"))
+    want = torch.einsum("nhls,nshm->nlhm", A / (A.sum(-1, keepdim=True) + 1e-5), v.double())
+    assert (out.double() - want).abs().max().item() < 1e-5
