@@ -29,12 +29,19 @@ for p in (ROOT, os.path.join(ROOT, "fast-transformers_amd")):
 
 HBM_PEAK_GBPS = 8000.0          # MI355X HBM3E, published
 MFMA_FP32_PEAK_TFLOPS = 157.3   # MI355X dense fp32 matrix, published
+MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 matrix, published
 
-# HBM bytes per scan-kernel launch (mean of the forward and the backward launch) from
+# HBM-side bytes per scan-kernel launch (mean of the forward and the backward launch) from
 # rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script, scaled by what the same
 # counters read for the 256 MiB copy of --calibrate-copy; the runs are summarised in
-# profiles/scan_dma_kernel_<workload>_traffic.md.  None = not measured for that workload.
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {"cfg2": 234721354, "cfg3": 3186430251}
+# profiles/scan_dma_kernel_<workload>_traffic.md.  Each figure is stamped with the hash of
+# the kernel sources it was measured with (kernel_source_hash() below): the JSON line
+# carries it only while the sources are unchanged, otherwise null.
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {
+    # workload: (bytes, kernel source hash at the time of the measurement)
+    "cfg2": (234721354, "unstamped"),
+    "cfg3": (3186430251, "unstamped"),
+}
 
 WORKLOADS = {
     # name: (N, H, L, E, M, dtype, seed)
@@ -43,6 +50,26 @@ WORKLOADS = {
     "cfg4op": (10, 8, 4096, 64, 64, "f32", 4),
     "cfg5": (4, 32, 16384, 32, 128, "bf16", 5),
 }
+
+
+def kernel_source_hash():
+    """First 16 hex digits of the SHA-256 over the kernel sources (csrc/*.h, *.hip) and the
+    C ABI header, in name order."""
+    import glob
+    import hashlib
+    h = hashlib.sha256()
+    for path in sorted(glob.glob(os.path.join(ROOT, "fast-transformers_amd", "csrc", "*.h*")) +
+                       glob.glob(os.path.join(ROOT, "include", "*.h"))):
+        h.update(os.path.basename(path).encode())
+        h.update(open(path, "rb").read())
+    return h.hexdigest()[:16]
+
+
+def measured_traffic(workload):
+    entry = MEASURED_TRAFFIC_BYTES_PER_LAUNCH.get(workload)
+    if entry is None or entry[1] != kernel_source_hash():
+        return None
+    return entry[0]
 
 
 def alg_bytes_per_position(E, M, dtype):
@@ -62,6 +89,11 @@ def main():
     ap.add_argument("--workload", default="cfg2", choices=sorted(WORKLOADS) + ["cfg4"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--sets", type=int, default=0, help="input sets to rotate over (0 = auto)")
+    ap.add_argument("--ramp-ms", type=float, default=300.0,
+                    help="set-up: untimed steps for this many milliseconds before the warm-up "
+                         "steps, so that the GPU clocks have ramped (0 to skip)")
+    ap.add_argument("--print-kernel-hash", action="store_true",
+                    help="print the kernel source hash that stamps measured traffic and exit")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one 256 MiB device copy (a known-size kernel for scaling "
                          "the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)")
@@ -70,6 +102,9 @@ def main():
         args.steps = 50 if args.workload == "cfg4" else 1000
     if args.warmup is None:
         args.warmup = 5 if args.workload == "cfg4" else 200
+    if args.print_kernel_hash:
+        print(kernel_source_hash())
+        return
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU (the path shards over N*H with no "
               "communication; no multi-GPU figure is produced). Use --gpus 1.", file=sys.stderr)
@@ -154,6 +189,14 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
+    # set-up: a fresh GPU takes a few hundred milliseconds of load to reach its clocks
+    t_ramp = time.perf_counter()
+    i = 0
+    while (time.perf_counter() - t_ramp) * 1e3 < args.ramp_ms:
+        for _ in range(20):
+            step(i)
+            i += 1
+        torch.cuda.synchronize()
     for i in range(args.warmup):
         step(i)
     torch.cuda.synchronize()
@@ -199,6 +242,20 @@ def main():
     launch_ms = (fwd_avg + bwd_avg) / 2
     launch_bytes = (fb + bb) * TH / 2
     launch_gbps = launch_bytes / (launch_ms * 1e-3) / 1e9
+    # Both rooflines for the same launch.  Algorithmic flops are those of the recurrence,
+    # 14 E M per position for forward + backward; for fp32 rows they are priced against the
+    # fp32 matrix peak, for bf16 rows against the bf16 one.  The binding roofline is the one
+    # with the larger minimum time.
+    launch_flops = 14 * E * M * TH / 2
+    mfma_peak = MFMA_FP32_PEAK_TFLOPS if dtype == "f32" else MFMA_BF16_PEAK_TFLOPS
+    launch_tflops = launch_flops / (launch_ms * 1e-3) / 1e12
+    t_hbm, t_mfma = launch_bytes / (HBM_PEAK_GBPS * 1e9), launch_flops / (mfma_peak * 1e12)
+    hbm_entry = {"achieved": round(launch_gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                 "frac": round(launch_gbps / HBM_PEAK_GBPS, 4)}
+    mfma_entry = {"achieved": round(launch_tflops, 2), "peak": mfma_peak, "unit": "TFLOP/s",
+                  "frac": round(launch_tflops / mfma_peak, 4)}
+    bound = "mfma" if t_mfma > t_hbm else "hbm"
+    binding = mfma_entry if bound == "mfma" else hbm_entry
 
     result = {
         "metric": "causal_dot_product fwd+bwd Mtokens/s (H=8,E=M=64); % of HBM/MFMA roofline",
@@ -225,15 +282,21 @@ def main():
                    "fwdbwd_alg_TFLOPs": round(14 * E * M * TH / (ms_per_step * 1e-3) / 1e12, 2),
                    "fwdbwd_frac_of_hbm_roofline":
                        round((fb + bb) * TH / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)},
-        "roofline": {"bound": "hbm",
-                     "kernel": ("scan_dma_kernel" if dtype == "f32" and max(E, M) <= 64
+        "roofline": {"bound": bound,
+                     "kernel": ("scan_wg_kernel" if os.environ.get("FTC_WG", "0") == "1"
+                                and dtype == "f32" and max(E, M) <= 128
+                                else "scan_dma_kernel" if dtype == "f32" and max(E, M) <= 64
                                 else "scan_mfma_kernel")
                                + " (mean over the forward and the backward call)",
-                     "achieved": round(launch_gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": round(launch_gbps / HBM_PEAK_GBPS, 4),
+                     "achieved": binding["achieved"], "peak": binding["peak"],
+                     "unit": binding["unit"], "frac": binding["frac"],
+                     "hbm": hbm_entry, "mfma": mfma_entry,
+                     "min_time_us": {"hbm": round(t_hbm * 1e6, 2), "mfma": round(t_mfma * 1e6, 2)},
                      "launch_ms_avg": round(launch_ms, 5),
                      "alg_bytes_per_launch": int(launch_bytes),
-                     "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH.get(args.workload)},
+                     "alg_flops_per_launch": int(launch_flops),
+                     "traffic": measured_traffic(args.workload),
+                     "kernel_source_hash": kernel_source_hash()},
     }
 
     if not args.no_cpu:
@@ -268,6 +331,10 @@ def encoder_workload(args):
         op_events.append((e0, e1))
 
     with torch.no_grad():
+        t_ramp = time.perf_counter()
+        while (time.perf_counter() - t_ramp) * 1e3 < args.ramp_ms:
+            enc(x, attn_mask=mask)
+            torch.cuda.synchronize()
         for _ in range(args.warmup):
             enc(x, attn_mask=mask)
         torch.cuda.synchronize()
@@ -283,7 +350,22 @@ def encoder_workload(args):
         cla.causal_dot_product_hip = native
     op_ms = sum(a.elapsed_time(b) for a, b in op_events) / args.steps
     TH = N * 8 * L
-    print(json.dumps({
+    # roofline of the operator's launches inside the encoder (8 per forward pass, one per
+    # layer): forward only, so 4 E M flops and (2E + 2M) * 4 bytes per position
+    launch_ms = op_ms / 8
+    fb, _ = alg_bytes_per_position(64, 64, "f32")
+    launch_bytes, launch_flops = fb * TH, 4 * 64 * 64 * TH
+    gbps = launch_bytes / (launch_ms * 1e-3) / 1e9
+    tflops = launch_flops / (launch_ms * 1e-3) / 1e12
+    t_hbm = launch_bytes / (HBM_PEAK_GBPS * 1e9)
+    t_mfma = launch_flops / (MFMA_FP32_PEAK_TFLOPS * 1e12)
+    hbm_entry = {"achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                 "frac": round(gbps / HBM_PEAK_GBPS, 4)}
+    mfma_entry = {"achieved": round(tflops, 2), "peak": MFMA_FP32_PEAK_TFLOPS,
+                  "unit": "TFLOP/s", "frac": round(tflops / MFMA_FP32_PEAK_TFLOPS, 4)}
+    bound = "mfma" if t_mfma > t_hbm else "hbm"
+    binding = mfma_entry if bound == "mfma" else hbm_entry
+    result = {
         "metric": "causal-linear encoder eval forward Mtokens/s (8 layers, d_model 512); "
                   "causal_dot_product share reported in config",
         "value": round(N * L / (ms * 1e-3) / 1e6, 3), "unit": "Mtokens/s", "n_gpus": 1,
@@ -294,15 +376,31 @@ def encoder_workload(args):
                                "X=rand(10,4096,512), 8 heads, E=M=64, FFN 1024",
                    "causal_dot_product_ms_per_forward": round(op_ms, 4),
                    "causal_dot_product_share": round(op_ms / ms, 4),
-                   "causal_dot_product_fwd_alg_GBps":
-                       round(8 * 1024 * TH / (op_ms * 1e-3) / 1e9, 1)},
-    }))
+                   "causal_dot_product_fwd_alg_GBps": round(gbps, 1)},
+        "roofline": {"bound": bound,
+                     "kernel": "scan_dma_kernel (the operator's forward launch, one per layer; "
+                               "the rest of the encoder is torch's GEMMs and elementwise work)",
+                     "achieved": binding["achieved"], "peak": binding["peak"],
+                     "unit": binding["unit"], "frac": binding["frac"],
+                     "hbm": hbm_entry, "mfma": mfma_entry,
+                     "min_time_us": {"hbm": round(t_hbm * 1e6, 2), "mfma": round(t_mfma * 1e6, 2)},
+                     "launch_ms_avg": round(launch_ms, 5),
+                     "alg_bytes_per_launch": int(launch_bytes),
+                     "alg_flops_per_launch": int(launch_flops),
+                     "traffic": None,
+                     "kernel_source_hash": kernel_source_hash()},
+    }
+    if not args.no_cpu:
+        result["cpu_baseline"] = cpu_baseline(N, 8, L, 64, 64, 4, "cfg4", forward_only=True)
+    print(json.dumps(result))
 
 
-def cpu_baseline(N, H, L, E, M, seed, workload):
+def cpu_baseline(N, H, L, E, M, seed, workload, forward_only=False):
     """The reference's CPU extension (oracle/_ref) or its restatement, fwd+bwd, fp32, timed
     the way the reference's benchmark does (warm-up calls, then timed calls, wall clock;
-    tests/causal_product/test_causal_product_cpu.py:87-99)."""
+    tests/causal_product/test_causal_product_cpu.py:87-99).  ``forward_only``: the
+    operator's share of an eval forward pass (the encoder around it is not part of the
+    checker), in tokens of one layer's call per second."""
     import torch
     import oracle
     Q, K, V, G = oracle.make_inputs(N, H, L, E, M, seed)
@@ -316,7 +414,8 @@ def cpu_baseline(N, H, L, E, M, seed, workload):
 
     def call():
         fwd(Q, K, V, out)
-        bwd(Q, K, V, G, gq, gk, gv)
+        if not forward_only:
+            bwd(Q, K, V, G, gq, gk, gv)
 
     t = time.perf_counter()
     call()
@@ -336,9 +435,11 @@ def cpu_baseline(N, H, L, E, M, seed, workload):
         pass
     return {"value": round(N * L / dt / 1e6, 4), "unit": "Mtokens/s",
             "cores": min(threads, N * H), "kind": kind,
-            "sample": "%s fwd+bwd fp32, %d warm-up + %d timed calls, %.1f ms per call; "
+            "sample": "%s %s fp32, %d warm-up + %d timed calls, %.1f ms per call; "
                       "OpenMP over N*H=%d chains, host cpu_count=%d"
-                      % (workload, warm, timed, dt * 1e3, N * H, os.cpu_count())}
+                      % (workload,
+                         "operator forward only (one layer's call)" if forward_only else "fwd+bwd",
+                         warm, timed, dt * 1e3, N * H, os.cpu_count())}
 
 
 if __name__ == "__main__":
