@@ -330,4 +330,41 @@ int ftc_causal_dot_backward(const ftc_tensor4 *queries, const ftc_tensor4 *keys,
     return run_scans(scans, n, d.N, d.H, d.L, workspace, workspace_bytes, s);
 }
 
+int64_t ftc_causal_linear_attention_workspace_bytes(int64_t N, int64_t H, int64_t L, int64_t E,
+                                                    int64_t M, int32_t dtype) {
+    if (N < 0 || H < 0 || L < 0 || E < 0 || M < 0) return fail(FTC_ERR_INVALID, "negative size");
+    if (dtype != FTC_F32 && dtype != FTC_BF16) return fail(FTC_ERR_INVALID, "unknown dtype");
+    if (dtype != FTC_F32 || !(E == 32 || E == 64) || !(M == 32 || M == 64))
+        return fail(FTC_ERR_UNSUPPORTED,
+                    "the fused attention kernel takes fp32 rows with E, M in {32, 64}");
+    if (N * H * L == 0) return 0;
+    return fused_attention_workspace_bytes(N, H, L, E, M);
+}
+
+int ftc_causal_linear_attention(const ftc_tensor4 *queries, const ftc_tensor4 *keys,
+                                const ftc_tensor4 *values, const int64_t *key_lengths, float eps,
+                                const ftc_tensor4 *out, void *workspace, size_t workspace_bytes,
+                                void *stream) {
+    Dims d;
+    int rc = read_dims(queries, values, &d);
+    if (rc) return rc;
+    if ((rc = check_tensor(queries, "queries", d.N, d.H, d.L, d.E, FTC_F32, FTC_F32))) return rc;
+    if ((rc = check_tensor(keys, "keys", d.N, d.H, d.L, d.E, FTC_F32, FTC_F32))) return rc;
+    if ((rc = check_tensor(values, "values", d.N, d.H, d.L, d.M, FTC_F32, FTC_F32))) return rc;
+    if ((rc = check_tensor(out, "out", d.N, d.H, d.L, d.M, FTC_F32, FTC_F32))) return rc;
+    if (!(eps == eps)) return fail(FTC_ERR_INVALID, "eps is not a number");
+    if (!(d.E == 32 || d.E == 64) || !(d.M == 32 || d.M == 64))
+        return fail(FTC_ERR_UNSUPPORTED,
+                    "the fused attention kernel takes fp32 rows with E, M in {32, 64}");
+    if (d.N * d.H * d.L == 0) return FTC_OK;
+    const ScanDesc fwd = {as_operand(queries), as_operand(keys), as_operand(values),
+                          as_operand_out(out), false};
+    if (!fused_attention_supported(fwd, d.L))
+        return fail(FTC_ERR_UNSUPPORTED,
+                    "the fused attention kernel needs 16-byte aligned rows that do not overlap");
+    const FusedAttention fused = {key_lengths, eps};
+    return mfma_scan(&fwd, 1, d.N, d.H, d.L, workspace, workspace_bytes, (hipStream_t)stream,
+                     &fused);
+}
+
 }  // extern "C"

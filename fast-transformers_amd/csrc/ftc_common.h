@@ -109,9 +109,20 @@ bool mfma_scan_same_launch(const ScanDesc &x, const ScanDesc &y);
 // Workspace for `nscans` scans of one (D, F) run side by side in one launch.
 int64_t mfma_scan_workspace_bytes(int64_t N, int64_t H, int64_t L, int64_t D, int64_t F,
                                   int nscans);
-// Runs scans[0..nscans) (all of the same row widths) in one launch.
+// The fused attention form of a forward scan: a and b go through the feature map
+// elu(x) + 1, rows of b at or beyond key_lengths[n] count as zero, and every output row is
+// divided by (phi(a_l) . sum_{j <= l} phi(b_j) + eps).
+struct FusedAttention {
+    const int64_t *key_lengths;  // N values on the device, or nullptr (every key counts)
+    float eps;
+};
+bool fused_attention_supported(const ScanDesc &scan, int64_t L);
+int64_t fused_attention_workspace_bytes(int64_t N, int64_t H, int64_t L, int64_t D, int64_t F);
+// Runs scans[0..nscans) (all of the same row widths) in one launch.  `fused`: a single
+// forward scan in its fused attention form.
 int mfma_scan(const ScanDesc *scans, int nscans, int64_t N, int64_t H, int64_t L,
-              void *workspace, size_t workspace_bytes, hipStream_t stream);
+              void *workspace, size_t workspace_bytes, hipStream_t stream,
+              const FusedAttention *fused = nullptr);
 
 // Fill every row of `out` with zeros (used for empty contractions).
 int zero_rows(const OperandOut &out, int64_t N, int64_t H, int64_t L, hipStream_t stream);

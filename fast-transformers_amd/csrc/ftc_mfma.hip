@@ -21,10 +21,12 @@ bool use_wg_kernel(int64_t D, int64_t F, bool all_f32) {
     return false;
 }
 
-// `wg`: the plan is for workgroups of F / 32 wavefronts (each has its own flag words)
-MfmaPlan make_plan(int64_t N, int64_t H, int64_t L, int64_t D, int64_t F, int nscans, bool wg) {
+// `wg`: the plan is for workgroups of F / 32 wavefronts (each has its own flag words);
+// `norm`: for their fused attention form, with one more wavefront and state slab per unit
+MfmaPlan make_plan(int64_t N, int64_t H, int64_t L, int64_t D, int64_t F, int nscans, bool wg,
+                   bool norm = false) {
     MfmaPlan pl;
-    const int64_t flags_per_unit = wg ? F / 32 : 1;
+    const int64_t flags_per_unit = wg ? F / 32 + (norm ? 1 : 0) : 1;
     const int64_t chains = std::max<int64_t>(1, N * H);
     const int64_t total_chunks = (L + kChunk - 1) / kChunk;
     // Resident at a time: 1024 wavefronts (one per SIMD: register footprint), or one workgroup
@@ -32,7 +34,7 @@ MfmaPlan make_plan(int64_t N, int64_t H, int64_t L, int64_t D, int64_t F, int ns
     // length (in chunks) that minimises an estimate of the makespan: rounds of resident
     // wavefronts times the work of one wavefront (pass 1 costs about half of pass 2, the
     // exchange of segment sums about three chunks).
-    const int64_t slots = wg ? 256 * scan_wg_units_per_block((int)F) : 1024;
+    const int64_t slots = wg ? 256 * scan_wg_units_per_block((int)F, norm) : 1024;
     int64_t best_c = total_chunks;
     double best_cost = (double)total_chunks * (double)((chains * nscans + slots - 1) / slots);
     for (int64_t c = 1; c < total_chunks && c <= 4096; c++) {
@@ -60,8 +62,8 @@ MfmaPlan make_plan(int64_t N, int64_t H, int64_t L, int64_t D, int64_t F, int ns
     pl.waves = chains * pl.nseg;
     pl.workspace_bytes = 0;
     if (pl.nseg > 1)
-        pl.workspace_bytes =
-            kControlBytes + 2 * nscans * pl.waves * D * F * (int64_t)sizeof(float);
+        pl.workspace_bytes = kControlBytes + 2 * nscans * pl.waves * D * (F + (norm ? 32 : 0)) *
+                                                 (int64_t)sizeof(float);
 #ifdef FTC_TIMELINE
     pl.workspace_bytes += nscans * pl.waves * 128;  // time stamps (ftc_wg_kernel.h)
 #endif
@@ -149,13 +151,25 @@ int64_t mfma_scan_workspace_bytes(int64_t N, int64_t H, int64_t L, int64_t D, in
                     make_plan(N, H, L, D, F, nscans, true).workspace_bytes);
 }
 
+bool fused_attention_supported(const ScanDesc &sd, int64_t L) {
+    return combo_of(sd) == kFFFF && !sd.reverse && !sd.initial.ptr && !sd.final_.ptr &&
+           scan_wg_norm_covers(sd.a.width, sd.v.width) && mfma_scan_supported(sd, L);
+}
+
+int64_t fused_attention_workspace_bytes(int64_t N, int64_t H, int64_t L, int64_t D, int64_t F) {
+    return make_plan(N, H, L, D, F, 1, true, true).workspace_bytes;
+}
+
 int mfma_scan(const ScanDesc *scans, int nscans, int64_t N, int64_t H, int64_t L,
-              void *workspace, size_t workspace_bytes, hipStream_t stream) {
+              void *workspace, size_t workspace_bytes, hipStream_t stream,
+              const FusedAttention *fused) {
     if (nscans < 1 || nscans > kMaxScans) return fail(FTC_ERR_INVALID, "bad scan count");
     const int D = scans[0].a.width, F = scans[0].v.width;
     const Combo combo = combo_of(scans[0]);
-    const bool wg = use_wg_kernel(D, F, combo == kFFFF);
-    const MfmaPlan pl = make_plan(N, H, L, D, F, nscans, wg);
+    if (fused && (nscans != 1 || !fused_attention_supported(scans[0], L)))
+        return fail(FTC_ERR_UNSUPPORTED, "no fused attention kernel for this shape or layout");
+    const bool wg = fused || use_wg_kernel(D, F, combo == kFFFF);
+    const MfmaPlan pl = make_plan(N, H, L, D, F, nscans, wg, fused != nullptr);
     if (pl.workspace_bytes > 0 && (!workspace || workspace_bytes < (size_t)pl.workspace_bytes))
         return fail(FTC_ERR_WORKSPACE, "workspace of %lld bytes needed, %zu given",
                     (long long)pl.workspace_bytes, workspace_bytes);
@@ -192,6 +206,8 @@ int mfma_scan(const ScanDesc *scans, int nscans, int64_t N, int64_t H, int64_t L
     if ((int64_t)(pl.seg_len + 2 * kChunk) * max_stride * 4 >= 0x7fffffffLL)
         return fail(FTC_ERR_UNSUPPORTED, "segment too long for 32-bit offsets");
     args.L = L;
+    args.eps = fused ? fused->eps : 0.f;
+    args.key_len = fused ? fused->key_lengths : nullptr;
     args.H = (int32_t)H;
     args.seg_len = pl.seg_len;
     args.nseg = pl.nseg;
@@ -217,7 +233,7 @@ int mfma_scan(const ScanDesc *scans, int nscans, int64_t N, int64_t H, int64_t L
     bool dma = D <= 64 && combo == kFFFF;
     if (const char *env = getenv("FTC_DMA")) dma = dma && atoi(env) != 0;  // tuning aid
     if (wg) {
-        launch_scan_wg_ffff(D, F, workspace, args, stream);
+        launch_scan_wg_ffff(D, F, fused != nullptr, workspace, args, stream);
     } else if (dma) {
         launch_scan_dma_ffff(D, F, workspace, args, stream);
     } else switch (combo) {

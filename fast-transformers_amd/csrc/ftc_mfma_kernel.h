@@ -455,6 +455,9 @@ struct ScanArgs {
     int32_t waves_per_scan;
     int32_t total_waves;  // nscans * waves_per_scan
     int32_t group;        // steps per group of the two-level state sum
+    // fused attention form of the workgroup kernel only (ftc_wg_kernel.h, NORM)
+    float eps;               // added to the denominator
+    const int64_t *key_len;  // keys per batch entry, N values on the device; nullptr: all L
 };
 
 // Which (scan, chain, L-segment) a wavefront works on.

@@ -36,6 +36,25 @@
 // All units of a workgroup pass the same barriers, so every loop runs for the largest chunk
 // count among them; a unit that has run out of chunks (or does not exist: the last
 // workgroup of a scan may have fewer units) only keeps time.
+//
+// NORM = true is causally masked linear attention in one pass over the rows
+// (fast_transformers/attention/causal_linear_attention.py:71-104 with the feature map of
+// feature_maps/base.py:71-73):
+//
+//   out[c, l, :] = sum_{j <= l} (phi(a_l) . phi'(b_j)) v_j  /  (phi(a_l) . sum_{j <= l} phi'(b_j) + eps)
+//   phi(x) = x > 0 ? x + 1 : exp(x)   (= elu(x) + 1);   phi'(b_j) = phi(b_j) if j < key_len[n] else 0
+//
+//  * The producers apply phi to the rows of a and b as they cut them, and zero the rows of b
+//    at or beyond the key length (and beyond the end of the segment, where phi(0) = 1 would
+//    otherwise enter).
+//  * The denominator is the same scan with a column of ones for values.  A unit gets one
+//    more consumer (w = F / 32) whose "values" are a constant tile in LDS: column 0 one,
+//    columns 1 .. 31 zero.  Its state is sum phi'(b_j) (in column 0), and row 0 of its Ot is
+//    the denominator of the chunk's 32 positions, which it leaves in LDS before the
+//    barrier that ends the chunk.  The other consumers hold their Ot across that barrier,
+//    divide, and store.  With F = 64 a unit takes three of the four consumers of a
+//    workgroup and the fourth idles (one unit per workgroup); with F = 32 there are two
+//    units of two consumers each.
 #pragma once
 #include "ftc_mfma_dma_kernel.h"
 
@@ -112,6 +131,17 @@ __device__ __forceinline__ void split_pair_under_mfma(float x0, float x1, uint32
             x1 = x1 - __uint_as_float(__float_as_uint(x1) & 0xffff0000u);
         }
     }
+}
+
+// elu(x) + 1 on four values of a row; `keep` false: the row is masked out (zeros).
+__device__ __forceinline__ float feature_phi(float x) { return x > 0.f ? x + 1.f : expf(x); }
+__device__ __forceinline__ u32x4 feature_quad(const u32x4 raw, bool keep) {
+    u32x4 r;
+    r.x = keep ? __float_as_uint(feature_phi(__uint_as_float(raw.x))) : 0u;
+    r.y = keep ? __float_as_uint(feature_phi(__uint_as_float(raw.y))) : 0u;
+    r.z = keep ? __float_as_uint(feature_phi(__uint_as_float(raw.z))) : 0u;
+    r.w = keep ? __float_as_uint(feature_phi(__uint_as_float(raw.w))) : 0u;
+    return r;
 }
 
 // Four consecutive fp32 values of a row -> 8 bytes of each of the three piece tiles.
@@ -192,12 +222,15 @@ __device__ __forceinline__ bool unit_request(const ScanArgs &p, gu32 *flags, int
     return true;
 }
 
-template <int D, int F>
+template <int D, int F, bool NORM>
 __global__ __launch_bounds__(512, 2) void scan_wg_kernel(uint32_t *__restrict__ ws_ptr,
                                                          ScanArgs p) {
-    constexpr int NW = F / 32;          // consumers (and producers) per unit
-    constexpr int NS = 4 / NW;          // units per workgroup
-    constexpr int T = 64 * NW;          // producer lanes per unit
+    constexpr int NWV = F / 32;               // consumers of a unit that own value columns
+    constexpr int NW = NWV + (NORM ? 1 : 0);  // consumers per unit
+    constexpr int NS = 4 / NW;                // units per workgroup
+    constexpr int NP = NORM ? 2 : NW;         // producers per unit
+    constexpr int T = 64 * NP;                // producer lanes per unit
+    constexpr int kOnesTile = kChunk * 64;    // bytes of a piece tile of the constant values
     constexpr int DT = D / 32;          // state tiles per slab
     constexpr int KD = D / 16;          // k-steps over d
     constexpr int RBA = D * 2, RBV = F * 2;             // bytes per row of a bf16 piece tile
@@ -207,8 +240,9 @@ __global__ __launch_bounds__(512, 2) void scan_wg_kernel(uint32_t *__restrict__ 
     constexpr int kUnitBytes = 2 * kBufBytes;                    // two buffers
     constexpr int QA = D / 4, QV = F / 4;               // 16-byte fp32 quads per row
     constexpr int LA = kChunk * QA / T, LV = kChunk * QV / T;  // quads per producer lane
-    static_assert(4 % NW == 0 && kChunk * QA % T == 0 && kChunk * QV % T == 0, "shape");
-    static_assert(NS * kUnitBytes <= 160 * 1024 - 256, "LDS");
+    static_assert(NP <= NW && NS >= 1 && kChunk * QA % T == 0 && kChunk * QV % T == 0, "shape");
+    static_assert(T % QA == 0, "a lane's quads of a and b share their columns");
+    static_assert(NS * kUnitBytes + (NORM ? 3 * kOnesTile + 1024 : 0) <= 160 * 1024 - 256, "LDS");
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -216,6 +250,8 @@ __global__ __launch_bounds__(512, 2) void scan_wg_kernel(uint32_t *__restrict__ 
     const bool producer = wave >= 4;
     const int slot = (wave & 3) / NW;  // unit of this workgroup
     const int w = (wave & 3) % NW;     // slab of a consumer, index of a producer
+    const bool in_use = slot < NS;     // false: a wavefront left over (three consumers per unit)
+    const bool is_den = NORM && w == NWV;  // the consumer that carries the denominator
     const int ln = lane & 31, g = lane >> 5;
 
     gu32 *hdr = (gu32 *)ws_ptr;
@@ -225,19 +261,29 @@ __global__ __launch_bounds__(512, 2) void scan_wg_kernel(uint32_t *__restrict__ 
     __shared__ __align__(16) char pieces_mem[NS * kUnitBytes];
     __shared__ uint32_t order_sh[4];
     __shared__ int count_sh[4][2];
-    lds_char *const unit_pc = (lds_char *)pieces_mem + slot * kUnitBytes;
+    __shared__ __align__(16) char ones_mem[NORM ? 3 * kOnesTile : 16];
+    __shared__ float den_sh[NORM ? NS : 1][2][kChunk];
+    lds_char *const unit_pc = (lds_char *)pieces_mem + (in_use ? slot : 0) * kUnitBytes;
+    if constexpr (NORM) {
+        for (int i = tid; i < 3 * kOnesTile / 4; i += 512) ((uint32_t *)ones_mem)[i] = 0u;
+    }
 
     // ---- which unit: one ticket per unit, taken by lane 0 of its first consumer ----
     Segment sg;
     bool valid;
     {
         uint32_t order;
-        const bool leader = !producer && w == 0 && lane == 0;
-        valid = unit_request<NS>(p, flags, slot, leader, sg, order);
+        const bool leader = in_use && !producer && w == 0 && lane == 0;
+        valid = unit_request<NS>(p, flags, slot, leader, sg, order) && in_use;
         if (leader) order_sh[slot] = order;
         __syncthreads();
         order = order_sh[slot];
         if (valid) valid = segment_locate(p, hdr, leader ? 0 : 1, order, sg);
+        if constexpr (NORM) {
+            // column 0 of piece 0 of the constant values is one (bf16 0x3f80)
+            if (tid < kChunk)
+                *(uint16_t *)(ones_mem + PieceSwizzle<64>::addr(tid, 0)) = (uint16_t)0x3f80;
+        }
     }
     const ScanOperands &op = p.scan[valid ? sg.scan_id : 0];
     const bool REV = valid && sg.rev;
@@ -249,7 +295,7 @@ __global__ __launch_bounds__(512, 2) void scan_wg_kernel(uint32_t *__restrict__ 
     const bool need_own_sum = exchange && step + 1 < p.nseg;
     // chunk counts of the two passes, largest over the units of the workgroup
     const int n1 = need_own_sum ? nchunks : 0, n2 = nchunks;
-    if (!producer && w == 0 && lane == 0) {
+    if (in_use && !producer && w == 0 && lane == 0) {
         count_sh[slot][0] = n1;
         count_sh[slot][1] = n2;
     }
@@ -265,7 +311,18 @@ __global__ __launch_bounds__(512, 2) void scan_wg_kernel(uint32_t *__restrict__ 
 
     if (producer) {
         // =========================== producers ===========================
-        const int ptid = w * 64 + lane;
+        const bool active = in_use && w < NP;  // a producer without rows only keeps time
+        const int ptid = (active ? w : 0) * 64 + lane;
+        // NORM: rows of b at or beyond this limit (counted from the start of the segment) are
+        // zeroed: the key length of the batch entry and the end of the segment
+        int b_limit = 0;
+        if constexpr (NORM) {
+            if (valid) {
+                const int64_t len = p.key_len ? p.key_len[n] : p.L;
+                b_limit = (int)max((int64_t)0, min((int64_t)rows, len - lo));
+            }
+        }
+        const int prow = ptid / QA;  // row of quad 0 of this lane; quad q: prow + q * (T / QA)
         const uint32_t a_slb = (uint32_t)op.a_sl * 4, b_slb = (uint32_t)op.b_sl * 4,
                        v_slb = (uint32_t)op.v_sl * 4;
         const char *a_seg =
@@ -301,9 +358,12 @@ __global__ __launch_bounds__(512, 2) void scan_wg_kernel(uint32_t *__restrict__ 
         // take turns, so that a request has a whole chunk's time to be served.
         struct Raw {
             u32x4 a[LA], b[LA], v[LV];
+            int row0;
         };
         Raw raw0, raw1;
         auto fetch = [&](Raw &r, int row0, bool with_a) {
+            if (!active) return;
+            r.row0 = row0;
 #pragma unroll
             for (int q = 0; q < LA; q++) {
                 if (with_a)
@@ -318,11 +378,18 @@ __global__ __launch_bounds__(512, 2) void scan_wg_kernel(uint32_t *__restrict__ 
                     v_rs, v_goff[q] + (uint32_t)row0 * v_slb, 0, 0);
         };
         auto cut = [&](const Raw &r, int buf, bool with_a) {
+            if (!active) return;
             lds_char *const pc = unit_pc + buf * kBufBytes;
 #pragma unroll
             for (int q = 0; q < LA; q++) {
-                if (with_a) split_quad_to_lds(r.a[q], pc, kTileA, a_waddr[q]);
-                split_quad_to_lds(r.b[q], pc + kOffB, kTileA, a_waddr[q]);
+                if constexpr (NORM) {
+                    const bool keep = (uint32_t)(r.row0 + prow + q * (T / QA)) < (uint32_t)b_limit;
+                    if (with_a) split_quad_to_lds(feature_quad(r.a[q], true), pc, kTileA, a_waddr[q]);
+                    split_quad_to_lds(feature_quad(r.b[q], keep), pc + kOffB, kTileA, a_waddr[q]);
+                } else {
+                    if (with_a) split_quad_to_lds(r.a[q], pc, kTileA, a_waddr[q]);
+                    split_quad_to_lds(r.b[q], pc + kOffB, kTileA, a_waddr[q]);
+                }
             }
 #pragma unroll
             for (int q = 0; q < LV; q++) split_quad_to_lds(r.v[q], pc + kOffV, kTileV, v_waddr[q]);
@@ -399,7 +466,10 @@ __global__ __launch_bounds__(512, 2) void scan_wg_kernel(uint32_t *__restrict__ 
     //  b^T, tile dt: columns 32 dt + 16 (G % 2) + 8 (x % 2) + 4 (x / 2) + 0..3, x = s % 4
     //  v (this consumer's slab): columns 32 w + 16 (G % 2) + 4 x + 0..3
     // (rows 16 .. 31 of a tile have the swizzle keys of rows 0 .. 15)
+    // The values of the denominator's consumer are the constant tile: other base, other
+    // tile and half-tile strides (vts, vhs), rows of 64 bytes.
     int bt_addr[DT][2], vt_addr[2];
+    const int vts = is_den ? kOnesTile : kTileV, vhs = is_den ? 16 * 64 : 16 * RBV;
     {
         const int G = lane >> 4, s = lane & 15, x = s & 3;
 #pragma unroll
@@ -409,9 +479,13 @@ __global__ __launch_bounds__(512, 2) void scan_wg_kernel(uint32_t *__restrict__ 
             for (int dt = 0; dt < DT; dt++)
                 bt_addr[dt][u] = kOffB + PieceSwizzle<RBA>::addr(
                     row, 2 * (32 * dt + 16 * (G % 2) + 8 * (x % 2) + 4 * (x / 2)));
-            vt_addr[u] = kOffV + PieceSwizzle<RBV>::addr(row, 2 * (32 * w + 16 * (G % 2) + 4 * x));
+            vt_addr[u] = is_den ? PieceSwizzle<64>::addr(row, 2 * (16 * (G % 2) + 4 * x))
+                                : PieceSwizzle<RBV>::addr(row, 2 * (32 * w + 16 * (G % 2) + 4 * x));
         }
     }
+    auto v_tiles = [&](const lds_char *pc) -> const lds_char * {
+        return is_den ? (const lds_char *)ones_mem : pc + kOffV;
+    };
     // causal mask inside a chunk as bit masks (all ones: keep): accumulator register r of
     // lane (i = ln, g) holds row j = 8 (r / 4) + 4 g + r % 4 of Pt
     uint32_t keep[16];
@@ -428,12 +502,13 @@ __global__ __launch_bounds__(512, 2) void scan_wg_kernel(uint32_t *__restrict__ 
         for (int r = 0; r < 16; r++) S[dt][r] = 0.f;
     // position-major fragments of the chunk in buffer pc: v (this slab's columns), b^T
     auto v_frags = [&](const lds_char *pc, Frag (&f)[2][3]) {
+        const lds_char *const vpc = v_tiles(pc);
 #pragma unroll
         for (int hh = 0; hh < 2; hh++)
 #pragma unroll
             for (int k = 0; k < 3; k++)
-                f[hh][k] = lds_frag_tr(pc + k * kTileV + hh * 16 * RBV + vt_addr[0],
-                                       pc + k * kTileV + hh * 16 * RBV + vt_addr[1]);
+                f[hh][k] = lds_frag_tr(vpc + k * vts + hh * vhs + vt_addr[0],
+                                       vpc + k * vts + hh * vhs + vt_addr[1]);
     };
     auto bt_frags = [&](const lds_char *pc, Frag (&f)[2][DT][3]) {
 #pragma unroll
@@ -489,7 +564,7 @@ __global__ __launch_bounds__(512, 2) void scan_wg_kernel(uint32_t *__restrict__ 
 #pragma unroll
         for (int dt = 0; dt < DT; dt++) S[dt] = X[dt][0];
     }
-    if (valid && op.s0)
+    if (!NORM && valid && op.s0)
         wg_add_caller_state<DT>(op.s0 + (int64_t)n * op.s0_sn + (int64_t)h * op.s0_sh, op.s0_sd,
                                 32 * w + ln, g, S);
 
@@ -511,9 +586,11 @@ __global__ __launch_bounds__(512, 2) void scan_wg_kernel(uint32_t *__restrict__ 
     FTC_STAMP(2);
     wg_barrier();
     FTC_STAMP(3);
+    f32x16 O_held;  // NORM: Ot of a chunk, kept across the barrier behind which its denominator is
     for (int c = 0; c < n2max; c++) {
         if (c < n2) {
             const lds_char *pc = unit_pc + (c & 1) * kBufBytes;
+            const lds_char *const vpc = v_tiles(pc);
             Frag af[KD][3], bf[KD][3], v_frag[2][3], bt[2][DT][3], sf[2][3], p_frag[2][3];
             f32x16 P, O;
 #pragma unroll
@@ -535,8 +612,8 @@ __global__ __launch_bounds__(512, 2) void scan_wg_kernel(uint32_t *__restrict__ 
             auto tr_frag = [&](int i) {
                 const int hh = i / (3 + 3 * DT), j = i % (3 + 3 * DT);
                 if (j < 3)
-                    v_frag[hh][j] = lds_frag_tr(pc + j * kTileV + hh * 16 * RBV + vt_addr[0],
-                                                pc + j * kTileV + hh * 16 * RBV + vt_addr[1]);
+                    v_frag[hh][j] = lds_frag_tr(vpc + j * vts + hh * vhs + vt_addr[0],
+                                                vpc + j * vts + hh * vhs + vt_addr[1]);
                 else {
                     const int dt = (j - 3) / 3, k = (j - 3) % 3;
                     bt[hh][dt][k] = lds_frag_tr(pc + k * kTileA + hh * 16 * RBA + bt_addr[dt][0],
@@ -587,18 +664,37 @@ __global__ __launch_bounds__(512, 2) void scan_wg_kernel(uint32_t *__restrict__ 
 #pragma unroll
                 for (int m = 0; m < 6; m++) O = mfma(v_frag[hh][kPa[m]], p_frag[hh][kPb[m]], O);
             // lane (i = ln, g) holds f = 32 w + 8 q + 4 g + 0..3 in registers 4 q .. 4 q + 3
-            const uint32_t o_off = o_lane + (uint32_t)chunk_row0(c) * o_slb;
+            if constexpr (NORM) {
+                if (is_den) {
+                    if (g == 0) den_sh[slot][c & 1][ln] = O[0] + p.eps;
+                } else {
+                    O_held = O;
+                }
+            } else {
+                const uint32_t o_off = o_lane + (uint32_t)chunk_row0(c) * o_slb;
 #pragma unroll
-            for (int q = 0; q < 4; q++)
-                buffer_store4(o_rs, o_off + (uint32_t)(4 * 8 * q), O[4 * q + 0], O[4 * q + 1],
-                              O[4 * q + 2], O[4 * q + 3]);
+                for (int q = 0; q < 4; q++)
+                    buffer_store4(o_rs, o_off + (uint32_t)(4 * 8 * q), O[4 * q + 0], O[4 * q + 1],
+                                  O[4 * q + 2], O[4 * q + 3]);
+            }
         }
         wg_barrier();
+        if constexpr (NORM) {
+            if (c < n2 && !is_den) {
+                const float z = 1.0f / den_sh[slot][c & 1][ln];
+                const uint32_t o_off = o_lane + (uint32_t)chunk_row0(c) * o_slb;
+#pragma unroll
+                for (int q = 0; q < 4; q++)
+                    buffer_store4(o_rs, o_off + (uint32_t)(4 * 8 * q), O_held[4 * q + 0] * z,
+                                  O_held[4 * q + 1] * z, O_held[4 * q + 2] * z,
+                                  O_held[4 * q + 3] * z);
+            }
+        }
         if (c < 8) FTC_STAMP(8 + c);
     }
     FTC_STAMP(4);
     if (!valid) return;
-    if (op.s_out && step == p.nseg - 1)
+    if (!NORM && op.s_out && step == p.nseg - 1)
         wg_store_caller_state<DT>(op.s_out + (int64_t)n * op.so_sn + (int64_t)h * op.so_sh,
                                   op.so_sd, 32 * w + ln, g, S);
 
@@ -623,9 +719,12 @@ __global__ __launch_bounds__(512, 2) void scan_wg_kernel(uint32_t *__restrict__ 
 }
 
 // units (chain segments) per workgroup for output rows of F values
-inline int scan_wg_units_per_block(int F) { return 4 / (F / 32); }
-void launch_scan_wg_ffff(int D, int F, void *ws, const ScanArgs &args, hipStream_t stream);
+// `norm`: the fused attention form of the kernel (NORM = true)
+inline int scan_wg_units_per_block(int F, bool norm) { return 4 / (F / 32 + (norm ? 1 : 0)); }
+void launch_scan_wg_ffff(int D, int F, bool norm, void *ws, const ScanArgs &args,
+                         hipStream_t stream);
 bool scan_wg_covers(int D, int F);
+bool scan_wg_norm_covers(int D, int F);
 
 }  // namespace mfma
 }  // namespace ftc

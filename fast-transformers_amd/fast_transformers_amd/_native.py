@@ -28,6 +28,8 @@ EXPORTED_SYMBOLS = (
     "ftc_causal_dot_product_state",
     "ftc_causal_dot_backward_workspace_bytes",
     "ftc_causal_dot_backward",
+    "ftc_causal_linear_attention_workspace_bytes",
+    "ftc_causal_linear_attention",
 )
 
 
@@ -60,7 +62,8 @@ def load():
     lib.ftc_last_error.restype = ctypes.c_char_p
     lib.ftc_last_error.argtypes = []
     for name in ("ftc_causal_dot_product_workspace_bytes",
-                 "ftc_causal_dot_backward_workspace_bytes"):
+                 "ftc_causal_dot_backward_workspace_bytes",
+                 "ftc_causal_linear_attention_workspace_bytes"):
         f = getattr(lib, name)
         f.restype = ctypes.c_int64
         f.argtypes = [ctypes.c_int64] * 5 + [ctypes.c_int32]
@@ -77,6 +80,10 @@ def load():
     lib.ftc_causal_dot_backward.restype = ctypes.c_int
     lib.ftc_causal_dot_backward.argtypes = [t4] * 7 + [ctypes.c_void_p, ctypes.c_size_t,
                                                        ctypes.c_void_p]
+    lib.ftc_causal_linear_attention.restype = ctypes.c_int
+    lib.ftc_causal_linear_attention.argtypes = [t4] * 3 + [ctypes.c_void_p, ctypes.c_float, t4,
+                                                           ctypes.c_void_p, ctypes.c_size_t,
+                                                           ctypes.c_void_p]
     _lib = lib
     return lib
 

@@ -13,11 +13,18 @@ straight into ``(N, L, H, M)`` storage.  And the normaliser's ``q_l . sum_{j<=l}
 the same causal product with a column of ones for values, so it is a second call of the
 operator instead of a cumulative sum over L followed by a batched dot product (which on
 this stack cost ten and fifty times the operator itself).
+
+When nothing has to be differentiated (eval, ``torch.no_grad``) and the feature map is the
+default one, the whole body of ``forward`` -- both feature maps, the key-length mask, the
+product, the normaliser and the final scale -- is one launch of
+``ftc_causal_linear_attention`` (head dimensions 32 or 64, float32).  Training keeps the
+composition above, whose pieces autograd differentiates.
 """
 import torch
 from torch.nn import Module
 
-from ..causal_product import causal_dot_product_hip, causal_dot_backward_hip
+from ..causal_product import causal_dot_product_hip, causal_dot_backward_hip, \
+    causal_linear_attention_hip, fused_attention_covers
 
 
 class ActivationFunctionFeatureMap(Module):
@@ -138,12 +145,40 @@ class CausalLinearAttention(Module):
         return (torch.cat([K, K.new_zeros(N, L - S, H, E)], dim=1),
                 torch.cat([V, V.new_zeros(N, L - S, H, M)], dim=1))
 
+    def _fused_forward(self, queries, keys, values, key_lengths):
+        """The whole forward in one launch (feature map, key-length mask, product,
+        normaliser), when nothing has to be differentiated and a fused kernel covers the
+        sizes; None otherwise."""
+        if torch.is_grad_enabled() and (queries.requires_grad or keys.requires_grad
+                                        or values.requires_grad):
+            return None
+        fm = self.feature_map
+        if not (isinstance(fm, ActivationFunctionFeatureMap)
+                and fm.activation_function is _elu_plus_one):
+            return None
+        if queries.shape[1] != keys.shape[1] or keys.shape[1] != values.shape[1]:
+            return None
+        qv, kv, vv = (t.permute(0, 2, 1, 3) for t in (queries, keys, values))
+        if not fused_attention_covers(qv, vv):
+            return None
+        lengths = getattr(key_lengths, "lengths", None)
+        if lengths is None:  # not a length mask: the composition multiplies by its matrix
+            return None
+        lengths = lengths.to(device=queries.device, dtype=torch.int64).contiguous()
+        N, L, H, _ = queries.shape
+        out = torch.empty((N, L, H, values.shape[3]), device=queries.device, dtype=torch.float32)
+        causal_linear_attention_hip(qv, kv, vv, lengths, self.eps, out.permute(0, 2, 1, 3))
+        return out
+
     def forward(self, queries, keys, values, attn_mask, query_lengths, key_lengths):
+        if not attn_mask.lower_triangular:
+            raise RuntimeError("CausalLinearAttention only supports full lower triangular masks")
+        fused = self._fused_forward(queries, keys, values, key_lengths)
+        if fused is not None:
+            return fused
         self.feature_map.new_feature_map(queries.device)
         Q = self.feature_map.forward_queries(queries)
         K = self.feature_map.forward_keys(keys)
-        if not attn_mask.lower_triangular:
-            raise RuntimeError("CausalLinearAttention only supports full lower triangular masks")
         K = K * key_lengths.float_matrix[:, :, None, None]
         K, values = self._make_sizes_compatible(Q, K, values)
         # q_l . cumsum(k)_l  ==  sum_{j<=l} (q_l . k_j) * 1

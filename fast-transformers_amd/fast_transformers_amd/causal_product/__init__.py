@@ -177,6 +177,51 @@ def causal_dot_backward_hip(queries, keys, values, grad_out, grad_queries, grad_
     _native.check(rc, "ftc_causal_dot_backward")
 
 
+FTC_ERR_UNSUPPORTED = -2
+
+
+def fused_attention_covers(queries, values):
+    """True when ``ftc_causal_linear_attention`` has a kernel for tensors of these sizes and
+    element type ((N, H, L, E) queries, (N, H, L, M) values)."""
+    if queries.dtype != torch.float32 or values.dtype != torch.float32:
+        return False
+    if queries.device.type != "cuda":
+        return False
+    return queries.shape[3] in (32, 64) and values.shape[3] in (32, 64)
+
+
+def causal_linear_attention_hip(queries, keys, values, key_lengths, eps, out):
+    """In-place fused forward of causally masked linear attention with the feature map
+    ``elu(x) + 1``: replaces the body of the reference module's forward
+    (``attention/causal_linear_attention.py:71-104``) in one launch.  ``queries``, ``keys``:
+    raw (N, H, L, E) projections; ``values``, ``out``: (N, H, L, M); ``key_lengths``: int64
+    tensor of N lengths on the same device, or None.  Raises ``RuntimeError`` for sizes
+    without a fused kernel (see ``fused_attention_covers``)."""
+    lib = _native.load()
+    q, k, v = (_prepare(t, n) for t, n in
+               ((queries, "queries"), (keys, "keys"), (values, "values")))
+    o = _check_out(out, "out")
+    N, H, L, E = q.shape
+    M = v.shape[3]
+    if key_lengths is not None:
+        if key_lengths.dtype != torch.int64 or key_lengths.device != q.device or \
+                key_lengths.shape != (N,) or not key_lengths.is_contiguous():
+            raise RuntimeError("causal_linear_attention: key_lengths must be a contiguous int64 "
+                               "tensor of N values on the device of the queries")
+    with torch.cuda.device(q.device):
+        nbytes = _native.check(
+            lib.ftc_causal_linear_attention_workspace_bytes(N, H, L, E, M,
+                                                            _native.dtype_code(q.dtype)),
+            "ftc_causal_linear_attention_workspace_bytes")
+        ws, nbytes = _workspace(nbytes, q.device)
+        dq, dk, dv, do = (_native.describe(t) for t in (q, k, v, o))
+        rc = lib.ftc_causal_linear_attention(
+            dq, dk, dv, key_lengths.data_ptr() if key_lengths is not None else None, float(eps),
+            do, ws.data_ptr() if ws is not None else None, nbytes,
+            torch.cuda.current_stream().cuda_stream)
+    _native.check(rc, "ftc_causal_linear_attention")
+
+
 def _cpu_args(name, *tensors):
     for t in tensors:
         if t.dim() != 4 or t.device.type != "cpu":

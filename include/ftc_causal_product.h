@@ -151,6 +151,38 @@ int ftc_causal_dot_backward(const ftc_tensor4 *queries, const ftc_tensor4 *keys,
                             const ftc_tensor4 *grad_values, void *workspace,
                             size_t workspace_bytes, void *stream);
 
+/*
+ * Scratch bytes ftc_causal_linear_attention needs (>= 0), FTC_ERR_UNSUPPORTED when no fused
+ * kernel covers these sizes, or another negative ftc_status.
+ */
+int64_t ftc_causal_linear_attention_workspace_bytes(int64_t N, int64_t H, int64_t L, int64_t E,
+                                                    int64_t M, int32_t dtype);
+
+/*
+ * Causally masked linear attention with the feature map elu(x) + 1, in one pass over the
+ * rows.  Replaces the body of CausalLinearAttention.forward
+ * (attention/causal_linear_attention.py:71-104) for the default feature map
+ * (feature_maps/base.py:71-73): the two feature-map passes (:75-76), the key-length mask
+ * (:83), cumsum + einsum for the normaliser (:95), causal_linear with its layout copies
+ * (:19-24, :98-102) and the final scale (:104):
+ *
+ *   phi(x) = x > 0 ? x + 1 : exp(x)
+ *   Kf[n,h,j,:] = phi(keys[n,h,j,:]) if j < key_lengths[n] else 0
+ *   out[n,h,l,:] = sum_{j<=l} (phi(queries[n,h,l,:]) . Kf[n,h,j,:]) values[n,h,j,:]
+ *                  / (phi(queries[n,h,l,:]) . sum_{j<=l} Kf[n,h,j,:] + eps)
+ *
+ * queries, keys: (N,H,L,E) raw projections (before the feature map); values, out:
+ * (N,H,L,M); all FTC_F32, any N/H/L strides with 16-byte aligned rows (the module's
+ * (N,L,H,X) tensors are passed as permuted views).  key_lengths: N int64 values on the
+ * device, or NULL when every key counts.  Forward only.  Sizes: E, M in {32, 64};
+ * anything else returns FTC_ERR_UNSUPPORTED and the caller composes the result from
+ * ftc_causal_dot_product as before.
+ */
+int ftc_causal_linear_attention(const ftc_tensor4 *queries, const ftc_tensor4 *keys,
+                                const ftc_tensor4 *values, const int64_t *key_lengths, float eps,
+                                const ftc_tensor4 *out, void *workspace, size_t workspace_bytes,
+                                void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -18,6 +18,8 @@ Contents
 * ``recurrent_forward``: the step-wise einsum form of
   ``fast_transformers/recurrent/attention/self_attention/linear_attention.py:79-88``
   without the feature map and normaliser.
+* ``causal_linear_attention``: the caller of the op restated, feature map, key-length mask
+  and normaliser included (attention/causal_linear_attention.py:71-104).
 * ``make_inputs``: the seeded input generator for the measured configurations
   (Q, K = elu(x)+1 with x ~ N(0,1); V, G ~ N(0,1); draw order x_q, x_k, V, G).
 * ``load_reference_extension``: the reference's own CPU extension compiled by
@@ -184,6 +186,34 @@ def recurrent_forward(Q, K, V):
         S = S + torch.einsum("nhe,nhm->nhem", K[:, :, l], V[:, :, l])
         out[:, :, l] = torch.einsum("nhe,nhem->nhm", Q[:, :, l], S)
     return out
+
+
+def causal_linear_attention(queries, keys, values, key_lengths=None, eps=1e-6):
+    """``CausalLinearAttention.forward`` with the default feature map, restated
+    (attention/causal_linear_attention.py:71-104; feature_maps/base.py:71-73) over
+    ``(N, L, H, E)`` / ``(N, L, H, M)`` CPU tensors, equal numbers of queries and keys;
+    ``key_lengths``: N integers, or None when every key counts.
+
+    phi = elu + 1 on queries and keys (:75-76); keys at or beyond the length are zeroed
+    (:83); Z = 1 / (q . cumsum(k) + eps) (:95); the unnormalised rows come from the C
+    restatement of the native op on (N, H, L, X) copies (:19-24, :98-102); result rows are
+    scaled by Z (:104).
+
+    Pinned by: the outputs of the reference module itself stored in
+    tests/golden/attention_causal_linear.npz; the dense normalised closed form of the
+    reference's API test (tests/causal_product/test_causal_product.py:34-52) and the
+    step-wise form (recurrent/attention/self_attention/linear_attention.py:55-88), both in
+    tests/test_oracle.py."""
+    Q = torch.nn.functional.elu(queries) + 1
+    K = torch.nn.functional.elu(keys) + 1
+    N, L = Q.shape[0], Q.shape[1]
+    if key_lengths is not None:
+        keep = torch.arange(L)[None, :] < torch.as_tensor(key_lengths).reshape(N, 1)
+        K = K * keep.to(K.dtype)[:, :, None, None]
+    Z = 1 / (torch.einsum("nlhi,nlhi->nlh", Q, K.cumsum(1)) + eps)
+    product = forward(Q.permute(0, 2, 1, 3).contiguous(), K.permute(0, 2, 1, 3).contiguous(),
+                      values.permute(0, 2, 1, 3).contiguous())
+    return product.permute(0, 2, 1, 3).contiguous() * Z[:, :, :, None]
 
 
 def make_inputs(N, H, L, E, M, seed, dtype=torch.float32, positive_uniform=False):

@@ -1,4 +1,5 @@
-"""Writes tests/golden/encoder_causal_linear.npz from the reference's own modules.
+"""Writes tests/golden/encoder_causal_linear.npz and tests/golden/attention_causal_linear.npz
+from the reference's own modules.
 
     python tests/golden/make_encoder_golden.py          (build container only)
 
@@ -18,6 +19,11 @@ imports ``fast_transformers.builders`` from there, builds a 2-layer encoder
 ``state_dict``, two inputs (full length, and ragged lengths) and the outputs of
 ``encoder(x, attn_mask=TriangularCausalMask(L), length_mask=...)``.  Nothing of the
 reference is stored in this repository; the fixture is data (< 100 KB).
+
+The second file pins the attention module alone (attention/causal_linear_attention.py:71-104
+with the default feature map): raw queries and keys with both signs (so that both branches
+of elu(x) + 1 are taken), values, ragged key lengths, and the module's output, at two shapes
+(E = M = 8 over 37 positions; E = 64, M = 32 over 40 positions).
 """
 import os
 import subprocess
@@ -113,6 +119,25 @@ def main():
     print(out, os.path.getsize(out), "bytes;", len(arrays), "arrays")
     for k in sorted(arrays):
         print("  ", k, arrays[k].shape)
+
+    from fast_transformers.attention import CausalLinearAttention
+    arrays = {}
+    for tag, (N, L, H, E, M, lens) in {"a": (2, 37, 3, 8, 8, [37, 20]),
+                                        "b": (2, 40, 1, 64, 32, [40, 13])}.items():
+        att = CausalLinearAttention(E).eval()
+        q = 1.5 * torch.randn(N, L, H, E)
+        k = 1.5 * torch.randn(N, L, H, E)
+        v = torch.randn(N, L, H, M)
+        lengths = torch.tensor(lens)
+        with torch.no_grad():
+            y = att(q, k, v, TriangularCausalMask(L), LengthMask(torch.full((N,), L), max_len=L),
+                    LengthMask(lengths, max_len=L))
+        arrays.update({tag + "_q": q.numpy(), tag + "_k": k.numpy(), tag + "_v": v.numpy(),
+                       tag + "_lengths": lengths.numpy(), tag + "_y": y.numpy(),
+                       tag + "_eps": np.array(att.eps)})
+    out = os.path.join(HERE, "attention_causal_linear.npz")
+    np.savez_compressed(out, **arrays)
+    print(out, os.path.getsize(out), "bytes;", len(arrays), "arrays")
 
 
 if __name__ == "__main__":

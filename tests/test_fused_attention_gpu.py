@@ -1,0 +1,198 @@
+"""ftc_causal_linear_attention: feature map, key-length mask, causal product and normaliser in
+one launch, called through the C ABI and checked against
+
+(a) the outputs of the reference's own CausalLinearAttention
+    (tests/golden/attention_causal_linear.npz, written by tests/golden/make_encoder_golden.py),
+(b) the CPU restatement ``oracle.causal_linear_attention`` (float32 as the reference runs it,
+    float64 as the anchor) on seeded inputs: every supported pair of head dimensions,
+    chunk and segment boundaries, ragged / zero / over-long key lengths, (N, L, H, X) views,
+(c) properties that hold at any size: rows are weighted means of the values seen so far
+    (constant values come back unchanged), prefix property, independence of masked keys,
+and, at module level, against the composition of separate operator calls that training uses.
+
+Tolerance: 1e-4 relative to the largest magnitude of the chain (fp32 bar of the operator),
+and an element-wise violation fraction (1e-5 + 1e-4 |want|) no worse than twice what the
+float32 CPU restatement shows against float64, plus 6e-4.
+"""
+import ctypes
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from parity import scale_error, violation_fraction
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def lib():
+    if not torch.cuda.is_available():
+        pytest.fail("GPU tests need a GPU")
+    from fast_transformers_amd import _native
+    return _native.load()
+
+
+def fused(lib, q, k, v, lengths, eps, out=None):
+    """q, k, v: (N, L, H, X) device tensors (any strides the ABI takes); straight C ABI call."""
+    from fast_transformers_amd import _native
+    N, L, H, E = q.shape
+    M = v.shape[3]
+    if out is None:
+        out = torch.full((N, L, H, M), float("nan"), device=q.device, dtype=torch.float32)
+    nbytes = lib.ftc_causal_linear_attention_workspace_bytes(N, H, L, E, M, _native.FTC_F32)
+    assert nbytes >= 0, _native.last_error()
+    ws = torch.zeros(max(nbytes, 256), dtype=torch.uint8, device=q.device)
+    d = [_native.describe(t.permute(0, 2, 1, 3)) for t in (q, k, v, out)]
+    rc = lib.ftc_causal_linear_attention(
+        ctypes.byref(d[0]), ctypes.byref(d[1]), ctypes.byref(d[2]),
+        ctypes.c_void_p(lengths.data_ptr()) if lengths is not None else None,
+        ctypes.c_float(eps), ctypes.byref(d[3]), ctypes.c_void_p(ws.data_ptr()), nbytes,
+        ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+    assert rc == 0, _native.last_error()
+    torch.cuda.synchronize()
+    assert int(ws[8:12].view(torch.int32).item()) == 0, "a wavefront gave up waiting"
+    return out
+
+
+def inputs(N, L, H, E, M, seed, scale=1.5):
+    gen = torch.Generator().manual_seed(seed)
+    q = scale * torch.randn(N, L, H, E, generator=gen)
+    k = scale * torch.randn(N, L, H, E, generator=gen)
+    v = torch.randn(N, L, H, M, generator=gen)
+    return q, k, v
+
+
+def gate(got, q, k, v, lengths, eps):
+    """got: (N, L, H, M) on the host."""
+    want32 = oracle.causal_linear_attention(q, k, v, lengths, eps)
+    want64 = oracle.causal_linear_attention(q.double(), k.double(), v.double(), lengths, eps)
+    nhl = lambda t: t.permute(0, 2, 1, 3)
+    assert torch.isfinite(got).all()
+    assert scale_error(nhl(got), nhl(want32)) <= 1e-4
+    assert scale_error(nhl(got), nhl(want64)) <= max(4 * scale_error(nhl(want32), nhl(want64)), 2e-6)
+    v_ref = violation_fraction(want32, want64)
+    assert violation_fraction(got, want64) <= 2 * v_ref + 6e-4
+    assert violation_fraction(got, want32) <= 2 * v_ref + 6e-4
+
+
+def test_against_the_reference_modules_outputs(lib):
+    data = np.load(os.path.join(os.path.dirname(__file__), "golden", "attention_causal_linear.npz"))
+    q, k, v, y = (torch.from_numpy(data["b_" + x]) for x in ("q", "k", "v", "y"))
+    lengths = torch.from_numpy(data["b_lengths"])
+    got = fused(lib, q.cuda(), k.cuda(), v.cuda(), lengths.cuda(), float(data["b_eps"])).cpu()
+    assert (got - y).abs().max().item() <= 1e-4 * max(1.0, y.abs().max().item())
+    assert violation_fraction(got, y) == 0.0
+
+
+SHAPES = [
+    # N, L, H, E, M, key lengths (None: all)
+    (2, 1, 2, 64, 64, None),
+    (2, 31, 3, 64, 64, [31, 7]),
+    (1, 32, 2, 64, 32, [32]),
+    (3, 33, 1, 32, 64, [33, 0, 32]),
+    (2, 100, 4, 32, 32, [64, 100]),
+    (2, 1000, 8, 64, 64, [1000, 517]),
+    (1, 4096, 2, 64, 64, [3000]),          # several segments; the length cuts one of them
+    (2, 4100, 3, 32, 64, [4100, 33]),      # whole segments beyond the length
+    (1, 2500, 5, 64, 32, [9999]),          # longer than the sequence: every key counts
+    (3, 777, 2, 32, 32, None),
+]
+
+
+@pytest.mark.parametrize("shape", SHAPES, ids=lambda s: "n%d_l%d_h%d_e%d_m%d" % s[:5])
+def test_against_the_cpu_restatement(lib, shape):
+    N, L, H, E, M, lens = shape
+    q, k, v = inputs(N, L, H, E, M, seed=100 + L)
+    lengths = torch.tensor(lens) if lens is not None else None
+    got = fused(lib, q.cuda(), k.cuda(), v.cuda(),
+                lengths.cuda() if lengths is not None else None, 1e-6).cpu()
+    gate(got, q, k, v, lengths, 1e-6)
+
+
+def test_strided_views_and_eps(lib):
+    """Rows taken out of wider storage (the fused projection layout of an attention layer)
+    and a large eps."""
+    N, L, H, E, M = 2, 300, 4, 64, 64
+    q, k, v = inputs(N, L, H, E, M, seed=7)
+    wide = torch.zeros(N, L, H, 3 * 64, device="cuda")
+    wide[..., :64], wide[..., 64:128], wide[..., 128:] = q.cuda(), k.cuda(), v.cuda()
+    out_wide = torch.full((N, L, H, 2 * M), float("nan"), device="cuda")
+    lengths = torch.tensor([300, 123])
+    fused(lib, wide[..., :64], wide[..., 64:128], wide[..., 128:], lengths.cuda(), 0.25,
+          out=out_wide[..., M:])
+    assert torch.isnan(out_wide[..., :M]).all()
+    gate(out_wide[..., M:].cpu(), q, k, v, lengths, 0.25)
+
+
+def test_constant_values_come_back_and_masked_keys_do_not_matter(lib):
+    N, L, H, E, M = 2, 5000, 4, 64, 64
+    q, k, _ = inputs(N, L, H, E, M, seed=8)
+    v = torch.full((N, L, H, M), -3.25)
+    lengths = torch.tensor([5000, 1234]).cuda()
+    got = fused(lib, q.cuda(), k.cuda(), v.cuda(), lengths, 0.0)
+    assert (got + 3.25).abs().max().item() < 1e-4
+    # keys and values beyond the length are never seen
+    k2, v2 = k.clone(), torch.randn(N, L, H, M, generator=torch.Generator().manual_seed(9))
+    v3 = v2.clone()
+    k2[1, 1234:] = 50.0
+    v3[1, 1234:] = 1e6
+    a = fused(lib, q.cuda(), k.cuda(), v2.cuda(), lengths, 1e-6)
+    b = fused(lib, q.cuda(), k2.cuda(), v3.cuda(), lengths, 1e-6)
+    assert torch.equal(a, b)
+
+
+def test_prefix_property_at_full_size(lib):
+    """Config 4's operator shape: the first rows of a long call equal a short call's rows to
+    rounding (the segmentation differs), and a repeated call is bit-identical."""
+    N, L, H, E, M = 10, 4096, 8, 64, 64
+    q, k, v = (t.cuda() for t in inputs(N, L, H, E, M, seed=4))
+    whole = fused(lib, q, k, v, None, 1e-6)
+    again = fused(lib, q, k, v, None, 1e-6)
+    assert torch.equal(whole, again)
+    short = fused(lib, q[:, :1500].contiguous(), k[:, :1500].contiguous(),
+                  v[:, :1500].contiguous(), None, 1e-6)
+    assert scale_error(whole[:, :1500].permute(0, 2, 1, 3), short.permute(0, 2, 1, 3)) <= 2e-6
+    # a bounded sample against the CPU restatement
+    got = whole[:2].cpu()
+    gate(got, q[:2].cpu(), k[:2].cpu(), v[:2].cpu(), None, 1e-6)
+
+
+def test_sizes_without_a_fused_kernel_are_refused(lib):
+    from fast_transformers_amd import _native
+    assert lib.ftc_causal_linear_attention_workspace_bytes(1, 1, 64, 48, 64, _native.FTC_F32) == -2
+    assert lib.ftc_causal_linear_attention_workspace_bytes(1, 1, 64, 64, 64, _native.FTC_BF16) == -2
+    q = torch.zeros(1, 64, 1, 48, device="cuda")
+    v = torch.zeros(1, 64, 1, 64, device="cuda")
+    d = [_native.describe(t.permute(0, 2, 1, 3)) for t in (q, q, v, v.clone())]
+    rc = lib.ftc_causal_linear_attention(ctypes.byref(d[0]), ctypes.byref(d[1]), ctypes.byref(d[2]),
+                                         None, ctypes.c_float(1e-6), ctypes.byref(d[3]), None, 0,
+                                         None)
+    assert rc == -2 and "fused" in _native.last_error()
+
+
+def test_module_takes_the_fused_path_without_grad_and_agrees_with_the_composition(lib):
+    from fast_transformers_amd import attention, masking
+    from fast_transformers_amd.attention import causal_linear_attention as cla
+    N, L, H, E, M = 2, 700, 4, 64, 64
+    q, k, v = (t.cuda() for t in inputs(N, L, H, E, M, seed=11))
+    lengths = masking.LengthMask(torch.tensor([700, 301]).cuda(), max_len=L)
+    full = masking.LengthMask(torch.full((N,), L).cuda(), max_len=L)
+    mask = masking.TriangularCausalMask(L, device="cuda")
+    module = attention.CausalLinearAttention(E).cuda()
+    calls = []
+    native = cla.causal_linear_attention_hip
+    cla.causal_linear_attention_hip = lambda *a: (calls.append(1), native(*a))[1]
+    try:
+        with torch.no_grad():
+            y_fused = module(q, k, v, mask, full, lengths)
+        assert calls == [1]
+        qg = q.clone().requires_grad_(True)
+        y_composed = module(qg, k, v, mask, full, lengths)
+        assert calls == [1] and y_composed.requires_grad
+    finally:
+        cla.causal_linear_attention_hip = native
+    assert scale_error(y_fused.permute(0, 2, 1, 3), y_composed.detach().permute(0, 2, 1, 3)) <= 1e-5
+    gate(y_fused.cpu(), q.cpu(), k.cpu(), v.cpu(), torch.tensor([700, 301]), module.eps)

@@ -275,3 +275,74 @@ def test_stateful_forward_continues_into_the_stepwise_form():
         S = S + torch.einsum("nhd,nhm->nhdm", K[:, :, l], V[:, :, l])
         row = torch.einsum("nhd,nhdm->nhm", Q[:, :, l], S)
         assert max_relative_error(row, whole[:, :, l]) < 1e-12
+
+
+# ---------------------------------------------------------------------------
+# the caller restated: feature map, key-length mask, normaliser
+# ---------------------------------------------------------------------------
+def _attention_inputs(N, L, H, E, M, seed, dtype=torch.float64):
+    gen = torch.Generator().manual_seed(seed)
+    q = 1.5 * torch.randn(N, L, H, E, generator=gen)
+    k = 1.5 * torch.randn(N, L, H, E, generator=gen)
+    v = torch.randn(N, L, H, M, generator=gen)
+    return q.to(dtype), k.to(dtype), v.to(dtype)
+
+
+def test_attention_restatement_reproduces_the_reference_module_outputs():
+    """tests/golden/attention_causal_linear.npz holds what the reference's own
+    CausalLinearAttention returned (make_encoder_golden.py)."""
+    import numpy as np
+    import os
+    data = np.load(os.path.join(os.path.dirname(__file__), "golden", "attention_causal_linear.npz"))
+    for tag in ("a", "b"):
+        q, k, v, y = (torch.from_numpy(data[tag + "_" + x]) for x in ("q", "k", "v", "y"))
+        lengths = torch.from_numpy(data[tag + "_lengths"])
+        got = oracle.causal_linear_attention(q, k, v, lengths, float(data[tag + "_eps"]))
+        assert got.shape == y.shape
+        assert (got - y).abs().max().item() < 1e-5 * max(1.0, y.abs().max().item())
+        # the ragged entry really is ragged: it differs from the unmasked result past its length
+        full = oracle.causal_linear_attention(q, k, v, None, float(data[tag + "_eps"]))
+        n, cut = 1, int(lengths[1])
+        assert torch.equal(full[n, :cut], got[n, :cut])
+        assert (full[n, cut:] - got[n, cut:]).abs().max() > 1e-3
+
+
+def test_attention_restatement_is_the_dense_normalised_form():
+    """tests/causal_product/test_causal_product.py:34-40: masked phi(Q) phi(K)^T, rows divided
+    by their sums (+ eps), times V."""
+    q, k, v = _attention_inputs(2, 45, 3, 6, 5, seed=51)
+    lengths = torch.tensor([45, 17])
+    got = oracle.causal_linear_attention(q, k, v, lengths, eps=1e-6)
+    phi = lambda x: torch.where(x > 0, x + 1, torch.exp(x))
+    keep = (torch.arange(45)[None, :] < lengths[:, None]).double()
+    A = torch.einsum("nlhe,nshe->nhls", phi(q), phi(k) * keep[:, :, None, None])
+    A = A * torch.tril(torch.ones(45, 45, dtype=torch.float64))
+    A = A / (A.sum(-1, keepdim=True) + 1e-6)
+    want = torch.einsum("nhls,nshm->nlhm", A, v)
+    assert max_relative_error(got, want) < 1e-9
+
+
+def test_attention_restatement_is_the_stepwise_form():
+    """recurrent/attention/self_attention/linear_attention.py:55-88: Zi += phi(k);
+    Si += phi(k) v^T; out = phi(q) Si / (phi(q) . Zi + eps)."""
+    q, k, v = _attention_inputs(2, 33, 2, 4, 7, seed=52)
+    got = oracle.causal_linear_attention(q, k, v, None, eps=1e-6)
+    phi = lambda x: torch.nn.functional.elu(x) + 1
+    Si = torch.zeros(2, 2, 4, 7, dtype=torch.float64)
+    Zi = torch.zeros(2, 2, 4, dtype=torch.float64)
+    for l in range(33):
+        Q, K = phi(q[:, l]), phi(k[:, l])
+        Zi = Zi + K
+        Si = Si + torch.einsum("nhd,nhm->nhdm", K, v[:, l])
+        Z = 1. / (torch.einsum("nhd,nhd->nh", Q, Zi) + 1e-6)
+        V = torch.einsum("nhd,nhdm,nh->nhm", Q, Si, Z)
+        assert max_relative_error(got[:, l], V) < 1e-9
+
+
+def test_attention_rows_are_convex_combinations_of_values():
+    """With eps = 0 every output row is a weighted mean of the values seen so far (weights
+    positive, summing to one): constant values come back unchanged."""
+    q, k, _ = _attention_inputs(1, 50, 2, 8, 3, seed=53)
+    v = torch.full((1, 50, 2, 3), 2.5, dtype=torch.float64)
+    got = oracle.causal_linear_attention(q, k, v, None, eps=0.0)
+    assert (got - 2.5).abs().max().item() < 1e-9
