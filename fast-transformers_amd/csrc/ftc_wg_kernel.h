@@ -133,14 +133,20 @@ __device__ __forceinline__ void split_pair_under_mfma(float x0, float x1, uint32
     }
 }
 
-// elu(x) + 1 on four values of a row; `keep` false: the row is masked out (zeros).
-__device__ __forceinline__ float feature_phi(float x) { return x > 0.f ? x + 1.f : expf(x); }
-__device__ __forceinline__ u32x4 feature_quad(const u32x4 raw, bool keep) {
+// elu(x) + 1 = max(x, 0) + exp(min(x, 0)): five instructions, no select.  For x > 0 the
+// second term is exactly one.  For x <= 0 the exponent x log2(e) is rounded once, which costs
+// at most |x| 2^-24 ln 2 of relative accuracy -- in absolute terms never more than
+// 2^-24 ln 2 max_x |x| e^x = 1.6e-8, a fraction of the rounding of a feature near one.
+__device__ __forceinline__ float feature_phi(float x) {
+    return fmaxf(x, 0.f) + __builtin_amdgcn_exp2f(fminf(x, 0.f) * 1.44269502f);
+}
+// the feature map on four values of a row
+__device__ __forceinline__ u32x4 feature_quad(const u32x4 raw) {
     u32x4 r;
-    r.x = keep ? __float_as_uint(feature_phi(__uint_as_float(raw.x))) : 0u;
-    r.y = keep ? __float_as_uint(feature_phi(__uint_as_float(raw.y))) : 0u;
-    r.z = keep ? __float_as_uint(feature_phi(__uint_as_float(raw.z))) : 0u;
-    r.w = keep ? __float_as_uint(feature_phi(__uint_as_float(raw.w))) : 0u;
+    r.x = __float_as_uint(feature_phi(__uint_as_float(raw.x)));
+    r.y = __float_as_uint(feature_phi(__uint_as_float(raw.y)));
+    r.z = __float_as_uint(feature_phi(__uint_as_float(raw.z)));
+    r.w = __float_as_uint(feature_phi(__uint_as_float(raw.w)));
     return r;
 }
 
@@ -228,9 +234,10 @@ __global__ __launch_bounds__(512, 2) void scan_wg_kernel(uint32_t *__restrict__ 
     constexpr int NWV = F / 32;               // consumers of a unit that own value columns
     constexpr int NW = NWV + (NORM ? 1 : 0);  // consumers per unit
     constexpr int NS = 4 / NW;                // units per workgroup
-    constexpr int NP = NORM ? 2 : NW;         // producers per unit
+    constexpr int NP = 4 / NS;                // producers per unit
     constexpr int T = 64 * NP;                // producer lanes per unit
     constexpr int kOnesTile = kChunk * 64;    // bytes of a piece tile of the constant values
+    constexpr int PF = NORM ? 4 : 2;          // chunks requested ahead by the producers
     constexpr int DT = D / 32;          // state tiles per slab
     constexpr int KD = D / 16;          // k-steps over d
     constexpr int RBA = D * 2, RBV = F * 2;             // bytes per row of a bf16 piece tile
@@ -240,7 +247,8 @@ __global__ __launch_bounds__(512, 2) void scan_wg_kernel(uint32_t *__restrict__ 
     constexpr int kUnitBytes = 2 * kBufBytes;                    // two buffers
     constexpr int QA = D / 4, QV = F / 4;               // 16-byte fp32 quads per row
     constexpr int LA = kChunk * QA / T, LV = kChunk * QV / T;  // quads per producer lane
-    static_assert(NP <= NW && NS >= 1 && kChunk * QA % T == 0 && kChunk * QV % T == 0, "shape");
+    static_assert(NS >= 1 && NS * NP == 4 && kChunk * QA % T == 0 && kChunk * QV % T == 0, "shape");
+    static_assert(PF % 2 == 0, "register set and LDS buffer of a chunk follow from its parity");
     static_assert(T % QA == 0, "a lane's quads of a and b share their columns");
     static_assert(NS * kUnitBytes + (NORM ? 3 * kOnesTile + 1024 : 0) <= 160 * 1024 - 256, "LDS");
 
@@ -248,9 +256,10 @@ __global__ __launch_bounds__(512, 2) void scan_wg_kernel(uint32_t *__restrict__ 
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const bool producer = wave >= 4;
-    const int slot = (wave & 3) / NW;  // unit of this workgroup
-    const int w = (wave & 3) % NW;     // slab of a consumer, index of a producer
-    const bool in_use = slot < NS;     // false: a wavefront left over (three consumers per unit)
+    // consumer: unit and slab; producer: unit and index among the unit's producers
+    const int slot = (wave & 3) / (producer ? NP : NW);
+    const int w = (wave & 3) % (producer ? NP : NW);
+    const bool in_use = slot < NS;     // false: a consumer left over (three consumers per unit)
     const bool is_den = NORM && w == NWV;  // the consumer that carries the denominator
     const int ln = lane & 31, g = lane >> 5;
 
@@ -285,6 +294,10 @@ __global__ __launch_bounds__(512, 2) void scan_wg_kernel(uint32_t *__restrict__ 
                 *(uint16_t *)(ones_mem + PieceSwizzle<64>::addr(tid, 0)) = (uint16_t)0x3f80;
         }
     }
+    // Every lane of a wavefront holds the same answer; saying so keeps the segment's
+    // descriptors and loop bounds in scalar registers (a descriptor the compiler cannot prove
+    // uniform costs a loop over its distinct values around every load and store).
+    valid = __builtin_amdgcn_readfirstlane((int)valid) != 0;
     const ScanOperands &op = p.scan[valid ? sg.scan_id : 0];
     const bool REV = valid && sg.rev;
     const int step = valid ? sg.step : 0, n = valid ? sg.n : 0, h = valid ? sg.h : 0;
@@ -307,12 +320,22 @@ __global__ __launch_bounds__(512, 2) void scan_wg_kernel(uint32_t *__restrict__ 
         n2max = max(n2max, count_sh[s][1]);
     }
 
+    n1max = __builtin_amdgcn_readfirstlane(n1max);
+    n2max = __builtin_amdgcn_readfirstlane(n2max);
+#ifdef FTC_TIMELINE
+    // stamps 0 .. 4 and 8 .. 15: first consumer of the unit; 5 .. 7: its first producer
+    typedef __attribute__((address_space(1))) uint64_t gu64;
+    const bool stamp_on = valid && p.nseg > 1 && w == 0 && lane == 0;
+    gu64 *const stamp_base =
+        (gu64 *)((__attribute__((address_space(1))) char *)ws_ptr + kControlBytes +
+                 (int64_t)2 * p.total_waves * (D * 32 * NW * 4)) + (valid ? sg.ticket : 0) * 16;
+#endif
     auto chunk_row0 = [&](int c) -> int { return REV ? rows - kChunk * (c + 1) : kChunk * c; };
 
     if (producer) {
         // =========================== producers ===========================
-        const bool active = in_use && w < NP;  // a producer without rows only keeps time
-        const int ptid = (active ? w : 0) * 64 + lane;
+        const bool active = in_use;
+        const int ptid = w * 64 + lane;
         // NORM: rows of b at or beyond this limit (counted from the start of the segment) are
         // zeroed: the key length of the batch entry and the end of the segment
         int b_limit = 0;
@@ -354,13 +377,14 @@ __global__ __launch_bounds__(512, 2) void scan_wg_kernel(uint32_t *__restrict__ 
             v_goff[q] = (uint32_t)row * v_slb + 16u * c4;
             v_waddr[q] = PieceSwizzle<RBV>::addr(row, 8 * c4);
         }
-        // Rows are requested two chunks ahead of the cut, into two sets of registers that
-        // take turns, so that a request has a whole chunk's time to be served.
+        // Rows are requested PF chunks ahead of the cut, into PF sets of registers that take
+        // turns, so that a request has several chunks' time to be served.  (With one unit per
+        // workgroup the requests in flight are all that keeps the memory system busy.)
         struct Raw {
             u32x4 a[LA], b[LA], v[LV];
             int row0;
         };
-        Raw raw0, raw1;
+        Raw raw[PF];
         auto fetch = [&](Raw &r, int row0, bool with_a) {
             if (!active) return;
             r.row0 = row0;
@@ -380,12 +404,18 @@ __global__ __launch_bounds__(512, 2) void scan_wg_kernel(uint32_t *__restrict__ 
         auto cut = [&](const Raw &r, int buf, bool with_a) {
             if (!active) return;
             lds_char *const pc = unit_pc + buf * kBufBytes;
+            // NORM: every row of the chunk lies below the limit for rows of b (scalar test)
+            const bool whole = NORM && r.row0 >= 0 && r.row0 + kChunk <= b_limit;
 #pragma unroll
             for (int q = 0; q < LA; q++) {
                 if constexpr (NORM) {
-                    const bool keep = (uint32_t)(r.row0 + prow + q * (T / QA)) < (uint32_t)b_limit;
-                    if (with_a) split_quad_to_lds(feature_quad(r.a[q], true), pc, kTileA, a_waddr[q]);
-                    split_quad_to_lds(feature_quad(r.b[q], keep), pc + kOffB, kTileA, a_waddr[q]);
+                    if (with_a) split_quad_to_lds(feature_quad(r.a[q]), pc, kTileA, a_waddr[q]);
+                    u32x4 bq = feature_quad(r.b[q]);
+                    if (!whole) {  // a chunk that the key length or the end of the segment cuts
+                        if ((uint32_t)(r.row0 + prow + q * (T / QA)) >= (uint32_t)b_limit)
+                            bq = u32x4{0u, 0u, 0u, 0u};
+                    }
+                    split_quad_to_lds(bq, pc + kOffB, kTileA, a_waddr[q]);
                 } else {
                     if (with_a) split_quad_to_lds(r.a[q], pc, kTileA, a_waddr[q]);
                     split_quad_to_lds(r.b[q], pc + kOffB, kTileA, a_waddr[q]);
@@ -397,59 +427,36 @@ __global__ __launch_bounds__(512, 2) void scan_wg_kernel(uint32_t *__restrict__ 
         // rows of a chunk that does not exist lie outside the descriptor and read as zero
         auto pass1_row0 = [&](int i) -> int { return i < n1 ? chunk_row0(n1 - 1 - i) : -2 * kChunk; };
         auto pass2_row0 = [&](int c) -> int { return c < n2 ? chunk_row0(c) : -2 * kChunk; };
-
-        // ---- pass 1: chunk i of the walk (against the direction of pass 2) -> buffer i % 2;
-        // even chunks travel through raw0, odd ones through raw1 ----
-        if (n1max > 0) {
-            fetch(raw0, pass1_row0(0), false);
-            fetch(raw1, pass1_row0(1), false);
-            cut(raw0, 0, false);
-            fetch(raw0, pass1_row0(2), false);
+        // One pass over nmax chunks: chunk i of the walk goes to LDS buffer i % 2 through
+        // register set i % PF; one barrier before the first chunk and one per chunk.
+        auto run_pass = [&](int nmax, auto row0_of, bool with_a) {
+#pragma unroll
+            for (int j = 0; j < PF; j++) fetch(raw[j], row0_of(j), with_a);
+            cut(raw[0], 0, with_a);
+            fetch(raw[0], row0_of(PF), with_a);
             wg_barrier();
-            for (int i = 0; i < n1max; i += 2) {
-                if (i + 1 < n1max) {
-                    cut(raw1, 1, false);
-                    fetch(raw1, pass1_row0(i + 3), false);
+            for (int c = 0; c < nmax; c += PF) {
+#pragma unroll
+                for (int j = 0; j < PF; j++) {
+                    if (with_a && c + j == 4) FTC_STAMP(5);  // pass 2, fifth chunk
+                    if (c + j + 1 < nmax) {
+                        cut(raw[(j + 1) % PF], (j + 1) & 1, with_a);
+                        fetch(raw[(j + 1) % PF], row0_of(c + j + 1 + PF), with_a);
+                    }
+                    if (with_a && c + j == 4) FTC_STAMP(6);
+                    wg_barrier();
+                    if (with_a && c + j == 4) FTC_STAMP(7);
+                    if (c + j + 1 >= nmax) return;
                 }
-                wg_barrier();
-                if (i + 1 >= n1max) break;
-                if (i + 2 < n1max) {
-                    cut(raw0, 0, false);
-                    fetch(raw0, pass1_row0(i + 4), false);
-                }
-                wg_barrier();
             }
-        }
-        // ---- pass 2 ----
-        fetch(raw0, pass2_row0(0), true);
-        fetch(raw1, pass2_row0(1), true);
-        cut(raw0, 0, true);
-        fetch(raw0, pass2_row0(2), true);
-        wg_barrier();
-        for (int c = 0; c < n2max; c += 2) {
-            if (c + 1 < n2max) {
-                cut(raw1, 1, true);
-                fetch(raw1, pass2_row0(c + 3), true);
-            }
-            wg_barrier();
-            if (c + 1 >= n2max) break;
-            if (c + 2 < n2max) {
-                cut(raw0, 0, true);
-                fetch(raw0, pass2_row0(c + 4), true);
-            }
-            wg_barrier();
-        }
+        };
+        // pass 1 walks against the direction of pass 2
+        if (n1max > 0) run_pass(n1max, pass1_row0, false);
+        run_pass(n2max, pass2_row0, true);
         return;
     }
 
     // =========================== consumers ===========================
-#ifdef FTC_TIMELINE
-    typedef __attribute__((address_space(1))) uint64_t gu64;
-    const bool stamp_on = valid && p.nseg > 1 && w == 0 && lane == 0;
-    gu64 *const stamp_base =
-        (gu64 *)((__attribute__((address_space(1))) char *)ws_ptr + kControlBytes +
-                 (int64_t)2 * p.total_waves * (D * F * 4)) + (valid ? sg.ticket : 0) * 16;
-#endif
     FTC_STAMP(0);
     const uint32_t vticket = (uint32_t)w * total_units + (valid ? sg.ticket : 0);
     const uint32_t o_slb = (uint32_t)op.o_sl * 4;
