@@ -321,14 +321,21 @@ def encoder_workload(args):
     x = torch.rand(N, L, D, generator=torch.Generator().manual_seed(4)).cuda()
     mask = TriangularCausalMask(L, device="cuda")
     op_events = []
-    native = cla.causal_dot_product_hip
+    # the native entry points the attention module may call: the fused one (feature map,
+    # mask, product and normaliser in one launch) when it covers the sizes, else the product
+    natives = {name: getattr(cla, name)
+               for name in ("causal_linear_attention_hip", "causal_dot_product_hip")}
+    used = set()
 
-    def timed(*a):
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record()
-        native(*a)
-        e1.record()
-        op_events.append((e0, e1))
+    def timed(name):
+        def call(*a):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            natives[name](*a)
+            e1.record()
+            op_events.append((e0, e1))
+            used.add(name)
+        return call
 
     with torch.no_grad():
         t_ramp = time.perf_counter()
@@ -343,18 +350,22 @@ def encoder_workload(args):
             enc(x, attn_mask=mask)
         torch.cuda.synchronize()
         ms = (time.perf_counter() - t0) * 1e3 / args.steps
-        cla.causal_dot_product_hip = timed
+        for name in natives:
+            setattr(cla, name, timed(name))
         for _ in range(args.steps):
             enc(x, attn_mask=mask)
         torch.cuda.synchronize()
-        cla.causal_dot_product_hip = native
+        for name in natives:
+            setattr(cla, name, natives[name])
     op_ms = sum(a.elapsed_time(b) for a, b in op_events) / args.steps
+    fused = used == {"causal_linear_attention_hip"}
     TH = N * 8 * L
     # roofline of the operator's launches inside the encoder (8 per forward pass, one per
-    # layer): forward only, so 4 E M flops and (2E + 2M) * 4 bytes per position
+    # layer): forward only, so 4 E M flops and (2E + 2M) * 4 bytes per position; the fused
+    # launch also carries the normaliser (4 E flops more) and reads and writes the same rows
     launch_ms = op_ms / 8
     fb, _ = alg_bytes_per_position(64, 64, "f32")
-    launch_bytes, launch_flops = fb * TH, 4 * 64 * 64 * TH
+    launch_bytes, launch_flops = fb * TH, 4 * 64 * (64 + (1 if fused else 0)) * TH
     gbps = launch_bytes / (launch_ms * 1e-3) / 1e9
     tflops = launch_flops / (launch_ms * 1e-3) / 1e12
     t_hbm = launch_bytes / (HBM_PEAK_GBPS * 1e9)
@@ -374,12 +385,15 @@ def encoder_workload(args):
         "data": "synthetic",
         "config": {"workload": "cfg4: 8-layer causal-linear TransformerEncoder eval forward, "
                                "X=rand(10,4096,512), 8 heads, E=M=64, FFN 1024",
+                   "native_entry": sorted(used),
                    "causal_dot_product_ms_per_forward": round(op_ms, 4),
                    "causal_dot_product_share": round(op_ms / ms, 4),
                    "causal_dot_product_fwd_alg_GBps": round(gbps, 1)},
         "roofline": {"bound": bound,
-                     "kernel": "scan_dma_kernel (the operator's forward launch, one per layer; "
-                               "the rest of the encoder is torch's GEMMs and elementwise work)",
+                     "kernel": ("scan_wg_kernel<64,64,NORM> (ftc_causal_linear_attention" if fused
+                                else "scan_dma_kernel (ftc_causal_dot_product")
+                               + ": the operator's forward launch, one per layer; the rest of "
+                                 "the encoder is torch's GEMMs and elementwise work)",
                      "achieved": binding["achieved"], "peak": binding["peak"],
                      "unit": binding["unit"], "frac": binding["frac"],
                      "hbm": hbm_entry, "mfma": mfma_entry,
