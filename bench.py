@@ -39,8 +39,8 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 matrix, published
 # carries it only while the sources are unchanged, otherwise null.
 MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {
     # workload: (bytes, kernel source hash at the time of the measurement)
-    "cfg2": (234721354, "unstamped"),
-    "cfg3": (3186430251, "unstamped"),
+    "cfg2": (234377741, "de4abfaf397a1ec2"),
+    "cfg3": (3188786471, "de4abfaf397a1ec2"),
 }
 
 WORKLOADS = {
@@ -359,11 +359,35 @@ def encoder_workload(args):
             setattr(cla, name, natives[name])
     op_ms = sum(a.elapsed_time(b) for a, b in op_events) / args.steps
     fused = used == {"causal_linear_attention_hip"}
+    # The events above bracket the Python wrapper, so when the GPU has run dry they also see
+    # the host preparing the call.  The launch itself: the same native entry on the
+    # encoder's (N, L, H, 64) layout, back to back over rotating inputs (> 512 MB, cold).
+    with torch.no_grad():
+        gen = torch.Generator(device="cuda").manual_seed(4)
+        sets = [[torch.randn(N, L, 8, 64, device="cuda", generator=gen) for _ in range(3)]
+                + [torch.empty(N, L, 8, 64, device="cuda")] for _ in range(3)]
+        nhl = lambda t: t.permute(0, 2, 1, 3)
+
+        def launch(i):
+            q, k, v, o = sets[i % 3]
+            if fused:
+                natives["causal_linear_attention_hip"](nhl(q), nhl(k), nhl(v), None, 1e-6, nhl(o))
+            else:
+                natives["causal_dot_product_hip"](nhl(q), nhl(k), nhl(v), nhl(o))
+        for i in range(10):
+            launch(i)
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for i in range(60):
+            launch(i)
+        e1.record()
+        torch.cuda.synchronize()
+        launch_ms = e0.elapsed_time(e1) / 60
+        del sets
     TH = N * 8 * L
     # roofline of the operator's launches inside the encoder (8 per forward pass, one per
     # layer): forward only, so 4 E M flops and (2E + 2M) * 4 bytes per position; the fused
     # launch also carries the normaliser (4 E flops more) and reads and writes the same rows
-    launch_ms = op_ms / 8
     fb, _ = alg_bytes_per_position(64, 64, "f32")
     launch_bytes, launch_flops = fb * TH, 4 * 64 * (64 + (1 if fused else 0)) * TH
     gbps = launch_bytes / (launch_ms * 1e-3) / 1e9
@@ -378,7 +402,7 @@ def encoder_workload(args):
     binding = mfma_entry if bound == "mfma" else hbm_entry
     result = {
         "metric": "causal-linear encoder eval forward Mtokens/s (8 layers, d_model 512); "
-                  "causal_dot_product share reported in config",
+                  "share of the native attention launches reported in config",
         "value": round(N * L / (ms * 1e-3) / 1e6, 3), "unit": "Mtokens/s", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
@@ -386,8 +410,9 @@ def encoder_workload(args):
         "config": {"workload": "cfg4: 8-layer causal-linear TransformerEncoder eval forward, "
                                "X=rand(10,4096,512), 8 heads, E=M=64, FFN 1024",
                    "native_entry": sorted(used),
-                   "causal_dot_product_ms_per_forward": round(op_ms, 4),
-                   "causal_dot_product_share": round(op_ms / ms, 4),
+                   "native_launch_ms": round(launch_ms, 5),
+                   "native_share_of_forward": round(8 * launch_ms / ms, 4),
+                   "native_ms_per_forward_bracketed_in_model": round(op_ms, 4),
                    "causal_dot_product_fwd_alg_GBps": round(gbps, 1)},
         "roofline": {"bound": bound,
                      "kernel": ("scan_wg_kernel<64,64,NORM> (ftc_causal_linear_attention" if fused
