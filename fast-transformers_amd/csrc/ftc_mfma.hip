@@ -21,6 +21,21 @@ bool use_wg_kernel(int64_t D, int64_t F, bool all_f32) {
     return false;
 }
 
+// all-fp32 scans with a 64 x 64 state can run one workgroup per chain with no split of L
+// (ftc_tp_kernel.h)
+bool use_tp_kernel(const ScanDesc *scans, int nscans, int64_t chains, int64_t L, bool all_f32) {
+    if (!all_f32 || scans[0].a.width != 64 || scans[0].v.width != 64) return false;
+    // a chain is walked by one workgroup from end to end: beyond 256 chunks the split of L
+    // of the other kernels is faster, and its segment sums also keep the rounding of a long
+    // running state in check
+    if (L > 256 * kChunk) return false;
+    if (const char *env = getenv("FTC_TP")) return atoi(env) != 0;  // tuning aid
+    // One workgroup per chain and scan: worth it once they fill most of the 256 CUs (the
+    // backward of 80 chains does, with its three scans; the forward of 80 chains is faster
+    // split along L).  Measured on cfg2: backward 50 us against 71 us, forward 49 against 46.
+    return chains * nscans >= 160;
+}
+
 // `wg`: the plan is for workgroups of F / 32 wavefronts (each has its own flag words);
 // `norm`: for their fused attention form, with one more wavefront and state slab per unit
 MfmaPlan make_plan(int64_t N, int64_t H, int64_t L, int64_t D, int64_t F, int nscans, bool wg,
@@ -168,8 +183,15 @@ int mfma_scan(const ScanDesc *scans, int nscans, int64_t N, int64_t H, int64_t L
     const Combo combo = combo_of(scans[0]);
     if (fused && (nscans != 1 || !fused_attention_supported(scans[0], L)))
         return fail(FTC_ERR_UNSUPPORTED, "no fused attention kernel for this shape or layout");
+    const bool tp = !fused && use_tp_kernel(scans, nscans, N * H, L, combo == kFFFF);
     const bool wg = fused || use_wg_kernel(D, F, combo == kFFFF);
-    const MfmaPlan pl = make_plan(N, H, L, D, F, nscans, wg, fused != nullptr);
+    MfmaPlan pl = make_plan(N, H, L, D, F, nscans, wg, fused != nullptr);
+    if (tp) {  // one workgroup per chain, nothing to exchange
+        pl.nseg = 1;
+        pl.seg_len = (int)std::min<int64_t>(L, 1 << 30);
+        pl.waves = std::max<int64_t>(1, N * H);
+        pl.workspace_bytes = 0;
+    }
     if (pl.workspace_bytes > 0 && (!workspace || workspace_bytes < (size_t)pl.workspace_bytes))
         return fail(FTC_ERR_WORKSPACE, "workspace of %lld bytes needed, %zu given",
                     (long long)pl.workspace_bytes, workspace_bytes);
@@ -208,6 +230,11 @@ int mfma_scan(const ScanDesc *scans, int nscans, int64_t N, int64_t H, int64_t L
     args.L = L;
     args.eps = fused ? fused->eps : 0.f;
     args.key_len = fused ? fused->key_lengths : nullptr;
+#ifdef FTC_TIMELINE
+    if (tp)  // tuning aid: where the chain-parallel kernel writes its time stamps
+        if (const char *env = getenv("FTC_STAMP_PTR"))
+            args.key_len = (const int64_t *)(uintptr_t)strtoull(env, nullptr, 0);
+#endif
     args.H = (int32_t)H;
     args.seg_len = pl.seg_len;
     args.nseg = pl.nseg;
@@ -232,7 +259,9 @@ int mfma_scan(const ScanDesc *scans, int nscans, int64_t N, int64_t H, int64_t L
     // fp32 states of up to 64 rows: the kernel that feeds its fragments from LDS tiles
     bool dma = D <= 64 && combo == kFFFF;
     if (const char *env = getenv("FTC_DMA")) dma = dma && atoi(env) != 0;  // tuning aid
-    if (wg) {
+    if (tp) {
+        launch_scan_tp(args, stream);
+    } else if (wg) {
         launch_scan_wg_ffff(D, F, fused != nullptr, workspace, args, stream);
     } else if (dma) {
         launch_scan_dma_ffff(D, F, workspace, args, stream);

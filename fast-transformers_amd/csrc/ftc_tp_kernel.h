@@ -1,0 +1,429 @@
+// Chain-parallel form of the MFMA causal scan for gfx950, all-fp32 rows, 64 x 64 state.
+//
+//   out[c, l, f] = sum_{j <= l} (a[c,l,:] . b[c,j,:]) * v[c,j,f]      (REV: j >= l)
+//
+// One workgroup walks one whole chain, chunk after chunk, with no split of L: every row is
+// read once, there is no first pass over a segment, no exchange of states between
+// workgroups, no workspace.  What makes a single chain fast enough is that the work of a
+// chunk is spread over four matrix cores: the 64 x 64 state is held as four slabs of 16
+// columns, one per consumer wavefront (one per SIMD), and the 32 x 32 chunk product Pt is
+// computed once, a quadrant per wavefront, and shared through LDS.
+//
+//  * Wavefronts 4..7 (producers) fetch the rows of a chunk, cut every fp32 value into its
+//    three bf16 pieces and write them as row-major piece tiles into double-buffered LDS,
+//    four chunks ahead (as in ftc_wg_kernel.h).
+//  * Wavefronts 0..3 (consumers), v_mfma_f32_16x16x32_bf16 (A: row = lane % 16, B: column =
+//    lane % 16, both with k-slots t = 0..7 of lane group g = lane / 16; accumulator: column
+//    = lane % 16, rows 4 g + r).  Consumer w owns output columns 16 w .. 16 w + 15:
+//      (1)  Pt quadrant (jh, ih) = b[16 jh ..] a[16 ih ..]^T over d, masked (the quadrant of
+//           the fourth wavefront lies wholly beyond the causal mask: zeros), cut into
+//           pieces and written to LDS as rows i with j contiguous;
+//      (2b) Ot_w  = S_w^T a^T       16 f x 32 i, contraction over d;
+//      (3)  S_w  += b^T v_w         64 d x 16 f, contraction over the chunk's positions j;
+//      -- barrier: all of Pt is in LDS --
+//      (2a) Ot_w += v_w^T Pt        contraction over j;   store Ot_w.
+//    Row m of state tile dt = 2 ks + u stands for d = 32 ks + 8 (m / 4) + 4 u + m % 4 (the
+//    b^T fragments of (3) are read in that column order), so that the accumulator registers
+//    of S_w (column f = lane % 16, rows 4 g + r of tiles 2 ks and 2 ks + 1) are, as they
+//    stand, the A operand of k-step ks of (2b) with k-slots d = 32 ks + 8 g + t -- the order
+//    of a 16-byte read of a row of a or b, whose fragments serve (1) and (2b) alike.
+//  * Two workgroup barriers per chunk: after Pt is written -- by then the producers have
+//    cut the next chunk, whose fragments the consumers request right away, under (2a) --
+//    and at the end of the chunk (Pt and the LDS buffer of the chunk may be overwritten).
+#pragma once
+#include "ftc_wg_kernel.h"
+
+namespace ftc {
+namespace mfma {
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ f32x4 mfma16(const Frag &a, const Frag &b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a),
+                                                   __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+}
+// k-slots 0..3 from the 8 bytes at p0, 4..7 from those at p1
+__device__ __forceinline__ Frag lds_frag8x2(const lds_char *p0, const lds_char *p1) {
+    const u32x2 lo = *(const lds_vec2 *)p0;
+    const u32x2 hi = *(const lds_vec2 *)p1;
+    return Frag{{lo.x, lo.y, hi.x, hi.y}};
+}
+
+// Column order of the b tiles.  Row m of state tile dt = 2 ks + u stands for
+// d = 32 ks + 8 (m / 4) + 4 u + m % 4, and the transposing reads that fetch b^T for such a
+// tile want its 16 columns side by side (two full 16-byte slots per row: free of bank
+// conflicts under the swizzle): within each block of 32 columns the groups of four with
+// u = 0 come first, then those with u = 1.  (d a multiple of 4.)
+__device__ __forceinline__ constexpr int b_tile_column(int d) {
+    return 32 * (d / 32) + 16 * ((d / 4) % 2) + 4 * ((d % 32) / 8) + d % 4;
+}
+
+__global__ __launch_bounds__(512, 2) void scan_tp_kernel(ScanArgs p) {
+    constexpr int D = 64, F = 64;
+    constexpr int T = 256;                     // producer lanes
+    constexpr int PF = 4;                      // chunks requested ahead
+    constexpr int RBA = D * 2, RBV = F * 2;    // bytes per row of a bf16 piece tile
+    constexpr int kTileA = kChunk * RBA, kTileV = kChunk * RBV;
+    constexpr int kOffB = 3 * kTileA, kOffV = 6 * kTileA;
+    constexpr int kBufBytes = 6 * kTileA + 3 * kTileV;
+    constexpr int kTileP = kChunk * 64;        // Pt pieces: 32 rows (i) of 32 j
+    constexpr int QA = D / 4, QV = F / 4;
+    constexpr int LA = kChunk * QA / T, LV = kChunk * QV / T;
+    static_assert(kChunk == 32 && T % QA == 0 && T % QV == 0, "shape");
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const bool producer = wave >= 4;
+    const int w = wave & 3;
+
+    __shared__ __align__(16) char pieces_mem[2 * kBufBytes];
+    __shared__ __align__(16) char pt_mem[3 * kTileP];
+    lds_char *const unit_pc = (lds_char *)pieces_mem;
+    lds_char *const pt_pc = (lds_char *)pt_mem;
+    for (int i = tid; i < 3 * kTileP / 4; i += 512) ((uint32_t *)pt_mem)[i] = 0u;
+
+    // ---- which chain: workgroups of one scan in groups of 8 (one per XCD), the groups of
+    // the scans of a launch side by side, so that scans reading the same rows share an L2 ----
+    const uint32_t chains = (uint32_t)p.waves_per_scan;
+    const uint32_t nscans = (uint32_t)p.total_waves / chains;
+    const uint32_t full = (chains / 8u) * 8u;
+    uint32_t scan_id, chain;
+    if (blockIdx.x < full * nscans) {
+        const uint32_t grp = blockIdx.x / (8u * nscans), r = blockIdx.x % (8u * nscans);
+        scan_id = r / 8u;
+        chain = grp * 8u + r % 8u;
+    } else {
+        const uint32_t t = blockIdx.x - full * nscans;
+        scan_id = t / (chains - full);
+        chain = full + t % (chains - full);
+    }
+    const ScanOperands &op = p.scan[scan_id];
+    const bool REV = op.rev != 0;
+    const int n = (int)(chain / (uint32_t)p.H), h = (int)(chain % (uint32_t)p.H);
+    const int rows = (int)p.L;
+    const int nchunks = (rows + kChunk - 1) / kChunk;
+    auto chunk_row0 = [&](int c) -> int { return REV ? rows - kChunk * (c + 1) : kChunk * c; };
+    __syncthreads();
+#ifdef FTC_TIMELINE
+    // tuning aid: 32 time stamps per workgroup behind the pointer that the host passes in
+    // p.key_len (FTC_STAMP_PTR), written by lane 0 of consumer 0 (0 .. 15) and of producer 0
+    // (16 .. 31) in chunk 4
+    typedef __attribute__((address_space(1))) uint64_t gu64;
+    const bool stamp_on = p.key_len != nullptr && w == 0 && lane == 0;
+    gu64 *const stamp_base = (gu64 *)p.key_len + blockIdx.x * 32 + (producer ? 16 : 0);
+#endif
+
+    if (producer) {
+        // =========================== producers ===========================
+        const int ptid = w * 64 + lane;
+        const uint32_t a_slb = (uint32_t)op.a_sl * 4, b_slb = (uint32_t)op.b_sl * 4,
+                       v_slb = (uint32_t)op.v_sl * 4;
+        const char *a_seg = (const char *)op.a + ((int64_t)n * op.a_sn + (int64_t)h * op.a_sh) * 4;
+        const char *b_seg = (const char *)op.b + ((int64_t)n * op.b_sn + (int64_t)h * op.b_sh) * 4;
+        const char *v_seg = (const char *)op.v + ((int64_t)n * op.v_sn + (int64_t)h * op.v_sh) * 4;
+        const __amdgpu_buffer_rsrc_t a_rs = __builtin_amdgcn_make_buffer_rsrc(
+            (void *)a_seg, 0, (rows - 1) * a_slb + D * 4, kRsrcFlags);
+        const __amdgpu_buffer_rsrc_t b_rs = __builtin_amdgcn_make_buffer_rsrc(
+            (void *)b_seg, 0, (rows - 1) * b_slb + D * 4, kRsrcFlags);
+        const __amdgpu_buffer_rsrc_t v_rs = __builtin_amdgcn_make_buffer_rsrc(
+            (void *)v_seg, 0, (rows - 1) * v_slb + F * 4, kRsrcFlags);
+        uint32_t a_goff[LA], b_goff[LA], v_goff[LV];
+        int a_waddr[LA], b_waddr[LA], v_waddr[LV];
+#pragma unroll
+        for (int q = 0; q < LA; q++) {
+            const int u = q * T + ptid, row = u / QA, c4 = u % QA;
+            a_goff[q] = (uint32_t)row * a_slb + 16u * c4;
+            b_goff[q] = (uint32_t)row * b_slb + 16u * c4;
+            a_waddr[q] = PieceSwizzle<RBA>::addr(row, 8 * c4);
+            b_waddr[q] = PieceSwizzle<RBA>::addr(row, 2 * b_tile_column(4 * c4));
+        }
+#pragma unroll
+        for (int q = 0; q < LV; q++) {
+            const int u = q * T + ptid, row = u / QV, c4 = u % QV;
+            v_goff[q] = (uint32_t)row * v_slb + 16u * c4;
+            v_waddr[q] = PieceSwizzle<RBV>::addr(row, 8 * c4);
+        }
+        struct Raw {
+            u32x4 a[LA], b[LA], v[LV];
+        };
+        Raw raw[PF];
+        // rows of a chunk that does not exist lie outside the descriptor and read as zero
+        auto row0_of = [&](int c) -> int { return c < nchunks ? chunk_row0(c) : -2 * kChunk; };
+        auto fetch = [&](Raw &r, int row0) {
+#pragma unroll
+            for (int q = 0; q < LA; q++) {
+                r.a[q] = __builtin_amdgcn_raw_buffer_load_b128(
+                    a_rs, a_goff[q] + (uint32_t)row0 * a_slb, 0, 0);
+                r.b[q] = __builtin_amdgcn_raw_buffer_load_b128(
+                    b_rs, b_goff[q] + (uint32_t)row0 * b_slb, 0, 0);
+            }
+#pragma unroll
+            for (int q = 0; q < LV; q++)
+                r.v[q] = __builtin_amdgcn_raw_buffer_load_b128(
+                    v_rs, v_goff[q] + (uint32_t)row0 * v_slb, 0, 0);
+        };
+        // The consumers ask for the row-major fragments (a, b) of the next chunk right after
+        // the barrier in the middle of a chunk and for the position-major ones (b again, v)
+        // after the one at its end: a and b are cut before the first, v between the two.
+        auto cut_ab = [&](const Raw &r, int buf) {
+            lds_char *const pc = unit_pc + buf * kBufBytes;
+#pragma unroll
+            for (int q = 0; q < LA; q++) {
+                split_quad_to_lds(r.a[q], pc, kTileA, a_waddr[q]);
+                split_quad_to_lds(r.b[q], pc + kOffB, kTileA, b_waddr[q]);
+            }
+        };
+        auto cut_v = [&](const Raw &r, int buf) {
+            lds_char *const pc = unit_pc + buf * kBufBytes;
+#pragma unroll
+            for (int q = 0; q < LV; q++) split_quad_to_lds(r.v[q], pc + kOffV, kTileV, v_waddr[q]);
+        };
+#pragma unroll
+        for (int j = 0; j < PF; j++) fetch(raw[j], row0_of(j));
+        cut_ab(raw[0], 0);
+        cut_v(raw[0], 0);
+        fetch(raw[0], row0_of(PF));
+        wg_barrier();
+        for (int c = 0; c < nchunks; c += PF) {
+#pragma unroll
+            for (int j = 0; j < PF; j++) {
+                if (c + j == 4) FTC_STAMP(0);
+                if (c + j + 1 < nchunks) cut_ab(raw[(j + 1) % PF], (j + 1) & 1);
+                if (c + j == 4) FTC_STAMP(1);
+                wg_barrier();  // middle of the chunk
+                if (c + j == 4) FTC_STAMP(2);
+                if (c + j + 1 < nchunks) {
+                    cut_v(raw[(j + 1) % PF], (j + 1) & 1);
+                    fetch(raw[(j + 1) % PF], row0_of(c + j + 1 + PF));
+                }
+                if (c + j == 4) FTC_STAMP(3);
+                wg_barrier();  // end of the chunk
+                if (c + j == 4) FTC_STAMP(4);
+                if (c + j + 1 >= nchunks) return;
+            }
+        }
+        return;
+    }
+
+    // =========================== consumers ===========================
+    const int ln = lane & 15, g = lane >> 4;
+    const uint32_t o_slb = (uint32_t)op.o_sl * 4;
+    char *o_seg = (char *)op.out + ((int64_t)n * op.o_sn + (int64_t)h * op.o_sh) * 4;
+    const __amdgpu_buffer_rsrc_t o_rs =
+        __builtin_amdgcn_make_buffer_rsrc((void *)o_seg, 0, (rows - 1) * o_slb + F * 4, kRsrcFlags);
+    // Pt quadrant of this wavefront: the two on the diagonal, the one inside the mask, and
+    // (consumer 3, so that all four run the same instructions) the one outside it: zeros
+    const int jh = w == 0 ? 0 : w == 1 ? 1 : ((w == 2) == REV ? 1 : 0);
+    const int ih = w == 0 ? 0 : w == 1 ? 1 : 1 - jh;
+    // Position tiles are numbered from this wavefront's own: local tile x is tile x ^ ih, so
+    // that the quadrant always multiplies local tile 0.
+    // row-major fragments of a and b: k-slots t <-> d = 32 ks + 8 g + t (one 16-byte read)
+    // (b: its tile keeps the two groups of four apart, see b_tile_column: two 8-byte reads)
+    int a_addr[2][2], b_addr[2][2];  // [local i tile][ks], [ks][u]
+#pragma unroll
+    for (int ks = 0; ks < 2; ks++) {
+#pragma unroll
+        for (int x = 0; x < 2; x++)
+            a_addr[x][ks] = PieceSwizzle<RBA>::addr(16 * (x ^ ih) + ln, 2 * (32 * ks + 8 * g));
+#pragma unroll
+        for (int u = 0; u < 2; u++)
+            b_addr[ks][u] = kOffB + PieceSwizzle<RBA>::addr(
+                                        16 * jh + ln, 2 * b_tile_column(32 * ks + 8 * g + 4 * u));
+    }
+    // State tile dt = 2 ks + u: row m <-> d = 32 ks + 8 (m / 4) + 4 u + m % 4, so that the
+    // accumulator registers of tiles 2 ks and 2 ks + 1 (rows 4 g + r) are k-slots 0..7 of
+    // k-step ks in the order above.
+    // Transposing reads: lane s of a group of 16 supplies 8 bytes (4 columns) of row
+    // 8 g + s / 4 (+ 4); the group's lane i then holds column i % 4 of the group that lane
+    // i / 4 supplied.
+    //  b^T, tile dt: lane i <-> row m = i of the tile, so lane s supplies columns
+    //  32 ks + 4 u + 8 (s % 4) + 0..3;  v: columns 16 w + 4 (s % 4) + 0..3
+    int bt_addr[4][2], vt_addr[2];
+#pragma unroll
+    for (int u2 = 0; u2 < 2; u2++) {
+        const int row = 8 * g + (ln >> 2) + 4 * u2;
+#pragma unroll
+        for (int dt = 0; dt < 4; dt++)
+            bt_addr[dt][u2] = kOffB + PieceSwizzle<RBA>::addr(
+                row, 2 * b_tile_column(32 * (dt / 2) + 4 * (dt % 2) + 8 * (ln & 3)));
+        vt_addr[u2] = kOffV + PieceSwizzle<RBV>::addr(row, 2 * (16 * w + 4 * (ln & 3)));
+    }
+    // Pt in LDS: row i, j contiguous.  Written 4 values at a time (j = 16 jh + 4 g + r), read
+    // as fragments with k-slots j = 8 g + t
+    const int pt_waddr = PieceSwizzle<64>::addr(16 * ih + ln, 2 * (16 * jh + 4 * g));
+    int pt_raddr[2];
+#pragma unroll
+    for (int x = 0; x < 2; x++) pt_raddr[x] = PieceSwizzle<64>::addr(16 * (x ^ ih) + ln, 16 * g);
+    uint32_t keep[4];
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+        const int j = 16 * jh + 4 * g + r, i = 16 * ih + ln;
+        keep[r] = (REV ? (j >= i) : (j <= i)) ? 0xffffffffu : 0u;
+        asm volatile("" : "+v"(keep[r]));
+    }
+    uint32_t o_lane[2];
+#pragma unroll
+    for (int x = 0; x < 2; x++)
+        o_lane[x] = (uint32_t)(16 * (x ^ ih) + ln) * o_slb + 4u * (16 * w + 4 * g);
+
+    f32x4 S[4];
+#pragma unroll
+    for (int dt = 0; dt < 4; dt++) S[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    constexpr int kPa[6] = {0, 1, 2, 0, 1, 0}, kPb[6] = {2, 1, 0, 1, 0, 0};  // piece products
+    // the caller's state: lane (f = 16 w + ln, g), tile dt, register r <-> row d below
+    auto state_row = [&](int dt, int r) -> int { return 32 * (dt / 2) + 8 * g + 4 * (dt % 2) + r; };
+    if (op.s0) {
+        const float *base = op.s0 + (int64_t)n * op.s0_sn + (int64_t)h * op.s0_sh + 16 * w + ln;
+#pragma unroll
+        for (int dt = 0; dt < 4; dt++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) S[dt][r] += base[(int64_t)state_row(dt, r) * op.s0_sd];
+    }
+
+    // A wavefront issues in order, and four of them share the LDS: reads are therefore
+    // written out between the matrix instructions they run under, one at a time, and
+    // scheduling barriers keep the compiler from regrouping them.
+    Frag af[2][2][3], bfr[2][3], bt[4][3], vf[3];
+    // row-major fragment number i of a chunk (18: b for the quadrant first, then a)
+    auto rm_frag = [&](const lds_char *pc, int i) {
+        const int k = i % 3, ks = (i / 3) % 2, x = i / 6;
+        if (x == 0)
+            bfr[ks][k] = lds_frag8x2(pc + k * kTileA + b_addr[ks][0], pc + k * kTileA + b_addr[ks][1]);
+        else
+            af[x - 1][ks][k] = lds_frag16(pc + k * kTileA + a_addr[x - 1][ks]);
+    };
+    // position-major fragment number i of a chunk (15: v first, then b^T tile by tile)
+    auto tr_frag = [&](const lds_char *pc, int i) {
+        if (i < 3)
+            vf[i] = lds_frag_tr(pc + i * kTileV + vt_addr[0], pc + i * kTileV + vt_addr[1]);
+        else {
+            const int dt = (i - 3) / 3, k = (i - 3) % 3;
+            bt[dt][k] = lds_frag_tr(pc + k * kTileA + bt_addr[dt][0], pc + k * kTileA + bt_addr[dt][1]);
+        }
+    };
+
+    wg_barrier();
+#pragma unroll
+    for (int i = 0; i < 18; i++) rm_frag(unit_pc, i);
+    // A matrix instruction that accumulates into the result of the one before it waits for
+    // that result (about twice the issue interval of independent ones), so every phase
+    // below keeps four to six accumulators in turn: the quadrant and Ot_w are summed in
+    // parts (by k-step) that are added at the end, and phases are interleaved.
+    for (int c = 0; c < nchunks; c++) {
+        const lds_char *pc = unit_pc + (c & 1) * kBufBytes;
+        Frag sf[2][3], pf[2][3];
+        f32x4 P4[4], O4[2][2];
+#pragma unroll
+        for (int i = 0; i < 4; i++) P4[i] = O4[i / 2][i % 2] = f32x4{0.f, 0.f, 0.f, 0.f};
+        if (c == 4) FTC_STAMP(0);
+        __builtin_amdgcn_sched_barrier(0);
+        // phase 1: (1) the quadrant; underneath: S_w cut into pieces in A operand order
+        // (slots 0..3 from tile 2 ks, 4..7 from tile 2 ks + 1), first position-major reads
+#pragma unroll
+        for (int i = 0; i < 12; i++) {
+            const int ks = i % 2, m = i / 2;
+            P4[i % 4] = mfma16(bfr[ks][kPa[m]], af[0][ks][kPb[m]], P4[i % 4]);
+            if (i < 8) {
+                const int ks2 = i / 4, q = i % 4;
+                uint32_t o[3];
+                split_pair_under_mfma(S[2 * ks2 + q / 2][2 * (q % 2)],
+                                      S[2 * ks2 + q / 2][2 * (q % 2) + 1], o);
+#pragma unroll
+                for (int k = 0; k < 3; k++) sf[ks2][k].w[q] = o[k];
+            }
+            tr_frag(pc, i);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        if (c == 4) FTC_STAMP(1);
+        // phase 2: first half of (2b) Ot_w = S_w^T a^T; underneath: the last position-major
+        // reads, then the quadrant is added up, masked, cut and handed to the others
+        f32x4 P;
+        uint32_t plo[3], phi[3];
+#pragma unroll
+        for (int i = 0; i < 12; i++) {
+            const int x = i % 2, ks = (i / 2) % 2, m = i / 4;  // piece products 0..2
+            O4[x][ks] = mfma16(sf[ks][kPa[m]], af[x][ks][kPb[m]], O4[x][ks]);
+            if (i < 3) tr_frag(pc, 12 + i);
+            if (i == 4) P = (P4[0] + P4[1]) + (P4[2] + P4[3]);
+            if (i == 6)
+                split_pair_under_mfma(__uint_as_float(__float_as_uint(P[0]) & keep[0]),
+                                      __uint_as_float(__float_as_uint(P[1]) & keep[1]), plo);
+            if (i == 8)
+                split_pair_under_mfma(__uint_as_float(__float_as_uint(P[2]) & keep[2]),
+                                      __uint_as_float(__float_as_uint(P[3]) & keep[3]), phi);
+            if (i == 10) {
+#pragma unroll
+                for (int k = 0; k < 3; k++) {
+                    const u32x2 xk = {plo[k], phi[k]};
+                    *(lds_vec2 *)(pt_pc + k * kTileP + pt_waddr) = xk;
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        if (c == 4) FTC_STAMP(2);
+        // phase 3: second half of (2b) in turn with (3) S_w += b^T v_w for tiles 0 and 1
+#pragma unroll
+        for (int i = 0; i < 12; i++) {
+            const int x = i % 2, ks = (i / 2) % 2, m = 3 + i / 4;  // piece products 3..5
+            O4[x][ks] = mfma16(sf[ks][kPa[m]], af[x][ks][kPb[m]], O4[x][ks]);
+            S[i % 2] = mfma16(bt[i % 2][kPa[i / 2]], vf[kPb[i / 2]], S[i % 2]);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        if (c == 4) FTC_STAMP(3);
+        if (c == 4) FTC_STAMP(4);
+        wg_barrier();
+        if (c == 4) FTC_STAMP(5);
+        // All of Pt is in LDS, and the producers passed this barrier after they had cut the
+        // next chunk: its row-major fragments are requested under what follows.
+        // phase 4: (3) for tiles 2 and 3 in turn with (2a) Ot_w += v_w^T Pt
+        const lds_char *pn = unit_pc + ((c + 1) & 1) * kBufBytes;
+#pragma unroll
+        for (int x = 0; x < 2; x++)
+#pragma unroll
+            for (int k = 0; k < 3; k++) pf[x][k] = lds_frag16(pt_pc + k * kTileP + pt_raddr[x]);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            S[2 + i % 2] = mfma16(bt[2 + i % 2][kPa[i / 2]], vf[kPb[i / 2]], S[2 + i % 2]);
+            if (c + 1 < nchunks) rm_frag(pn, i);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+#pragma unroll
+        for (int i = 0; i < 12; i++) {
+            if (i < 8) {
+                const int t = 4 + i;
+                S[2 + t % 2] = mfma16(bt[2 + t % 2][kPa[t / 2]], vf[kPb[t / 2]], S[2 + t % 2]);
+            }
+            const int x = i % 2, m = i / 2;
+            O4[x][m % 2] = mfma16(vf[kPa[m]], pf[x][kPb[m]], O4[x][m % 2]);
+            if (c + 1 < nchunks) {
+                rm_frag(pn, 4 + i);
+                if (i < 2) rm_frag(pn, 16 + i);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        if (c == 4) FTC_STAMP(6);
+        if (c == 4) FTC_STAMP(7);
+        // lane (i = 16 (x ^ ih) + ln, g) holds f = 16 w + 4 g + 0..3
+        const uint32_t o_off = (uint32_t)chunk_row0(c) * o_slb;
+#pragma unroll
+        for (int x = 0; x < 2; x++) {
+            const f32x4 o = O4[x][0] + O4[x][1];
+            buffer_store4(o_rs, o_off + o_lane[x], o[0], o[1], o[2], o[3]);
+        }
+        if (c == 4) FTC_STAMP(8);
+        wg_barrier();
+        if (c == 4) FTC_STAMP(9);
+    }
+    if (op.s_out) {
+        float *base = op.s_out + (int64_t)n * op.so_sn + (int64_t)h * op.so_sh + 16 * w + ln;
+#pragma unroll
+        for (int dt = 0; dt < 4; dt++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) base[(int64_t)state_row(dt, r) * op.so_sd] = S[dt][r];
+    }
+}
+
+}  // namespace mfma
+}  // namespace ftc

@@ -15,6 +15,8 @@
   product is float32 in both cases (``__init__.py:41`` allocates with the default
   dtype) and the gradients have the dtype of their inputs (``__init__.py:59-61``).
 """
+import os
+
 import torch
 
 from .. import _native
@@ -49,6 +51,12 @@ def _check_out(t, name):
 # One scratch buffer per (device, stream), grown on demand.  The library wants the control
 # block at its start zeroed before the first use and restores it after every call, so the
 # buffer is allocated zero-filled once and then handed to every later call on that stream.
+#
+# The error word of a workspace (byte 8 of the control block) is non-zero after a call that
+# was cut short.  Reading it means waiting for the GPU, so the wrapper does it where that is
+# cheap or asked for: before a cached workspace is replaced by a larger one, and after every
+# call when FTC_CHECK=1 is set in the environment (a debugging mode); ``check_workspaces()``
+# does it on demand.
 _workspaces = {}
 
 
@@ -59,9 +67,16 @@ def _workspace(nbytes, device):
            torch.cuda.current_stream(device).cuda_stream)
     ws = _workspaces.get(key)
     if ws is None or ws.numel() < nbytes:
+        if ws is not None:
+            check_workspaces()  # the old buffer's last word on the calls made with it
         ws = torch.zeros(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
         _workspaces[key] = ws
     return ws, ws.numel()
+
+
+def _after_call():
+    if os.environ.get("FTC_CHECK", "0") not in ("", "0"):
+        check_workspaces()
 
 
 def workspace_error_words():
@@ -108,6 +123,7 @@ def causal_dot_product_hip(queries, keys, values, product):
         rc = lib.ftc_causal_dot_product(dq, dk, dv, do, ws.data_ptr() if ws is not None else None,
                                         nbytes, torch.cuda.current_stream().cuda_stream)
     _native.check(rc, "ftc_causal_dot_product")
+    _after_call()
 
 
 def causal_dot_product_with_state(queries, keys, values, initial_state=None,
@@ -146,6 +162,7 @@ def causal_dot_product_with_state(queries, keys, values, initial_state=None,
                                               ws.data_ptr() if ws is not None else None, nbytes,
                                               torch.cuda.current_stream().cuda_stream)
     _native.check(rc, "ftc_causal_dot_product_state")
+    _after_call()
     return out, s1
 
 
@@ -175,6 +192,7 @@ def causal_dot_backward_hip(queries, keys, values, grad_out, grad_queries, grad_
         rc = lib.ftc_causal_dot_backward(*descs, ws.data_ptr() if ws is not None else None,
                                          nbytes, torch.cuda.current_stream().cuda_stream)
     _native.check(rc, "ftc_causal_dot_backward")
+    _after_call()
 
 
 FTC_ERR_UNSUPPORTED = -2
@@ -220,6 +238,7 @@ def causal_linear_attention_hip(queries, keys, values, key_lengths, eps, out):
             do, ws.data_ptr() if ws is not None else None, nbytes,
             torch.cuda.current_stream().cuda_stream)
     _native.check(rc, "ftc_causal_linear_attention")
+    _after_call()
 
 
 def _cpu_args(name, *tensors):

@@ -646,6 +646,24 @@ def test_dirty_control_block_is_reported_and_healed(cp):
     out = hip_forward(cp, Q, K, V)
     assert scale_error(out, want) <= 1e-4
     cp.check_workspaces()
+    # the debugging mode reads the error word after every call
+    ws.view(torch.int32)[64 + max_waves] = 1000
+    torch.cuda.synchronize()
+    os.environ["FTC_CHECK"] = "1"
+    try:
+        with pytest.raises(RuntimeError, match="cut short"):
+            hip_forward(cp, Q, K, V)
+        out = hip_forward(cp, Q, K, V)         # reset by the check: works again
+        assert scale_error(out, want) <= 1e-4
+    finally:
+        del os.environ["FTC_CHECK"]
+    # and a workspace is checked before a larger one replaces it
+    ws.view(torch.int32)[64 + max_waves] = 1000
+    torch.cuda.synchronize()
+    hip_forward(cp, Q, K, V)
+    with pytest.raises(RuntimeError, match="cut short"):
+        cp._workspace(ws.numel() + 1, ws.device)
+    cp.check_workspaces()
 
 
 def test_errors_and_empty_inputs(cp):
