@@ -23,17 +23,23 @@ bool use_wg_kernel(int64_t D, int64_t F, bool all_f32) {
 
 // all-fp32 scans with a 64 x 64 state can run one workgroup per chain with no split of L
 // (ftc_tp_kernel.h)
-bool use_tp_kernel(const ScanDesc *scans, int nscans, int64_t chains, int64_t L, bool all_f32) {
-    if (!all_f32 || scans[0].a.width != 64 || scans[0].v.width != 64) return false;
+// Returns the number of segments per chain (0: another kernel takes the launch).
+int tp_kernel_segments(const ScanDesc *scans, int nscans, int64_t chains, int64_t L, bool all_f32) {
+    if (!all_f32 || scans[0].a.width != 64 || scans[0].v.width != 64) return 0;
     // a chain is walked by one workgroup from end to end: beyond 256 chunks the split of L
     // of the other kernels is faster, and its segment sums also keep the rounding of a long
     // running state in check
-    if (L > 256 * kChunk) return false;
-    if (const char *env = getenv("FTC_TP")) return atoi(env) != 0;  // tuning aid
-    // One workgroup per chain and scan: worth it once they fill most of the 256 CUs (the
-    // backward of 80 chains does, with its three scans; the forward of 80 chains is faster
-    // split along L).  Measured on cfg2: backward 50 us against 71 us, forward 49 against 46.
-    return chains * nscans >= 160;
+    if (L > 256 * kChunk) return 0;
+    // One workgroup per CU at a time.  A workgroup that takes a whole chain reads every row
+    // once; with fewer chains than CUs a chain is cut into up to four segments whose
+    // workgroups each rebuild the state before their segment by themselves (a state-only
+    // chunk costs about a third of a full one), as long as that fills at least half the GPU.
+    const int64_t units = chains * nscans;
+    const int64_t total_chunks = (L + kChunk - 1) / kChunk;
+    int nseg = (int)std::max<int64_t>(1, std::min<int64_t>(std::min<int64_t>(4, 256 / units), total_chunks));
+    if (const char *env = getenv("FTC_TP_SEGS")) nseg = std::max(1, std::min(atoi(env), 16));  // tuning aid
+    if (const char *env = getenv("FTC_TP")) return atoi(env) != 0 ? nseg : 0;           // tuning aid
+    return units * nseg >= 128 ? nseg : 0;
 }
 
 // `wg`: the plan is for workgroups of F / 32 wavefronts (each has its own flag words);
@@ -183,13 +189,16 @@ int mfma_scan(const ScanDesc *scans, int nscans, int64_t N, int64_t H, int64_t L
     const Combo combo = combo_of(scans[0]);
     if (fused && (nscans != 1 || !fused_attention_supported(scans[0], L)))
         return fail(FTC_ERR_UNSUPPORTED, "no fused attention kernel for this shape or layout");
-    const bool tp = !fused && use_tp_kernel(scans, nscans, N * H, L, combo == kFFFF);
+    const int tp_nseg = fused ? 0 : tp_kernel_segments(scans, nscans, N * H, L, combo == kFFFF);
+    const bool tp = tp_nseg > 0;
     const bool wg = fused || use_wg_kernel(D, F, combo == kFFFF);
     MfmaPlan pl = make_plan(N, H, L, D, F, nscans, wg, fused != nullptr);
-    if (tp) {  // one workgroup per chain, nothing to exchange
-        pl.nseg = 1;
-        pl.seg_len = (int)std::min<int64_t>(L, 1 << 30);
-        pl.waves = std::max<int64_t>(1, N * H);
+    if (tp) {  // one workgroup per chain segment, nothing to exchange
+        const int64_t total_chunks = (L + kChunk - 1) / kChunk;
+        const int64_t seg_chunks = (total_chunks + tp_nseg - 1) / tp_nseg;
+        pl.seg_len = (int)(seg_chunks * kChunk);
+        pl.nseg = (int)((total_chunks + seg_chunks - 1) / seg_chunks);
+        pl.waves = std::max<int64_t>(1, N * H) * pl.nseg;
         pl.workspace_bytes = 0;
     }
     if (pl.workspace_bytes > 0 && (!workspace || workspace_bytes < (size_t)pl.workspace_bytes))
@@ -225,7 +234,8 @@ int mfma_scan(const ScanDesc *scans, int nscans, int64_t N, int64_t H, int64_t L
                                                    std::max(sd.v.stride_l, sd.out.stride_l)));
     }
     // buffer descriptors address a segment with 32-bit byte offsets
-    if ((int64_t)(pl.seg_len + 2 * kChunk) * max_stride * 4 >= 0x7fffffffLL)
+    // (the chain-parallel kernel addresses a whole chain through one descriptor)
+    if ((int64_t)((tp ? L : (int64_t)pl.seg_len) + 2 * kChunk) * max_stride * 4 >= 0x7fffffffLL)
         return fail(FTC_ERR_UNSUPPORTED, "segment too long for 32-bit offsets");
     args.L = L;
     args.eps = fused ? fused->eps : 0.f;

@@ -2,9 +2,12 @@
 //
 //   out[c, l, f] = sum_{j <= l} (a[c,l,:] . b[c,j,:]) * v[c,j,f]      (REV: j >= l)
 //
-// One workgroup walks one whole chain, chunk after chunk, with no split of L: every row is
-// read once, there is no first pass over a segment, no exchange of states between
-// workgroups, no workspace.  What makes a single chain fast enough is that the work of a
+// One workgroup walks one chain, chunk after chunk; nothing is exchanged between workgroups
+// and there is no workspace.  With enough chains a workgroup takes a whole chain and every
+// row is read once.  With fewer, a chain is cut into up to four segments, and the workgroup
+// of a segment first runs the state update alone -- step (3) below, a third of the matrix
+// work and no chunk product -- over the chunks before its own, so that it starts from the
+// same state, bit for bit, that a single walk would have reached.  What makes a single chain fast enough is that the work of a
 // chunk is spread over four matrix cores: the 64 x 64 state is held as four slabs of 16
 // columns, one per consumer wavefront (one per SIMD), and the 32 x 32 chunk product Pt is
 // computed once, a quadrant per wavefront, and shared through LDS.
@@ -85,24 +88,32 @@ __global__ __launch_bounds__(512, 2) void scan_tp_kernel(ScanArgs p) {
 
     // ---- which chain: workgroups of one scan in groups of 8 (one per XCD), the groups of
     // the scans of a launch side by side, so that scans reading the same rows share an L2 ----
-    const uint32_t chains = (uint32_t)p.waves_per_scan;
-    const uint32_t nscans = (uint32_t)p.total_waves / chains;
+    // (also the segments of a chain, which read the same early rows)
+    const uint32_t nseg = (uint32_t)p.nseg;
+    const uint32_t chains = (uint32_t)p.waves_per_scan / nseg;
+    const uint32_t per_chain = (uint32_t)p.total_waves / chains;  // scans x segments
     const uint32_t full = (chains / 8u) * 8u;
-    uint32_t scan_id, chain;
-    if (blockIdx.x < full * nscans) {
-        const uint32_t grp = blockIdx.x / (8u * nscans), r = blockIdx.x % (8u * nscans);
-        scan_id = r / 8u;
+    uint32_t which, chain;
+    if (blockIdx.x < full * per_chain) {
+        const uint32_t grp = blockIdx.x / (8u * per_chain), r = blockIdx.x % (8u * per_chain);
+        which = r / 8u;
         chain = grp * 8u + r % 8u;
     } else {
-        const uint32_t t = blockIdx.x - full * nscans;
-        scan_id = t / (chains - full);
+        const uint32_t t = blockIdx.x - full * per_chain;
+        which = t / (chains - full);
         chain = full + t % (chains - full);
     }
+    const uint32_t scan_id = which / nseg;
+    const int seg = (int)(which % nseg);
     const ScanOperands &op = p.scan[scan_id];
     const bool REV = op.rev != 0;
     const int n = (int)(chain / (uint32_t)p.H), h = (int)(chain % (uint32_t)p.H);
     const int rows = (int)p.L;
-    const int nchunks = (rows + kChunk - 1) / kChunk;
+    // chunks are numbered in walking order; this workgroup's own are c0 .. nchunks - 1, the
+    // ones before them only feed its state
+    const int seg_chunks = p.seg_len / kChunk;
+    const int c0 = seg * seg_chunks;
+    const int nchunks = min((rows + kChunk - 1) / kChunk, c0 + seg_chunks);
     auto chunk_row0 = [&](int c) -> int { return REV ? rows - kChunk * (c + 1) : kChunk * c; };
     __syncthreads();
 #ifdef FTC_TIMELINE
@@ -150,11 +161,18 @@ __global__ __launch_bounds__(512, 2) void scan_tp_kernel(ScanArgs p) {
         Raw raw[PF];
         // rows of a chunk that does not exist lie outside the descriptor and read as zero
         auto row0_of = [&](int c) -> int { return c < nchunks ? chunk_row0(c) : -2 * kChunk; };
-        auto fetch = [&](Raw &r, int row0) {
+        // Every request is made every time, whether its rows exist or not (the chunks before
+        // c0 need no rows of a; chunks past the end have none): a request outside the
+        // descriptor costs no memory traffic, and with a fixed number of requests per chunk
+        // the compiler can wait for the oldest ones only (s_waitcnt vmcnt(n) with n the
+        // number of younger requests) instead of for all of them.
+        auto fetch = [&](Raw &r, int c) {
+            const int row0 = row0_of(c);
+            const int row0_a = c >= c0 ? row0 : -2 * kChunk;
 #pragma unroll
             for (int q = 0; q < LA; q++) {
                 r.a[q] = __builtin_amdgcn_raw_buffer_load_b128(
-                    a_rs, a_goff[q] + (uint32_t)row0 * a_slb, 0, 0);
+                    a_rs, a_goff[q] + (uint32_t)row0_a * a_slb, 0, 0);
                 r.b[q] = __builtin_amdgcn_raw_buffer_load_b128(
                     b_rs, b_goff[q] + (uint32_t)row0 * b_slb, 0, 0);
             }
@@ -166,11 +184,11 @@ __global__ __launch_bounds__(512, 2) void scan_tp_kernel(ScanArgs p) {
         // The consumers ask for the row-major fragments (a, b) of the next chunk right after
         // the barrier in the middle of a chunk and for the position-major ones (b again, v)
         // after the one at its end: a and b are cut before the first, v between the two.
-        auto cut_ab = [&](const Raw &r, int buf) {
+        auto cut_ab = [&](const Raw &r, int buf, int c) {
             lds_char *const pc = unit_pc + buf * kBufBytes;
 #pragma unroll
             for (int q = 0; q < LA; q++) {
-                split_quad_to_lds(r.a[q], pc, kTileA, a_waddr[q]);
+                if (c >= c0) split_quad_to_lds(r.a[q], pc, kTileA, a_waddr[q]);  // (uniform)
                 split_quad_to_lds(r.b[q], pc + kOffB, kTileA, b_waddr[q]);
             }
         };
@@ -180,26 +198,24 @@ __global__ __launch_bounds__(512, 2) void scan_tp_kernel(ScanArgs p) {
             for (int q = 0; q < LV; q++) split_quad_to_lds(r.v[q], pc + kOffV, kTileV, v_waddr[q]);
         };
 #pragma unroll
-        for (int j = 0; j < PF; j++) fetch(raw[j], row0_of(j));
-        cut_ab(raw[0], 0);
+        for (int j = 0; j < PF; j++) fetch(raw[j], j);
+        cut_ab(raw[0], 0, 0);
         cut_v(raw[0], 0);
-        fetch(raw[0], row0_of(PF));
+        fetch(raw[0], PF);
         wg_barrier();
         for (int c = 0; c < nchunks; c += PF) {
 #pragma unroll
             for (int j = 0; j < PF; j++) {
-                if (c + j == 4) FTC_STAMP(0);
-                if (c + j + 1 < nchunks) cut_ab(raw[(j + 1) % PF], (j + 1) & 1);
-                if (c + j == 4) FTC_STAMP(1);
+                if (c + j == c0 + 4) FTC_STAMP(0);
+                cut_ab(raw[(j + 1) % PF], (j + 1) & 1, c + j + 1);  // past the end: zeros
+                if (c + j == c0 + 4) FTC_STAMP(1);
                 wg_barrier();  // middle of the chunk
-                if (c + j == 4) FTC_STAMP(2);
-                if (c + j + 1 < nchunks) {
-                    cut_v(raw[(j + 1) % PF], (j + 1) & 1);
-                    fetch(raw[(j + 1) % PF], row0_of(c + j + 1 + PF));
-                }
-                if (c + j == 4) FTC_STAMP(3);
+                if (c + j == c0 + 4) FTC_STAMP(2);
+                cut_v(raw[(j + 1) % PF], (j + 1) & 1);
+                fetch(raw[(j + 1) % PF], c + j + 1 + PF);
+                if (c + j == c0 + 4) FTC_STAMP(3);
                 wg_barrier();  // end of the chunk
-                if (c + j == 4) FTC_STAMP(4);
+                if (c + j == c0 + 4) FTC_STAMP(4);
                 if (c + j + 1 >= nchunks) return;
             }
         }
@@ -304,19 +320,39 @@ __global__ __launch_bounds__(512, 2) void scan_tp_kernel(ScanArgs p) {
     };
 
     wg_barrier();
+    // ---- the chunks before this workgroup's own: state update only ----
+    for (int c = 0; c < c0; c++) {
+        const lds_char *pc = unit_pc + (c & 1) * kBufBytes;
 #pragma unroll
-    for (int i = 0; i < 18; i++) rm_frag(unit_pc, i);
+        for (int i = 0; i < 15; i++) tr_frag(pc, i);
+#pragma unroll
+        for (int i = 0; i < 24; i++)
+            S[i % 4] = mfma16(bt[i % 4][kPa[i / 4]], vf[kPb[i / 4]], S[i % 4]);
+        wg_barrier();
+        // the producers have cut a and b of the next chunk: if it is the first of our own,
+        // its row-major fragments are due
+        if (c + 1 == c0) {
+            const lds_char *pn = unit_pc + ((c + 1) & 1) * kBufBytes;
+#pragma unroll
+            for (int i = 0; i < 18; i++) rm_frag(pn, i);
+        }
+        wg_barrier();
+    }
+    if (c0 == 0) {
+#pragma unroll
+        for (int i = 0; i < 18; i++) rm_frag(unit_pc, i);
+    }
     // A matrix instruction that accumulates into the result of the one before it waits for
     // that result (about twice the issue interval of independent ones), so every phase
     // below keeps four to six accumulators in turn: the quadrant and Ot_w are summed in
     // parts (by k-step) that are added at the end, and phases are interleaved.
-    for (int c = 0; c < nchunks; c++) {
+    for (int c = c0; c < nchunks; c++) {
         const lds_char *pc = unit_pc + (c & 1) * kBufBytes;
         Frag sf[2][3], pf[2][3];
         f32x4 P4[4], O4[2][2];
 #pragma unroll
         for (int i = 0; i < 4; i++) P4[i] = O4[i / 2][i % 2] = f32x4{0.f, 0.f, 0.f, 0.f};
-        if (c == 4) FTC_STAMP(0);
+        if (c == c0 + 4) FTC_STAMP(0);
         __builtin_amdgcn_sched_barrier(0);
         // phase 1: (1) the quadrant; underneath: S_w cut into pieces in A operand order
         // (slots 0..3 from tile 2 ks, 4..7 from tile 2 ks + 1), first position-major reads
@@ -335,7 +371,7 @@ __global__ __launch_bounds__(512, 2) void scan_tp_kernel(ScanArgs p) {
             tr_frag(pc, i);
             __builtin_amdgcn_sched_barrier(0);
         }
-        if (c == 4) FTC_STAMP(1);
+        if (c == c0 + 4) FTC_STAMP(1);
         // phase 2: first half of (2b) Ot_w = S_w^T a^T; underneath: the last position-major
         // reads, then the quadrant is added up, masked, cut and handed to the others
         f32x4 P;
@@ -361,7 +397,7 @@ __global__ __launch_bounds__(512, 2) void scan_tp_kernel(ScanArgs p) {
             }
             __builtin_amdgcn_sched_barrier(0);
         }
-        if (c == 4) FTC_STAMP(2);
+        if (c == c0 + 4) FTC_STAMP(2);
         // phase 3: second half of (2b) in turn with (3) S_w += b^T v_w for tiles 0 and 1
 #pragma unroll
         for (int i = 0; i < 12; i++) {
@@ -370,10 +406,10 @@ __global__ __launch_bounds__(512, 2) void scan_tp_kernel(ScanArgs p) {
             S[i % 2] = mfma16(bt[i % 2][kPa[i / 2]], vf[kPb[i / 2]], S[i % 2]);
             __builtin_amdgcn_sched_barrier(0);
         }
-        if (c == 4) FTC_STAMP(3);
-        if (c == 4) FTC_STAMP(4);
+        if (c == c0 + 4) FTC_STAMP(3);
+        if (c == c0 + 4) FTC_STAMP(4);
         wg_barrier();
-        if (c == 4) FTC_STAMP(5);
+        if (c == c0 + 4) FTC_STAMP(5);
         // All of Pt is in LDS, and the producers passed this barrier after they had cut the
         // next chunk: its row-major fragments are requested under what follows.
         // phase 4: (3) for tiles 2 and 3 in turn with (2a) Ot_w += v_w^T Pt
@@ -403,8 +439,8 @@ __global__ __launch_bounds__(512, 2) void scan_tp_kernel(ScanArgs p) {
             }
             __builtin_amdgcn_sched_barrier(0);
         }
-        if (c == 4) FTC_STAMP(6);
-        if (c == 4) FTC_STAMP(7);
+        if (c == c0 + 4) FTC_STAMP(6);
+        if (c == c0 + 4) FTC_STAMP(7);
         // lane (i = 16 (x ^ ih) + ln, g) holds f = 16 w + 4 g + 0..3
         const uint32_t o_off = (uint32_t)chunk_row0(c) * o_slb;
 #pragma unroll
@@ -412,11 +448,11 @@ __global__ __launch_bounds__(512, 2) void scan_tp_kernel(ScanArgs p) {
             const f32x4 o = O4[x][0] + O4[x][1];
             buffer_store4(o_rs, o_off + o_lane[x], o[0], o[1], o[2], o[3]);
         }
-        if (c == 4) FTC_STAMP(8);
+        if (c == c0 + 4) FTC_STAMP(8);
         wg_barrier();
-        if (c == 4) FTC_STAMP(9);
+        if (c == c0 + 4) FTC_STAMP(9);
     }
-    if (op.s_out) {
+    if (op.s_out && seg == (int)nseg - 1) {
         float *base = op.s_out + (int64_t)n * op.so_sn + (int64_t)h * op.so_sh + 16 * w + ln;
 #pragma unroll
         for (int dt = 0; dt < 4; dt++)

@@ -439,10 +439,12 @@ __global__ __launch_bounds__(512, 2) void scan_wg_kernel(uint32_t *__restrict__ 
 #pragma unroll
                 for (int j = 0; j < PF; j++) {
                     if (with_a && c + j == 4) FTC_STAMP(5);  // pass 2, fifth chunk
-                    if (c + j + 1 < nmax) {
-                        cut(raw[(j + 1) % PF], (j + 1) & 1, with_a);
-                        fetch(raw[(j + 1) % PF], row0_of(c + j + 1 + PF), with_a);
-                    }
+                    // Made every time, also past the last chunk (requests outside the
+                    // descriptor cost no traffic and return zeros): with a fixed number of
+                    // requests per chunk the compiler waits for the oldest only
+                    // (s_waitcnt vmcnt(n), n younger requests) instead of for all of them.
+                    cut(raw[(j + 1) % PF], (j + 1) & 1, with_a);
+                    fetch(raw[(j + 1) % PF], row0_of(c + j + 1 + PF), with_a);
                     if (with_a && c + j == 4) FTC_STAMP(6);
                     wg_barrier();
                     if (with_a && c + j == 4) FTC_STAMP(7);
