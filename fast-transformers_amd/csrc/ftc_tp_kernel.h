@@ -30,9 +30,11 @@
 //    of S_w (column f = lane % 16, rows 4 g + r of tiles 2 ks and 2 ks + 1) are, as they
 //    stand, the A operand of k-step ks of (2b) with k-slots d = 32 ks + 8 g + t -- the order
 //    of a 16-byte read of a row of a or b, whose fragments serve (1) and (2b) alike.
-//  * Two workgroup barriers per chunk: after Pt is written -- by then the producers have
-//    cut the next chunk, whose fragments the consumers request right away, under (2a) --
-//    and at the end of the chunk (Pt and the LDS buffer of the chunk may be overwritten).
+//  * One workgroup barrier per chunk, after Pt is written.  The piece tiles rotate through
+//    three LDS buffers and Pt through two: when the barrier of chunk c falls, the producers
+//    have cut chunk c + 1 (the consumers request its row-major fragments right away, under
+//    (2a)) and go on to cut chunk c + 2 into the buffer of chunk c - 1, which nobody has
+//    read since the barrier before.
 #pragma once
 #include "ftc_wg_kernel.h"
 
@@ -80,11 +82,10 @@ __global__ __launch_bounds__(512, 2) void scan_tp_kernel(ScanArgs p) {
     const bool producer = wave >= 4;
     const int w = wave & 3;
 
-    __shared__ __align__(16) char pieces_mem[2 * kBufBytes];
-    __shared__ __align__(16) char pt_mem[3 * kTileP];
+    __shared__ __align__(16) char pieces_mem[3 * kBufBytes];
+    __shared__ __align__(16) char pt_mem[2 * 3 * kTileP];
     lds_char *const unit_pc = (lds_char *)pieces_mem;
     lds_char *const pt_pc = (lds_char *)pt_mem;
-    for (int i = tid; i < 3 * kTileP / 4; i += 512) ((uint32_t *)pt_mem)[i] = 0u;
 
     // ---- which chain: workgroups of one scan in groups of 8 (one per XCD), the groups of
     // the scans of a launch side by side, so that scans reading the same rows share an L2 ----
@@ -181,42 +182,34 @@ __global__ __launch_bounds__(512, 2) void scan_tp_kernel(ScanArgs p) {
                 r.v[q] = __builtin_amdgcn_raw_buffer_load_b128(
                     v_rs, v_goff[q] + (uint32_t)row0 * v_slb, 0, 0);
         };
-        // The consumers ask for the row-major fragments (a, b) of the next chunk right after
-        // the barrier in the middle of a chunk and for the position-major ones (b again, v)
-        // after the one at its end: a and b are cut before the first, v between the two.
-        auto cut_ab = [&](const Raw &r, int buf, int c) {
+        // chunk k goes to LDS buffer k % 3 through register set k % PF
+        auto cut = [&](const Raw &r, int buf, int c) {
             lds_char *const pc = unit_pc + buf * kBufBytes;
 #pragma unroll
             for (int q = 0; q < LA; q++) {
                 if (c >= c0) split_quad_to_lds(r.a[q], pc, kTileA, a_waddr[q]);  // (uniform)
                 split_quad_to_lds(r.b[q], pc + kOffB, kTileA, b_waddr[q]);
             }
-        };
-        auto cut_v = [&](const Raw &r, int buf) {
-            lds_char *const pc = unit_pc + buf * kBufBytes;
 #pragma unroll
             for (int q = 0; q < LV; q++) split_quad_to_lds(r.v[q], pc + kOffV, kTileV, v_waddr[q]);
         };
 #pragma unroll
         for (int j = 0; j < PF; j++) fetch(raw[j], j);
-        cut_ab(raw[0], 0, 0);
-        cut_v(raw[0], 0);
-        fetch(raw[0], PF);
-        wg_barrier();
-        for (int c = 0; c < nchunks; c += PF) {
+        // Barrier number k (k = 0: before the first chunk; k >= 1: in the middle of chunk
+        // k - 1) finds chunk k cut.  The last one finds a chunk of zeros.
+        int buf = 0;
+        for (int c = 0; c <= nchunks; c += PF) {
 #pragma unroll
             for (int j = 0; j < PF; j++) {
                 if (c + j == c0 + 4) FTC_STAMP(0);
-                cut_ab(raw[(j + 1) % PF], (j + 1) & 1, c + j + 1);  // past the end: zeros
+                cut(raw[j], buf, c + j);
                 if (c + j == c0 + 4) FTC_STAMP(1);
-                wg_barrier();  // middle of the chunk
+                fetch(raw[j], c + j + PF);
+                buf = buf == 2 ? 0 : buf + 1;
                 if (c + j == c0 + 4) FTC_STAMP(2);
-                cut_v(raw[(j + 1) % PF], (j + 1) & 1);
-                fetch(raw[(j + 1) % PF], c + j + 1 + PF);
+                wg_barrier();
                 if (c + j == c0 + 4) FTC_STAMP(3);
-                wg_barrier();  // end of the chunk
-                if (c + j == c0 + 4) FTC_STAMP(4);
-                if (c + j + 1 >= nchunks) return;
+                if (c + j >= nchunks) return;
             }
         }
         return;
@@ -319,55 +312,62 @@ __global__ __launch_bounds__(512, 2) void scan_tp_kernel(ScanArgs p) {
         }
     };
 
+    auto next_buf = [](int b) -> int { return b == 2 ? 0 : b + 1; };
+    int buf = 0;  // LDS buffer of the chunk at hand
     wg_barrier();
     // ---- the chunks before this workgroup's own: state update only ----
     for (int c = 0; c < c0; c++) {
-        const lds_char *pc = unit_pc + (c & 1) * kBufBytes;
+        const lds_char *pc = unit_pc + buf * kBufBytes;
 #pragma unroll
         for (int i = 0; i < 15; i++) tr_frag(pc, i);
 #pragma unroll
         for (int i = 0; i < 24; i++)
             S[i % 4] = mfma16(bt[i % 4][kPa[i / 4]], vf[kPb[i / 4]], S[i % 4]);
+        buf = next_buf(buf);
         wg_barrier();
-        // the producers have cut a and b of the next chunk: if it is the first of our own,
-        // its row-major fragments are due
+        // the next chunk is cut: if it is the first of our own, its row-major fragments are due
         if (c + 1 == c0) {
-            const lds_char *pn = unit_pc + ((c + 1) & 1) * kBufBytes;
 #pragma unroll
-            for (int i = 0; i < 18; i++) rm_frag(pn, i);
+            for (int i = 0; i < 18; i++) rm_frag(unit_pc + buf * kBufBytes, i);
         }
-        wg_barrier();
     }
     if (c0 == 0) {
 #pragma unroll
         for (int i = 0; i < 18; i++) rm_frag(unit_pc, i);
     }
+    // S_w as pieces in A operand order (slots 0..3 from tile 2 ks, 4..7 from tile 2 ks + 1).
+    // Tiles 0 and 1 are final after phase 3 and are cut under phase 4, tiles 2 and 3 after
+    // phase 4 and are cut under phase 1 of the next chunk.
+    Frag sf[2][3];
+    auto cut_s = [&](int ks, int q) {
+        uint32_t o[3];
+        split_pair_under_mfma(S[2 * ks + q / 2][2 * (q % 2)], S[2 * ks + q / 2][2 * (q % 2) + 1], o);
+#pragma unroll
+        for (int k = 0; k < 3; k++) sf[ks][k].w[q] = o[k];
+    };
+#pragma unroll
+    for (int q = 0; q < 4; q++) cut_s(0, q);
+
     // A matrix instruction that accumulates into the result of the one before it waits for
     // that result (about twice the issue interval of independent ones), so every phase
     // below keeps four to six accumulators in turn: the quadrant and Ot_w are summed in
-    // parts (by k-step) that are added at the end, and phases are interleaved.
+    // parts that are added at the end, and phases are interleaved.
     for (int c = c0; c < nchunks; c++) {
-        const lds_char *pc = unit_pc + (c & 1) * kBufBytes;
-        Frag sf[2][3], pf[2][3];
+        const lds_char *pc = unit_pc + buf * kBufBytes;
+        lds_char *const ptc = pt_pc + (c & 1) * (3 * kTileP);
+        Frag pf[2][3];
         f32x4 P4[4], O4[2][2];
 #pragma unroll
         for (int i = 0; i < 4; i++) P4[i] = O4[i / 2][i % 2] = f32x4{0.f, 0.f, 0.f, 0.f};
         if (c == c0 + 4) FTC_STAMP(0);
         __builtin_amdgcn_sched_barrier(0);
-        // phase 1: (1) the quadrant; underneath: S_w cut into pieces in A operand order
-        // (slots 0..3 from tile 2 ks, 4..7 from tile 2 ks + 1), first position-major reads
+        // phase 1: (1) the quadrant; underneath: tiles 2, 3 of S_w cut into pieces, and the
+        // first position-major reads
 #pragma unroll
         for (int i = 0; i < 12; i++) {
             const int ks = i % 2, m = i / 2;
             P4[i % 4] = mfma16(bfr[ks][kPa[m]], af[0][ks][kPb[m]], P4[i % 4]);
-            if (i < 8) {
-                const int ks2 = i / 4, q = i % 4;
-                uint32_t o[3];
-                split_pair_under_mfma(S[2 * ks2 + q / 2][2 * (q % 2)],
-                                      S[2 * ks2 + q / 2][2 * (q % 2) + 1], o);
-#pragma unroll
-                for (int k = 0; k < 3; k++) sf[ks2][k].w[q] = o[k];
-            }
+            if (i < 4) cut_s(1, i);
             tr_frag(pc, i);
             __builtin_amdgcn_sched_barrier(0);
         }
@@ -392,7 +392,7 @@ __global__ __launch_bounds__(512, 2) void scan_tp_kernel(ScanArgs p) {
 #pragma unroll
                 for (int k = 0; k < 3; k++) {
                     const u32x2 xk = {plo[k], phi[k]};
-                    *(lds_vec2 *)(pt_pc + k * kTileP + pt_waddr) = xk;
+                    *(lds_vec2 *)(ptc + k * kTileP + pt_waddr) = xk;
                 }
             }
             __builtin_amdgcn_sched_barrier(0);
@@ -407,21 +407,23 @@ __global__ __launch_bounds__(512, 2) void scan_tp_kernel(ScanArgs p) {
             __builtin_amdgcn_sched_barrier(0);
         }
         if (c == c0 + 4) FTC_STAMP(3);
-        if (c == c0 + 4) FTC_STAMP(4);
+        buf = next_buf(buf);
         wg_barrier();
-        if (c == c0 + 4) FTC_STAMP(5);
-        // All of Pt is in LDS, and the producers passed this barrier after they had cut the
-        // next chunk: its row-major fragments are requested under what follows.
-        // phase 4: (3) for tiles 2 and 3 in turn with (2a) Ot_w += v_w^T Pt
-        const lds_char *pn = unit_pc + ((c + 1) & 1) * kBufBytes;
+        if (c == c0 + 4) FTC_STAMP(4);
+        // All of Pt is in LDS and the next chunk is cut: its row-major fragments are
+        // requested under what follows.
+        // phase 4: (3) for tiles 2 and 3 in turn with (2a) Ot_w += v_w^T Pt; underneath:
+        // tiles 0, 1 of S_w cut into pieces
+        const lds_char *pn = unit_pc + buf * kBufBytes;
 #pragma unroll
         for (int x = 0; x < 2; x++)
 #pragma unroll
-            for (int k = 0; k < 3; k++) pf[x][k] = lds_frag16(pt_pc + k * kTileP + pt_raddr[x]);
+            for (int k = 0; k < 3; k++) pf[x][k] = lds_frag16(ptc + k * kTileP + pt_raddr[x]);
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int i = 0; i < 4; i++) {
             S[2 + i % 2] = mfma16(bt[2 + i % 2][kPa[i / 2]], vf[kPb[i / 2]], S[2 + i % 2]);
+            cut_s(0, i);
             if (c + 1 < nchunks) rm_frag(pn, i);
             __builtin_amdgcn_sched_barrier(0);
         }
@@ -439,8 +441,7 @@ __global__ __launch_bounds__(512, 2) void scan_tp_kernel(ScanArgs p) {
             }
             __builtin_amdgcn_sched_barrier(0);
         }
-        if (c == c0 + 4) FTC_STAMP(6);
-        if (c == c0 + 4) FTC_STAMP(7);
+        if (c == c0 + 4) FTC_STAMP(5);
         // lane (i = 16 (x ^ ih) + ln, g) holds f = 16 w + 4 g + 0..3
         const uint32_t o_off = (uint32_t)chunk_row0(c) * o_slb;
 #pragma unroll
@@ -448,9 +449,7 @@ __global__ __launch_bounds__(512, 2) void scan_tp_kernel(ScanArgs p) {
             const f32x4 o = O4[x][0] + O4[x][1];
             buffer_store4(o_rs, o_off + o_lane[x], o[0], o[1], o[2], o[3]);
         }
-        if (c == c0 + 4) FTC_STAMP(8);
-        wg_barrier();
-        if (c == c0 + 4) FTC_STAMP(9);
+        if (c == c0 + 4) FTC_STAMP(6);
     }
     if (op.s_out && seg == (int)nseg - 1) {
         float *base = op.s_out + (int64_t)n * op.so_sn + (int64_t)h * op.so_sh + 16 * w + ln;
