@@ -189,6 +189,12 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
+    # which kernels the planner picks for this workload
+    fwd(0)
+    fwd_kernel = lib.ftc_last_kernel().decode()
+    bwd(0)
+    bwd_kernel = lib.ftc_last_kernel().decode()
+
     # set-up: a fresh GPU takes a few hundred milliseconds of load to reach its clocks
     t_ramp = time.perf_counter()
     i = 0
@@ -283,11 +289,8 @@ def main():
                    "fwdbwd_frac_of_hbm_roofline":
                        round((fb + bb) * TH / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)},
         "roofline": {"bound": bound,
-                     "kernel": ("scan_wg_kernel" if os.environ.get("FTC_WG", "0") == "1"
-                                and dtype == "f32" and max(E, M) <= 128
-                                else "scan_dma_kernel" if dtype == "f32" and max(E, M) <= 64
-                                else "scan_mfma_kernel")
-                               + " (mean over the forward and the backward call)",
+                     "kernel": "forward: %s, backward: %s (mean over the two launches)"
+                               % (fwd_kernel, bwd_kernel),
                      "achieved": binding["achieved"], "peak": binding["peak"],
                      "unit": binding["unit"], "frac": binding["frac"],
                      "hbm": hbm_entry, "mfma": mfma_entry,

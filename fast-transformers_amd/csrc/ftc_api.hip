@@ -25,6 +25,9 @@ namespace ftc {
 
 static thread_local char g_error[512] = "";
 
+static thread_local const char *g_kernel = "";
+void note_kernel(const char *name) { g_kernel = name; }
+
 int fail(int code, const char *fmt, ...) {
     va_list ap;
     va_start(ap, fmt);
@@ -165,6 +168,8 @@ extern "C" {
 int ftc_version(void) { return 1000; }
 
 const char *ftc_last_error(void) { return g_error; }
+
+const char *ftc_last_kernel(void) { return g_kernel; }
 
 int64_t ftc_causal_dot_product_workspace_bytes(int64_t N, int64_t H, int64_t L, int64_t E,
                                                int64_t M, int32_t dtype) {

@@ -42,6 +42,8 @@ inline OperandOut as_operand_out(const ftc_tensor4 *t) {
 
 // Records the message returned by ftc_last_error() and returns `code`.
 int fail(int code, const char *fmt, ...);
+// Records which kernel the last launch on this thread used (ftc_last_kernel()).
+void note_kernel(const char *name);
 
 // bf16 <-> fp32 with round-to-nearest-even (finite inputs; NaN stays NaN).
 __device__ __forceinline__ float bf16_to_f32(uint16_t b) {

@@ -298,6 +298,7 @@ int generic_scan(const Operand &a, const Operand &b, const Operand &v, const Ope
                  int64_t N, int64_t H, int64_t L, bool reverse, const StateRef &initial,
                  const StateRef &final_, void *workspace, size_t workspace_bytes,
                  hipStream_t stream) {
+    note_kernel("generic_scan_kernel");
     const int64_t D = a.width, F = v.width;
     if (D < 1 || F < 1 || D > kGenericMaxDim || F > kGenericMaxDim)
         return fail(FTC_ERR_UNSUPPORTED, "row widths must be in [1, %d] (got %lld and %lld)",

@@ -15,10 +15,13 @@ struct MfmaPlan {
 };
 
 // all-fp32 scans of these widths run as workgroups of F / 32 wavefronts (ftc_wg_kernel.h)
-bool use_wg_kernel(int64_t D, int64_t F, bool all_f32) {
+bool use_wg_kernel(int64_t D, int64_t F, int nscans, int64_t L, bool all_f32) {
     if (!all_f32 || !scan_wg_covers((int)D, (int)F)) return false;
     if (const char *env = getenv("FTC_WG")) return atoi(env) != 0;  // tuning aid
-    return false;
+    // Measured: a single scan over long chains (the forward) is 2-7 % faster in workgroup
+    // form (cfg3 forward 331 us against 349, N=8, H=16, L=4096: 164 against 177); launches of
+    // three scans and short chains are faster with one wavefront per segment.
+    return nscans == 1 && L >= 128 * kChunk && D == 64 && F == 64;
 }
 
 // all-fp32 scans with a 64 x 64 state can run one workgroup per chain with no split of L
@@ -198,7 +201,7 @@ int mfma_scan(const ScanDesc *scans, int nscans, int64_t N, int64_t H, int64_t L
         return fail(FTC_ERR_UNSUPPORTED, "no fused attention kernel for this shape or layout");
     const int tp_nseg = fused ? 0 : tp_kernel_segments(scans, nscans, N * H, L, combo == kFFFF);
     const bool tp = tp_nseg > 0;
-    const bool wg = fused || use_wg_kernel(D, F, combo == kFFFF);
+    const bool wg = fused || use_wg_kernel(D, F, nscans, L, combo == kFFFF);
     MfmaPlan pl = make_plan(N, H, L, D, F, nscans, wg, fused != nullptr);
     if (tp) {  // one workgroup per chain segment, nothing to exchange
         const int64_t total_chunks = (L + kChunk - 1) / kChunk;
@@ -276,6 +279,8 @@ int mfma_scan(const ScanDesc *scans, int nscans, int64_t N, int64_t H, int64_t L
     // fp32 states of up to 64 rows: the kernel that feeds its fragments from LDS tiles
     bool dma = D <= 64 && combo == kFFFF;
     if (const char *env = getenv("FTC_DMA")) dma = dma && atoi(env) != 0;  // tuning aid
+    note_kernel(tp ? "scan_tp_kernel" : wg ? (fused ? "scan_wg_kernel<NORM>" : "scan_wg_kernel")
+                : dma ? "scan_dma_kernel" : "scan_mfma_kernel");
     if (tp) {
         launch_scan_tp(args, stream);
     } else if (wg) {

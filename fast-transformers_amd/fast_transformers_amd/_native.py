@@ -21,6 +21,7 @@ _DTYPE_CODE = {torch.float32: FTC_F32, torch.bfloat16: FTC_BF16}
 EXPORTED_SYMBOLS = (
     "ftc_version",
     "ftc_last_error",
+    "ftc_last_kernel",
     "ftc_workspace_reset",
     "ftc_causal_dot_product_workspace_bytes",
     "ftc_causal_dot_product",
@@ -61,6 +62,8 @@ def load():
     lib.ftc_version.argtypes = []
     lib.ftc_last_error.restype = ctypes.c_char_p
     lib.ftc_last_error.argtypes = []
+    lib.ftc_last_kernel.restype = ctypes.c_char_p
+    lib.ftc_last_kernel.argtypes = []
     for name in ("ftc_causal_dot_product_workspace_bytes",
                  "ftc_causal_dot_backward_workspace_bytes",
                  "ftc_causal_linear_attention_workspace_bytes"):

@@ -74,6 +74,13 @@ int ftc_version(void);
 const char *ftc_last_error(void);
 
 /*
+ * Name of the kernel that the last launch made from this thread used ("" before the first):
+ * which of the library's scan kernels the planner chose for the sizes at hand.  For
+ * measurement and profiling; no counterpart in the reference.
+ */
+const char *ftc_last_kernel(void);
+
+/*
  * Clears the control block of a workspace (a fill kernel enqueued on `stream`; no memset, so
  * it may be captured in a graph).  No counterpart in the reference.  A workspace needs this
  * once before its first use unless it was allocated zero-filled, and again after a call whose

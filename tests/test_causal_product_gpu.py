@@ -666,6 +666,63 @@ def test_dirty_control_block_is_reported_and_healed(cp):
     cp.check_workspaces()
 
 
+TP_SHAPES = [
+    # N, H, L: enough chains for one workgroup per chain (and scan), or few enough that a
+    # chain is cut into segments whose workgroups rebuild their starting state
+    (16, 8, 1), (16, 8, 31), (20, 8, 33), (3, 16, 1000), (40, 4, 97), (2, 32, 2048), (9, 7, 640),
+]
+
+
+@pytest.mark.parametrize("shape", TP_SHAPES, ids=lambda s: "n%d_h%d_l%d" % s)
+def test_chain_parallel_kernel(cp, shape):
+    """The kernel that walks a chain with one workgroup (64 x 64 states, fp32): whole chains
+    and cut chains, ragged ends, both directions, (N, L, H, X) views, against the CPU checker
+    anchored on float64."""
+    from fast_transformers_amd import _native
+    N, H, L = shape
+    E = M = 64
+    Q, K, V, G = oracle.make_inputs(N, H, L, E, M, seed=300 + L)
+    nlh = lambda t: t.permute(0, 2, 1, 3).contiguous().cuda().permute(0, 2, 1, 3)  # NLHE storage
+    q, k, v, g = (nlh(t) for t in (Q, K, V, G))
+    out = torch.full((N, L, H, M), float("nan"), device="cuda").permute(0, 2, 1, 3)
+    cp.causal_dot_product_hip(q, k, v, out)
+    assert _native.load().ftc_last_kernel() == b"scan_tp_kernel"
+    dq, dk, dv = (torch.full((N, L, H, X), float("nan"), device="cuda").permute(0, 2, 1, 3)
+                  for X in (E, E, M))
+    cp.causal_dot_backward_hip(q, k, v, g, dq, dk, dv)
+    assert _native.load().ftc_last_kernel() == b"scan_tp_kernel"
+    torch.cuda.synchronize()
+    want = oracle.forward(Q, K, V)
+    exact = oracle.forward(Q.double(), K.double(), V.double())
+    _gate_against_float64("tp %s product" % (shape,), out.cpu(), want, exact)
+    refs = oracle.backward(Q, K, V, G)
+    exacts = oracle.backward(Q.double(), K.double(), V.double(), G.double())
+    for name, got, ref, ex in zip(("dQ", "dK", "dV"), (dq, dk, dv), refs, exacts):
+        _gate_against_float64("tp %s %s" % (shape, name), got.cpu(), ref, ex)
+
+
+def test_chain_parallel_kernel_cut_chains_equal_whole_chains(cp):
+    """A chain cut into segments starts every segment from the state a single walk reaches,
+    computed in the same order: the results are the same bit for bit however it is cut."""
+    N, H, L = 6, 8, 1500
+    Q, K, V, G = (t.cuda() for t in oracle.make_inputs(N, H, L, 64, 64, seed=17))
+    outs = []
+    for segs in ("1", "2", "4"):
+        os.environ["FTC_TP"], os.environ["FTC_TP_SEGS"] = "1", segs
+        try:
+            out = torch.empty(N, H, L, 64, device="cuda")
+            cp.causal_dot_product_hip(Q, K, V, out)
+            grads = [torch.empty(N, H, L, 64, device="cuda") for _ in range(3)]
+            cp.causal_dot_backward_hip(Q, K, V, G, *grads)
+            torch.cuda.synchronize()
+            outs.append([out] + grads)
+        finally:
+            del os.environ["FTC_TP"], os.environ["FTC_TP_SEGS"]
+    for other in outs[1:]:
+        for a, b in zip(outs[0], other):
+            assert torch.equal(a, b)
+
+
 def test_errors_and_empty_inputs(cp):
     Q = torch.rand(1, 2, 8, 4, device="cuda")
     V = torch.rand(1, 2, 8, 6, device="cuda")
