@@ -34,13 +34,13 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 matrix, published
 # HBM-side bytes per scan-kernel launch (mean of the forward and the backward launch) from
 # rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script, scaled by what the same
 # counters read for the 256 MiB copy of --calibrate-copy; the runs are summarised in
-# profiles/scan_dma_kernel_<workload>_traffic.md.  Each figure is stamped with the hash of
+# profiles/*_<workload>_traffic.md.  Each figure is stamped with the hash of
 # the kernel sources it was measured with (kernel_source_hash() below): the JSON line
 # carries it only while the sources are unchanged, otherwise null.
 MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {
     # workload: (bytes, kernel source hash at the time of the measurement)
-    "cfg2": (234377741, "de4abfaf397a1ec2"),
-    "cfg3": (3188786471, "de4abfaf397a1ec2"),
+    "cfg2": (136686655, "c4e2a3bf1241df80"),
+    "cfg3": (3154159844, "c4e2a3bf1241df80"),
 }
 
 WORKLOADS = {
