@@ -424,7 +424,7 @@ __global__ __launch_bounds__(512, 2) void scan_tp_kernel(ScanArgs p) {
         for (int i = 0; i < 4; i++) {
             S[2 + i % 2] = mfma16(bt[2 + i % 2][kPa[i / 2]], vf[kPb[i / 2]], S[2 + i % 2]);
             cut_s(0, i);
-            if (c + 1 < nchunks) rm_frag(pn, i);
+            rm_frag(pn, i);  // (past the last chunk: a buffer of zeros)
             __builtin_amdgcn_sched_barrier(0);
         }
 #pragma unroll
@@ -435,10 +435,8 @@ __global__ __launch_bounds__(512, 2) void scan_tp_kernel(ScanArgs p) {
             }
             const int x = i % 2, m = i / 2;
             O4[x][m % 2] = mfma16(vf[kPa[m]], pf[x][kPb[m]], O4[x][m % 2]);
-            if (c + 1 < nchunks) {
-                rm_frag(pn, 4 + i);
-                if (i < 2) rm_frag(pn, 16 + i);
-            }
+            rm_frag(pn, 4 + i);
+            if (i < 2) rm_frag(pn, 16 + i);
             __builtin_amdgcn_sched_barrier(0);
         }
         if (c == c0 + 4) FTC_STAMP(5);
