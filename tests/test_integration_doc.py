@@ -1,5 +1,6 @@
-"""The reference-side binding shown in INTEGRATION.md (section 3) is executed as written and
-checked against the CPU checker: the stub a maintainer would paste must actually work."""
+"""The reference-side binding that the integration notes at the repository root show (their
+section 3: a ctypes stub over the C ABI) is executed as written and checked against the CPU
+checker: the stub a maintainer would paste must actually work."""
 import os
 import re
 
