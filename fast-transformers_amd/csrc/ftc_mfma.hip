@@ -199,7 +199,15 @@ int mfma_scan(const ScanDesc *scans, int nscans, int64_t N, int64_t H, int64_t L
     const Combo combo = combo_of(scans[0]);
     if (fused && (nscans != 1 || !fused_attention_supported(scans[0], L)))
         return fail(FTC_ERR_UNSUPPORTED, "no fused attention kernel for this shape or layout");
-    const int tp_nseg = fused ? 0 : tp_kernel_segments(scans, nscans, N * H, L, combo == kFFFF);
+    // the chain-parallel kernel addresses a whole chain through one 32-bit descriptor
+    int64_t widest_stride = 0;
+    for (int i = 0; i < nscans; i++)
+        widest_stride = std::max(widest_stride,
+                                 std::max(std::max(scans[i].a.stride_l, scans[i].b.stride_l),
+                                          std::max(scans[i].v.stride_l, scans[i].out.stride_l)));
+    const bool chain_fits = (L + 2 * kChunk) * widest_stride * 4 < 0x7fffffffLL;
+    const int tp_nseg = fused || !chain_fits
+                            ? 0 : tp_kernel_segments(scans, nscans, N * H, L, combo == kFFFF);
     const bool tp = tp_nseg > 0;
     const bool wg = fused || use_wg_kernel(D, F, nscans, L, combo == kFFFF);
     MfmaPlan pl = make_plan(N, H, L, D, F, nscans, wg, fused != nullptr);
@@ -244,7 +252,6 @@ int mfma_scan(const ScanDesc *scans, int nscans, int64_t N, int64_t H, int64_t L
                                                    std::max(sd.v.stride_l, sd.out.stride_l)));
     }
     // buffer descriptors address a segment with 32-bit byte offsets
-    // (the chain-parallel kernel addresses a whole chain through one descriptor)
     if ((int64_t)((tp ? L : (int64_t)pl.seg_len) + 2 * kChunk) * max_stride * 4 >= 0x7fffffffLL)
         return fail(FTC_ERR_UNSUPPORTED, "segment too long for 32-bit offsets");
     args.L = L;

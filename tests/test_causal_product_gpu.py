@@ -701,6 +701,27 @@ def test_chain_parallel_kernel(cp, shape):
         _gate_against_float64("tp %s %s" % (shape, name), got.cpu(), ref, ex)
 
 
+def test_rows_far_apart_leave_the_chain_parallel_kernel(cp):
+    """A chain of 8192 rows that lie 65536 elements apart does not fit the 32-bit descriptor
+    that the chain-parallel kernel uses for a whole chain: the planner takes another kernel."""
+    from fast_transformers_amd import _native
+    N, H, L, E, M = 1, 144, 8192, 64, 64
+    cols = torch.rand(L, E + E + M, generator=torch.Generator().manual_seed(5))
+    wide = torch.empty(L, 65536, device="cuda")     # 2 GiB, only 192 columns are used
+    wide[:, :E + E + M] = cols.cuda()
+    # every chain reads its rows out of the same wide matrix (stride 0 over N and H)
+    dv = lambda c0, X: wide[:, c0:c0 + X][None, None].expand(N, H, L, X)
+    out = torch.empty(N, H, L, M, device="cuda")
+    cp.causal_dot_product_hip(dv(0, E), dv(E, E), dv(2 * E, M), out)
+    assert _native.load().ftc_last_kernel() != b"scan_tp_kernel"
+    torch.cuda.synchronize()
+    one = lambda c0, X: cols[:, c0:c0 + X][None, None].contiguous()
+    want = oracle.forward(one(0, E), one(E, E), one(2 * E, M))
+    assert scale_error(out[:, :1].cpu(), want) <= 1e-4
+    assert torch.equal(out[:, 0], out[:, 143])
+    del wide
+
+
 def test_chain_parallel_kernel_cut_chains_equal_whole_chains(cp):
     """A chain cut into segments starts every segment from the state a single walk reaches,
     computed in the same order: the results are the same bit for bit however it is cut."""
