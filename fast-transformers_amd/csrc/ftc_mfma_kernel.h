@@ -448,6 +448,10 @@ __device__ __forceinline__ void store_caller_state(float *base, int64_t row_stri
 }
 constexpr int kMaxScans = kMfmaMaxScans;
 
+constexpr int kMaxTpSegments = 16;
+// chunks that the chain-parallel kernel requests ahead (measured on cfg2: 6 and 8 are slower)
+constexpr int kTpAhead = 4;
+
 struct ScanArgs {
     ScanOperands scan[kMaxScans];
     int64_t L;
@@ -458,6 +462,9 @@ struct ScanArgs {
     // fused attention form of the workgroup kernel only (ftc_wg_kernel.h, NORM)
     float eps;               // added to the denominator
     const int64_t *key_len;  // keys per batch entry, N values on the device; nullptr: all L
+    // chain-parallel kernel only (ftc_tp_kernel.h): segment s of a chain is chunks
+    // tp_start[s] .. tp_start[s + 1] - 1 (starts are multiples of kTpAhead)
+    int32_t tp_start[kMaxTpSegments + 1];
 };
 
 // Which (scan, chain, L-segment) a wavefront works on.

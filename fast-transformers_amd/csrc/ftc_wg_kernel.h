@@ -435,7 +435,11 @@ __global__ __launch_bounds__(512, 2) void scan_wg_kernel(uint32_t *__restrict__ 
             cut(raw[0], 0, with_a);
             fetch(raw[0], row0_of(PF), with_a);
             wg_barrier();
-            for (int c = 0; c < nmax; c += PF) {
+            // Whole trips in the loop, the rest after it: a way out of the middle of the loop
+            // would join the paths at the loop's head, and the compiler would then wait for
+            // every request at the head instead of counting.
+            int c = 0;
+            for (; c + PF <= nmax; c += PF) {
 #pragma unroll
                 for (int j = 0; j < PF; j++) {
                     if (with_a && c + j == 4) FTC_STAMP(5);  // pass 2, fifth chunk
@@ -447,9 +451,15 @@ __global__ __launch_bounds__(512, 2) void scan_wg_kernel(uint32_t *__restrict__ 
                     fetch(raw[(j + 1) % PF], row0_of(c + j + 1 + PF), with_a);
                     if (with_a && c + j == 4) FTC_STAMP(6);
                     wg_barrier();
+                    __builtin_amdgcn_sched_barrier(0);  // one chunk at a time, in this order
                     if (with_a && c + j == 4) FTC_STAMP(7);
-                    if (c + j + 1 >= nmax) return;
                 }
+            }
+#pragma unroll
+            for (int j = 0; j < PF - 1; j++) {
+                if (c + j >= nmax) return;
+                cut(raw[(j + 1) % PF], (j + 1) & 1, with_a);
+                wg_barrier();
             }
         };
         // pass 1 walks against the direction of pass 2
