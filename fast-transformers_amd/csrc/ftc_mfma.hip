@@ -54,14 +54,14 @@ int tp_kernel_segments(const ScanDesc *scans, int nscans, int64_t chains, int64_
 
 // Where to cut a chain of `chunks` chunks into (at most) `nseg` segments for the
 // chain-parallel kernel.  The workgroup of a segment first rebuilds the state before its
-// segment from the chunks in front of it (measured: 0.45 of the time of a chunk that also
-// produces rows), so later segments are made shorter until all workgroups finish together:
+// segment from the chunks in front of it (measured: 0.35 to 0.45 of the time of a chunk that
+// also produces rows), so later segments are made shorter until all workgroups finish together:
 // the starts (multiples of kTpAhead chunks, what the producers request ahead) that minimise the
 // longest workgroup.  Returns the number of segments; start[0 .. n] filled (start[n] = chunks).
 int tp_segment_starts(int64_t chunks, int nseg, int32_t *start) {
     const int groups = (int)((chunks + kTpAhead - 1) / kTpAhead);
     nseg = std::max(1, std::min(std::min(nseg, groups), kMaxTpSegments));
-    double kStateOnly = 0.45;
+    double kStateOnly = 0.4;
     if (const char *env = getenv("FTC_TP_RATIO")) kStateOnly = atof(env);  // tuning aid
     // best[s][g]: smallest achievable longest time of segments s .. nseg-1 when segment s
     // starts at group g (dynamic programme from the last segment back)

@@ -186,39 +186,43 @@ __global__ __launch_bounds__(512, 2) void scan_tp_kernel(ScanArgs p) {
         Raw raw[PF];
         // rows of a chunk that does not exist lie outside the descriptor and read as zero
         auto row0_of = [&](int c) -> int { return c < nchunks ? chunk_row0(c) : -2 * kChunk; };
-        // Every request is made every time, whether its rows exist or not (the chunks before
-        // c0 need no rows of a; chunks past the end have none): a request outside the
-        // descriptor costs no memory traffic, and with a fixed number of requests per chunk
-        // the compiler can wait for the oldest ones only (s_waitcnt vmcnt(n) with n the
-        // number of younger requests) instead of for all of them.
+        // Every request is made every time, whether its rows exist or not (of a chunk before
+        // c0 the producers need rows 0 .. 15 of b and v only, see below; chunks past the end
+        // have none): a request outside the descriptor costs no memory traffic, and with a
+        // fixed number of requests per chunk the compiler can wait for the oldest ones only
+        // (s_waitcnt vmcnt(n) with n the number of younger requests) instead of for all.
+        static_assert(LA == 2 && LV == 2, "quad 0 of a lane: rows 0 .. 15, quad 1: rows 16 .. 31");
         auto fetch = [&](Raw &r, int c) {
             const int row0 = row0_of(c);
-            const int row0_a = c >= c0 ? row0 : -2 * kChunk;
+            const int row0_x = c >= c0 ? row0 : -2 * kChunk;
 #pragma unroll
             for (int q = 0; q < LA; q++) {
                 r.a[q] = __builtin_amdgcn_raw_buffer_load_b128(
-                    a_rs, a_goff[q] + (uint32_t)row0_a * a_slb, 0, 0);
+                    a_rs, a_goff[q] + (uint32_t)row0_x * a_slb, 0, 0);
                 r.b[q] = __builtin_amdgcn_raw_buffer_load_b128(
-                    b_rs, b_goff[q] + (uint32_t)row0 * b_slb, 0, 0);
+                    b_rs, b_goff[q] + (uint32_t)(q == 0 ? row0 : row0_x) * b_slb, 0, 0);
             }
 #pragma unroll
             for (int q = 0; q < LV; q++)
                 r.v[q] = __builtin_amdgcn_raw_buffer_load_b128(
-                    v_rs, v_goff[q] + (uint32_t)row0 * v_slb, 0, 0);
+                    v_rs, v_goff[q] + (uint32_t)(q == 0 ? row0 : row0_x) * v_slb, 0, 0);
         };
-        // chunk k goes to LDS buffer k % 3 through register set k % PF; the chunks before c0
-        // (a multiple of PF) only feed the state and need no piece of a
-        auto cut = [&](const Raw &r, int buf, bool with_a) {
+        // chunk k goes to LDS buffer k % 3 through register set k % PF.  The chunks before c0
+        // (a multiple of PF) only feed the state: no piece of a, and the consumers, who have
+        // little to do there, cut rows 16 .. 31 of b and v themselves.
+        auto cut = [&](const Raw &r, int buf, bool own) {
             lds_char *const pc = unit_pc + buf * kBufBytes;
 #pragma unroll
             for (int q = 0; q < LA; q++) {
-                if (with_a) split_quad_to_lds(r.a[q], pc, kTileA, a_waddr[q]);
-                // (an unused request would be moved out of the loop: same waits either way)
-                else asm volatile("" ::"v"(r.a[q]));
-                split_quad_to_lds(r.b[q], pc + kOffB, kTileA, b_waddr[q]);
+                if (own) split_quad_to_lds(r.a[q], pc, kTileA, a_waddr[q]);
+                if (own || q == 0) split_quad_to_lds(r.b[q], pc + kOffB, kTileA, b_waddr[q]);
             }
 #pragma unroll
-            for (int q = 0; q < LV; q++) split_quad_to_lds(r.v[q], pc + kOffV, kTileV, v_waddr[q]);
+            for (int q = 0; q < LV; q++)
+                if (own || q == 0) split_quad_to_lds(r.v[q], pc + kOffV, kTileV, v_waddr[q]);
+            // (a request whose answer is not used would be moved out of the loop: the waits
+            // are the same either way)
+            if (!own) asm volatile("" ::"v"(r.a[0]), "v"(r.a[1]), "v"(r.b[1]), "v"(r.v[1]));
         };
 #pragma unroll
         for (int j = 0; j < PF; j++) fetch(raw[j], j);
@@ -353,36 +357,100 @@ __global__ __launch_bounds__(512, 2) void scan_tp_kernel(ScanArgs p) {
             af[x - 1][ks][k] = lds_frag16(pc + k * kTileA + a_addr[x - 1][ks]);
     };
     // position-major fragment number i of a chunk (15: v first, then b^T tile by tile)
-    auto tr_frag = [&](const lds_char *pc, int i) {
+    auto tr_frag_into = [&](Frag (&btx)[4][3], Frag (&vfx)[3], const lds_char *pc, int i) {
         if (i < 3)
-            vf[i] = lds_frag_tr(pc + i * kTileV + vt_addr[0], pc + i * kTileV + vt_addr[1]);
+            vfx[i] = lds_frag_tr(pc + i * kTileV + vt_addr[0], pc + i * kTileV + vt_addr[1]);
         else {
             const int dt = (i - 3) / 3, k = (i - 3) % 3;
-            bt[dt][k] = lds_frag_tr(pc + k * kTileA + bt_addr[dt][0], pc + k * kTileA + bt_addr[dt][1]);
+            btx[dt][k] = lds_frag_tr(pc + k * kTileA + bt_addr[dt][0], pc + k * kTileA + bt_addr[dt][1]);
         }
     };
+    auto tr_frag = [&](const lds_char *pc, int i) { tr_frag_into(bt, vf, pc, i); };
 
     auto next_buf = [](int b) -> int { return b == 2 ? 0 : b + 1; };
     int buf = 0;  // LDS buffer of the chunk at hand
-    wg_barrier();
-    FTC_STAMP(13);  // first chunk cut
-    // ---- the chunks before this workgroup's own: state update only ----
-    for (int c = 0; c < c0; c++) {
-        const lds_char *pc = unit_pc + buf * kBufBytes;
+    if (c0 > 0) {
+        // ---- the chunks before this workgroup's own: state update only ----
+        // The consumers have little to do here, so they share the producers' work: rows
+        // 16 .. 31 of b and v of these chunks are fetched and cut by the consumers (lane
+        // 64 w + lane takes the quad that producer lane of the same number would take).
+        // The loop is skewed by one chunk: while the matrix instructions of chunk k - 1 run,
+        // the fragments of chunk k arrive in the other set of registers.
+        const int cid = w * 64 + lane, crow = (T + cid) / QA, cc4 = (T + cid) % QA;
+        const uint32_t b_slb = (uint32_t)op.b_sl * 4, v_slb = (uint32_t)op.v_sl * 4;
+        const char *b_seg = (const char *)op.b + ((int64_t)n * op.b_sn + (int64_t)h * op.b_sh) * 4;
+        const char *v_seg = (const char *)op.v + ((int64_t)n * op.v_sn + (int64_t)h * op.v_sh) * 4;
+        const __amdgpu_buffer_rsrc_t b_rs = __builtin_amdgcn_make_buffer_rsrc(
+            (void *)b_seg, 0, (rows - 1) * b_slb + D * 4, kRsrcFlags);
+        const __amdgpu_buffer_rsrc_t v_rs = __builtin_amdgcn_make_buffer_rsrc(
+            (void *)v_seg, 0, (rows - 1) * v_slb + F * 4, kRsrcFlags);
+        const uint32_t b_goff = (uint32_t)crow * b_slb + 16u * cc4,
+                       v_goff = (uint32_t)crow * v_slb + 16u * cc4;
+        const int b_waddr = TpSwizzle<RBA>::addr(crow, 2 * b_tile_column(4 * cc4)),
+                  v_waddr = TpSwizzle<RBV>::addr(crow, 8 * cc4);
+        struct RawC {
+            u32x4 b, v;
+        };
+        RawC rawc[PF];
+        // (every request every time, as the producers do: beyond c0 - 1 outside the descriptor)
+        auto cfetch = [&](RawC &r, int c) {
+            const int row0 = c < c0 ? chunk_row0(c) : -2 * kChunk;
+            r.b = __builtin_amdgcn_raw_buffer_load_b128(b_rs, b_goff + (uint32_t)row0 * b_slb, 0, 0);
+            r.v = __builtin_amdgcn_raw_buffer_load_b128(v_rs, v_goff + (uint32_t)row0 * v_slb, 0, 0);
+        };
+        auto ccut_b = [&](const RawC &r, int bufk) {
+            split_quad_to_lds(r.b, unit_pc + bufk * kBufBytes + kOffB, kTileA, b_waddr);
+        };
+        auto ccut_v = [&](const RawC &r, int bufk) {
+            split_quad_to_lds(r.v, unit_pc + bufk * kBufBytes + kOffV, kTileV, v_waddr);
+        };
 #pragma unroll
-        for (int i = 0; i < 15; i++) tr_frag(pc, i);
-#pragma unroll
-        for (int i = 0; i < 24; i++)
-            S[i % 4] = mfma16(bt[i % 4][kPa[i / 4]], vf[kPb[i / 4]], S[i % 4]);
-        buf = next_buf(buf);
+        for (int j = 0; j < PF; j++) cfetch(rawc[j], j);
+        ccut_b(rawc[0], 0);
+        ccut_v(rawc[0], 0);
+        cfetch(rawc[0], PF);
         wg_barrier();
-        // the next chunk is cut: if it is the first of our own, its row-major fragments are due
-        if (c + 1 == c0) {
+        FTC_STAMP(13);  // first chunk cut
+        Frag bt2[4][3] = {}, vf2[3] = {};  // (the first round multiplies zeros)
+        int bufn = 1;                      // LDS buffer of the chunk after the one at hand
+        for (int c = 0; c < c0; c += PF) {
 #pragma unroll
-            for (int i = 0; i < 18; i++) rm_frag(unit_pc + buf * kBufBytes, i);
+            for (int j = 0; j < PF; j++) {
+                const lds_char *pc = unit_pc + buf * kBufBytes;
+                // chunk c + j + 1 is cut under the matrix instructions of chunk c + j - 1
+                // (chunk c0 is all the producers')
+                const bool cut_next = j < PF - 1 || c + PF < c0;
+                const RawC &rn = rawc[(j + 1) % PF];
+#pragma unroll
+                for (int i = 0; i < 24; i++) {
+                    if (j % 2 == 0) {
+                        S[i % 4] = mfma16(bt2[i % 4][kPa[i / 4]], vf2[kPb[i / 4]], S[i % 4]);
+                        if (i < 15) tr_frag_into(bt, vf, pc, i);
+                    } else {
+                        S[i % 4] = mfma16(bt[i % 4][kPa[i / 4]], vf[kPb[i / 4]], S[i % 4]);
+                        if (i < 15) tr_frag_into(bt2, vf2, pc, i);
+                    }
+                    if (i == 15 && cut_next) ccut_b(rn, bufn);
+                    if (i == 19 && cut_next) ccut_v(rn, bufn);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+                cfetch(rawc[(j + 1) % PF], c + j + 1 + PF);
+                buf = bufn;
+                bufn = next_buf(bufn);
+                wg_barrier();
+                __builtin_amdgcn_sched_barrier(0);
+            }
         }
-    }
-    if (c0 == 0) {
+        // the last of these chunks (c0 is even: its fragments are in the second set)
+#pragma unroll
+        for (int i = 0; i < 24; i++) {
+            S[i % 4] = mfma16(bt2[i % 4][kPa[i / 4]], vf2[kPb[i / 4]], S[i % 4]);
+            if (i < 18) rm_frag(unit_pc + buf * kBufBytes, i);  // our own first chunk is cut
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    } else {
+        wg_barrier();
+        FTC_STAMP(13);  // first chunk cut
 #pragma unroll
         for (int i = 0; i < 18; i++) rm_frag(unit_pc, i);
     }
