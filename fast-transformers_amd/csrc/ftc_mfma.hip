@@ -42,10 +42,11 @@ int tp_kernel_segments(const ScanDesc *scans, int nscans, int64_t chains, int64_
     int nseg = (int)std::max<int64_t>(1, std::min<int64_t>(std::min<int64_t>(4, 256 / units), total_chunks));
     if (const char *env = getenv("FTC_TP_SEGS")) nseg = std::max(1, std::min(atoi(env), 16));  // tuning aid
     if (const char *env = getenv("FTC_TP")) return atoi(env) != 0 ? nseg : 0;           // tuning aid
-    // Measured (forward / backward, us): cfg2 37 / 51 against 46 / 71 for the kernels that
-    // split L and exchange states; N=10, H=8, L=4096: 124 / 188 against 117 / 245 -- cut
-    // chains pay off while they are short.
-    if (nseg > 1 && total_chunks > 64) return 0;
+    // Measured (forward, us, N=10 H=8): cfg2 (L=1000) 30 against 42 for the kernels that split
+    // L and exchange states; L=3000: 75 against 84; L=4096: 100 against 108; L=8192: 201
+    // against 201 -- cut chains pay off while the chunks that a workgroup walks for its
+    // state alone are few.
+    if (nseg > 1 && total_chunks > 128) return 0;
     // Beyond two rounds of workgroups the other kernels win again (1024 chains of 512
     // positions: 128 / 315 us against 135 / 348): there every chain has its own wavefront,
     // all resident at once, and nothing is split either.
