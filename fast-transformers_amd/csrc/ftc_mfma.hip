@@ -91,6 +91,37 @@ int tp_segment_starts(int64_t chunks, int nseg, int32_t *start) {
     return nseg;
 }
 
+// Longer chains on few CUs: the chain-parallel kernel with an exchange of segment sums.  A
+// chain is cut into as many equal segments as fill the GPU (one workgroup each); a workgroup
+// walks its own chunks twice, first for their state alone.  Returns the number of chunks per
+// segment (0: not this way) and the number of segments in *nseg.
+int tp_exchange_segments(int64_t units, int64_t L, int *nseg) {
+    const int64_t total_chunks = (L + kChunk - 1) / kChunk;
+    *nseg = 0;
+    if (const char *env = getenv("FTC_TPX"))  // tuning aid
+        if (atoi(env) == 0) return 0;
+    // Up to 64 chunks the cut chains without an exchange are as fast (cfg2: 30 us either way)
+    // and need no workspace.
+    if (units < 1 || units > 128 || total_chunks <= 64) return 0;
+    int64_t want = std::min<int64_t>(256 / units, total_chunks / 8);
+    if (const char *env = getenv("FTC_TPX_SEGS")) want = std::max(1, atoi(env));  // tuning aid
+    if (want < 2) return 0;
+    const int64_t seg_chunks = ((total_chunks + want - 1) / want + kTpAhead - 1) / kTpAhead * kTpAhead;
+    const int64_t n = (total_chunks + seg_chunks - 1) / seg_chunks;
+    // a workgroup walks at most 256 chunks with one running state (rounding), a chain has
+    // at most 64 x 64 steps (flags of a group are watched by one wavefront), and every
+    // consumer of every segment has a flag word
+    if (n < 2 || seg_chunks > 256 || n > 4096 || 4 * units * n > kMaxWaves) return 0;
+    *nseg = (int)n;
+    return (int)seg_chunks;
+}
+
+// workspace of the exchange: control block, then two state slots (own sum, group total) of
+// 64 x 16 floats per consumer, four consumers per segment
+int64_t tp_exchange_workspace_bytes(int64_t units, int nseg) {
+    return kControlBytes + 2 * 4 * units * nseg * (int64_t)(64 * 16 * 4);
+}
+
 // `wg`: the plan is for workgroups of F / 32 wavefronts (each has its own flag words);
 // `norm`: for their fused attention form, with one more wavefront and state slab per unit
 MfmaPlan make_plan(int64_t N, int64_t H, int64_t L, int64_t D, int64_t F, int nscans, bool wg,
@@ -217,8 +248,14 @@ bool mfma_scan_supported(const ScanDesc &sd, int64_t L) {
 int64_t mfma_scan_workspace_bytes(int64_t N, int64_t H, int64_t L, int64_t D, int64_t F,
                                   int nscans) {
     // whichever kernel the element types will select
-    return std::max(make_plan(N, H, L, D, F, nscans, false).workspace_bytes,
-                    make_plan(N, H, L, D, F, nscans, true).workspace_bytes);
+    int64_t bytes = std::max(make_plan(N, H, L, D, F, nscans, false).workspace_bytes,
+                             make_plan(N, H, L, D, F, nscans, true).workspace_bytes);
+    if (D == 64 && F == 64) {
+        int nseg = 0;
+        if (tp_exchange_segments(std::max<int64_t>(1, N * H) * nscans, L, &nseg) > 0)
+            bytes = std::max(bytes, tp_exchange_workspace_bytes(std::max<int64_t>(1, N * H) * nscans, nseg));
+    }
+    return bytes;
 }
 
 bool fused_attention_supported(const ScanDesc &sd, int64_t L) {
@@ -245,16 +282,25 @@ int mfma_scan(const ScanDesc *scans, int nscans, int64_t N, int64_t H, int64_t L
                                  std::max(std::max(scans[i].a.stride_l, scans[i].b.stride_l),
                                           std::max(scans[i].v.stride_l, scans[i].out.stride_l)));
     const bool chain_fits = (L + 2 * kChunk) * widest_stride * 4 < 0x7fffffffLL;
-    const int tp_nseg = fused || !chain_fits
-                            ? 0 : tp_kernel_segments(scans, nscans, N * H, L, combo == kFFFF);
-    const bool tp = tp_nseg > 0;
+    const bool tp_shape = !fused && chain_fits && combo == kFFFF && D == 64 && F == 64;
+    const int64_t chains = std::max<int64_t>(1, N * H);
+    int tpx_nseg = 0;
+    const int tpx_seg_chunks = tp_shape ? tp_exchange_segments(chains * nscans, L, &tpx_nseg) : 0;
+    const int tp_nseg = tp_shape && tpx_seg_chunks == 0
+                            ? tp_kernel_segments(scans, nscans, N * H, L, combo == kFFFF) : 0;
+    const bool tp = tp_nseg > 0 || tpx_seg_chunks > 0;
     const bool wg = fused || use_wg_kernel(D, F, nscans, L, combo == kFFFF);
     MfmaPlan pl = make_plan(N, H, L, D, F, nscans, wg, fused != nullptr);
     int32_t tp_start[kMaxTpSegments + 1] = {0};
-    if (tp) {  // one workgroup per chain segment, nothing to exchange
+    if (tpx_seg_chunks > 0) {  // one workgroup per chain segment, segment sums exchanged
+        pl.nseg = tpx_nseg;
+        pl.seg_len = tpx_seg_chunks * kChunk;
+        pl.waves = chains * pl.nseg;
+        pl.workspace_bytes = tp_exchange_workspace_bytes(chains * nscans, pl.nseg);
+    } else if (tp) {  // one workgroup per chain segment, nothing to exchange
         pl.nseg = tp_segment_starts((L + kChunk - 1) / kChunk, tp_nseg, tp_start);
         pl.seg_len = (int)L;
-        pl.waves = std::max<int64_t>(1, N * H) * pl.nseg;
+        pl.waves = chains * pl.nseg;
         pl.workspace_bytes = 0;
     }
     if (pl.workspace_bytes > 0 && (!workspace || workspace_bytes < (size_t)pl.workspace_bytes))
@@ -303,6 +349,8 @@ int mfma_scan(const ScanDesc *scans, int nscans, int64_t N, int64_t H, int64_t L
     args.H = (int32_t)H;
     args.seg_len = pl.seg_len;
     for (int i = 0; i <= kMaxTpSegments; i++) args.tp_start[i] = tp_start[i];
+    args.tp_exchange = tpx_seg_chunks > 0 ? 1 : 0;
+    args.tp_seg_chunks = tpx_seg_chunks;
     args.nseg = pl.nseg;
     args.waves_per_scan = (int32_t)pl.waves;
     args.total_waves = (int32_t)(pl.waves * nscans);
@@ -325,10 +373,10 @@ int mfma_scan(const ScanDesc *scans, int nscans, int64_t N, int64_t H, int64_t L
     // fp32 states of up to 64 rows: the kernel that feeds its fragments from LDS tiles
     bool dma = D <= 64 && combo == kFFFF;
     if (const char *env = getenv("FTC_DMA")) dma = dma && atoi(env) != 0;  // tuning aid
-    note_kernel(tp ? "scan_tp_kernel" : wg ? (fused ? "scan_wg_kernel<NORM>" : "scan_wg_kernel")
+    note_kernel(tp ? (tpx_seg_chunks > 0 ? "scan_tp_kernel (exchange)" : "scan_tp_kernel") : wg ? (fused ? "scan_wg_kernel<NORM>" : "scan_wg_kernel")
                 : dma ? "scan_dma_kernel" : "scan_mfma_kernel");
     if (tp) {
-        launch_scan_tp(args, stream);
+        launch_scan_tp(workspace, args, stream);
     } else if (wg) {
         launch_scan_wg_ffff(D, F, fused != nullptr, workspace, args, stream);
     } else if (dma) {

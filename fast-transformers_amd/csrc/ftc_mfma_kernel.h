@@ -465,6 +465,9 @@ struct ScanArgs {
     // chain-parallel kernel only (ftc_tp_kernel.h): segment s of a chain is chunks
     // tp_start[s] .. tp_start[s + 1] - 1 (starts are multiples of kTpAhead)
     int32_t tp_start[kMaxTpSegments + 1];
+    // ... or, with an exchange of segment sums (tp_exchange != 0), nseg segments of
+    // tp_seg_chunks chunks (a multiple of kTpAhead), taken in the order of arrival
+    int32_t tp_exchange, tp_seg_chunks;
 };
 
 // Which (scan, chain, L-segment) a wavefront works on.

@@ -87,7 +87,7 @@ __device__ __forceinline__ constexpr int b_tile_column(int d) {
     return 32 * (d / 32) + 16 * ((d / 4) % 2) + 4 * ((d % 32) / 8) + d % 4;
 }
 
-__global__ __launch_bounds__(512, 2) void scan_tp_kernel(ScanArgs p) {
+__global__ __launch_bounds__(512, 2) void scan_tp_kernel(uint32_t *__restrict__ ws_ptr, ScanArgs p) {
     constexpr int D = 64, F = 64;
     constexpr int T = 256;                     // producer lanes
     constexpr int PF = kTpAhead;               // chunks requested ahead
@@ -129,15 +129,49 @@ __global__ __launch_bounds__(512, 2) void scan_tp_kernel(ScanArgs p) {
         chain = full + t % (chains - full);
     }
     const uint32_t scan_id = which / nseg;
-    const int seg = (int)(which % nseg);
     const ScanOperands &op = p.scan[scan_id];
     const bool REV = op.rev != 0;
     const int n = (int)(chain / (uint32_t)p.H), h = (int)(chain % (uint32_t)p.H);
     const int rows = (int)p.L;
-    // chunks are numbered in walking order; this workgroup's own are c0 .. nchunks - 1, the
-    // ones before them only feed its state
-    const int c0 = p.tp_start[seg];
-    const int nchunks = min((rows + kChunk - 1) / kChunk, p.tp_start[seg + 1]);
+    const int total_chunks = (rows + kChunk - 1) / kChunk;
+    // Chunks are numbered in walking order; this workgroup's own are c0 .. nchunks - 1.  The
+    // state before them comes from one of two places:
+    //  * no exchange: the workgroup first walks chunks 0 .. c0 - 1 for their state alone;
+    //  * exchange (p.tp_exchange, longer chains): it first walks its OWN chunks for their
+    //    state alone, publishes that sum, and adds up the sums of the segments before it
+    //    (StateExchange in ftc_mfma_kernel.h: flags and state slots in the workspace, fixed
+    //    order of summation, bounded waits).  Segments are then taken in the order in which
+    //    the workgroups of a chain start running (a ticket per chain), so that a workgroup
+    //    only ever waits for workgroups that are running already.
+    const bool exchange = p.tp_exchange != 0 && nseg > 1;
+    gu32 *const hdr = (gu32 *)ws_ptr;
+    gu32 *const flags = hdr + kHdrWords;
+    const uint32_t chain_id = scan_id * chains + chain;  // over all scans of the launch
+    int seg = (int)(which % nseg);
+    __shared__ uint32_t order_sh;
+    if (exchange) {
+        if (tid == 0)
+            order_sh = __hip_atomic_fetch_add(flags + kMaxWaves + chain_id, 1u, __ATOMIC_RELAXED,
+                                              __HIP_MEMORY_SCOPE_AGENT);
+        __syncthreads();
+        seg = (int)__builtin_amdgcn_readfirstlane(order_sh);
+        if ((uint32_t)seg >= nseg) {  // the control block was not zero when the launch began
+            if (tid == 0)
+                __hip_atomic_store(hdr + kHdrError, 2u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            return;
+        }
+    }
+    const int c0 = exchange ? seg * p.tp_seg_chunks : p.tp_start[seg];
+    const int nchunks = min(total_chunks, exchange ? c0 + p.tp_seg_chunks : p.tp_start[seg + 1]);
+    // the chunks walked for their state alone: so0 .. so0 + n1 - 1 (n1 a multiple of PF; the
+    // last segment of an exchange has no reader for its sum)
+    const int so0 = exchange ? c0 : 0;
+    const int n1 = exchange ? (seg + 1 < (int)nseg ? nchunks - c0 : 0) : c0;
+    // position v of the walk: v < n1: a chunk walked for its state alone; then chunk
+    // c0 + v - n1.  With an exchange the first pass runs against the direction of the second,
+    // so that the second starts with the rows that the caches saw last.
+    const int nwalk = n1 + nchunks - c0;  // (position nwalk: a chunk of zeros)
+    auto so_chunk = [&](int v) -> int { return exchange ? so0 + n1 - 1 - v : so0 + v; };
     auto chunk_row0 = [&](int c) -> int { return REV ? rows - kChunk * (c + 1) : kChunk * c; };
     __syncthreads();
 #ifdef FTC_TIMELINE
@@ -184,17 +218,17 @@ __global__ __launch_bounds__(512, 2) void scan_tp_kernel(ScanArgs p) {
             u32x4 a[LA], b[LA], v[LV];
         };
         Raw raw[PF];
-        // rows of a chunk that does not exist lie outside the descriptor and read as zero
-        auto row0_of = [&](int c) -> int { return c < nchunks ? chunk_row0(c) : -2 * kChunk; };
-        // Every request is made every time, whether its rows exist or not (of a chunk before
-        // c0 the producers need rows 0 .. 15 of b and v only, see below; chunks past the end
-        // have none): a request outside the descriptor costs no memory traffic, and with a
-        // fixed number of requests per chunk the compiler can wait for the oldest ones only
-        // (s_waitcnt vmcnt(n) with n the number of younger requests) instead of for all.
+        // Every request is made every time, whether its rows exist or not (of a chunk walked
+        // for its state alone the producers need rows 0 .. 15 of b and v only, see below;
+        // positions past the end of the walk have no rows): a request outside the descriptor
+        // costs no memory traffic and reads as zero, and with a fixed number of requests per
+        // chunk the compiler can wait for the oldest ones only (s_waitcnt vmcnt(n) with n the
+        // number of younger requests) instead of for all.
         static_assert(LA == 2 && LV == 2, "quad 0 of a lane: rows 0 .. 15, quad 1: rows 16 .. 31");
-        auto fetch = [&](Raw &r, int c) {
-            const int row0 = row0_of(c);
-            const int row0_x = c >= c0 ? row0 : -2 * kChunk;
+        auto fetch = [&](Raw &r, int v) {  // v: position of the walk
+            const int c = v < n1 ? so_chunk(v) : c0 + v - n1;
+            const int row0 = v < nwalk ? chunk_row0(c) : -2 * kChunk;
+            const int row0_x = v >= n1 ? row0 : -2 * kChunk;
 #pragma unroll
             for (int q = 0; q < LA; q++) {
                 r.a[q] = __builtin_amdgcn_raw_buffer_load_b128(
@@ -207,9 +241,9 @@ __global__ __launch_bounds__(512, 2) void scan_tp_kernel(ScanArgs p) {
                 r.v[q] = __builtin_amdgcn_raw_buffer_load_b128(
                     v_rs, v_goff[q] + (uint32_t)(q == 0 ? row0 : row0_x) * v_slb, 0, 0);
         };
-        // chunk k goes to LDS buffer k % 3 through register set k % PF.  The chunks before c0
-        // (a multiple of PF) only feed the state: no piece of a, and the consumers, who have
-        // little to do there, cut rows 16 .. 31 of b and v themselves.
+        // position k of the walk goes to LDS buffer k % 3 through register set k % PF.  The
+        // first n1 positions (a multiple of PF) only feed the state: no piece of a, and the
+        // consumers, who have little to do there, cut rows 16 .. 31 of b and v themselves.
         auto cut = [&](const Raw &r, int buf, bool own) {
             lds_char *const pc = unit_pc + buf * kBufBytes;
 #pragma unroll
@@ -226,16 +260,16 @@ __global__ __launch_bounds__(512, 2) void scan_tp_kernel(ScanArgs p) {
         };
 #pragma unroll
         for (int j = 0; j < PF; j++) fetch(raw[j], j);
-        // Barrier number k (k = 0: before the first chunk; k >= 1: in the middle of chunk
-        // k - 1) finds chunk k cut.  The last one finds a chunk of zeros.
+        // Barrier number k (k = 0: before the first position; k >= 1: in the middle of
+        // position k - 1) finds position k cut.  The last one finds a chunk of zeros.
         // Two loops whose bodies are straight-line code, so that the waits inside them count
         // requests instead of draining them.
         int buf = 0;
-        for (int c = 0; c < c0; c += PF) {
+        for (int v = 0; v < n1; v += PF) {
 #pragma unroll
             for (int j = 0; j < PF; j++) {
                 cut(raw[j], buf, false);
-                fetch(raw[j], c + j + PF);
+                fetch(raw[j], v + j + PF);
                 buf = buf == 2 ? 0 : buf + 1;
                 wg_barrier();
                 __builtin_amdgcn_sched_barrier(0);  // one chunk at a time, in this order
@@ -243,24 +277,24 @@ __global__ __launch_bounds__(512, 2) void scan_tp_kernel(ScanArgs p) {
         }
         // (whole trips in the loop, the rest after it: a way out of the middle of the loop
         // would join the paths at the loop's head and spoil the counting)
-        int c = c0;
-        for (; c + PF <= nchunks + 1; c += PF) {
+        int v = n1;
+        for (; v + PF <= nwalk + 1; v += PF) {
 #pragma unroll
             for (int j = 0; j < PF; j++) {
-                if (c + j == c0 + 4) FTC_STAMP(0);
+                if (v + j == n1 + 4) FTC_STAMP(0);
                 cut(raw[j], buf, true);
-                if (c + j == c0 + 4) FTC_STAMP(1);
-                fetch(raw[j], c + j + PF);
+                if (v + j == n1 + 4) FTC_STAMP(1);
+                fetch(raw[j], v + j + PF);
                 buf = buf == 2 ? 0 : buf + 1;
-                if (c + j == c0 + 4) FTC_STAMP(2);
+                if (v + j == n1 + 4) FTC_STAMP(2);
                 wg_barrier();
                 __builtin_amdgcn_sched_barrier(0);  // one chunk at a time, in this order
-                if (c + j == c0 + 4) FTC_STAMP(3);
+                if (v + j == n1 + 4) FTC_STAMP(3);
             }
         }
 #pragma unroll
         for (int j = 0; j < PF - 1; j++) {
-            if (c + j > nchunks) return;
+            if (v + j > nwalk) return;
             cut(raw[j], buf, true);
             buf = buf == 2 ? 0 : buf + 1;
             wg_barrier();
@@ -336,13 +370,16 @@ __global__ __launch_bounds__(512, 2) void scan_tp_kernel(ScanArgs p) {
     constexpr int kPa[6] = {0, 1, 2, 0, 1, 0}, kPb[6] = {2, 1, 0, 1, 0, 0};  // piece products
     // the caller's state: lane (f = 16 w + ln, g), tile dt, register r <-> row d below
     auto state_row = [&](int dt, int r) -> int { return 32 * (dt / 2) + 8 * g + 4 * (dt % 2) + r; };
-    if (op.s0) {
+    auto add_caller_state = [&]() {
         const float *base = op.s0 + (int64_t)n * op.s0_sn + (int64_t)h * op.s0_sh + 16 * w + ln;
 #pragma unroll
         for (int dt = 0; dt < 4; dt++)
 #pragma unroll
             for (int r = 0; r < 4; r++) S[dt][r] += base[(int64_t)state_row(dt, r) * op.s0_sd];
-    }
+    };
+    // (with an exchange the sums that travel are those of the rows alone; every segment adds
+    // the caller's state on top of what it gathers)
+    if (op.s0 && !exchange) add_caller_state();
 
     // A wavefront issues in order, and four of them share the LDS: reads are therefore
     // written out between the matrix instructions they run under, one at a time, and
@@ -369,8 +406,8 @@ __global__ __launch_bounds__(512, 2) void scan_tp_kernel(ScanArgs p) {
 
     auto next_buf = [](int b) -> int { return b == 2 ? 0 : b + 1; };
     int buf = 0;  // LDS buffer of the chunk at hand
-    if (c0 > 0) {
-        // ---- the chunks before this workgroup's own: state update only ----
+    if (n1 > 0) {
+        // ---- the first n1 positions of the walk: state update only ----
         // The consumers have little to do here, so they share the producers' work: rows
         // 16 .. 31 of b and v of these chunks are fetched and cut by the consumers (lane
         // 64 w + lane takes the quad that producer lane of the same number would take).
@@ -392,9 +429,10 @@ __global__ __launch_bounds__(512, 2) void scan_tp_kernel(ScanArgs p) {
             u32x4 b, v;
         };
         RawC rawc[PF];
-        // (every request every time, as the producers do: beyond c0 - 1 outside the descriptor)
-        auto cfetch = [&](RawC &r, int c) {
-            const int row0 = c < c0 ? chunk_row0(c) : -2 * kChunk;
+        // (every request every time, as the producers do: from position n1 on outside the
+        // descriptor)
+        auto cfetch = [&](RawC &r, int v) {
+            const int row0 = v < n1 ? chunk_row0(so_chunk(v)) : -2 * kChunk;
             r.b = __builtin_amdgcn_raw_buffer_load_b128(b_rs, b_goff + (uint32_t)row0 * b_slb, 0, 0);
             r.v = __builtin_amdgcn_raw_buffer_load_b128(v_rs, v_goff + (uint32_t)row0 * v_slb, 0, 0);
         };
@@ -413,13 +451,13 @@ __global__ __launch_bounds__(512, 2) void scan_tp_kernel(ScanArgs p) {
         FTC_STAMP(13);  // first chunk cut
         Frag bt2[4][3] = {}, vf2[3] = {};  // (the first round multiplies zeros)
         int bufn = 1;                      // LDS buffer of the chunk after the one at hand
-        for (int c = 0; c < c0; c += PF) {
+        for (int c = 0; c < n1; c += PF) {
 #pragma unroll
             for (int j = 0; j < PF; j++) {
                 const lds_char *pc = unit_pc + buf * kBufBytes;
-                // chunk c + j + 1 is cut under the matrix instructions of chunk c + j - 1
-                // (chunk c0 is all the producers')
-                const bool cut_next = j < PF - 1 || c + PF < c0;
+                // position c + j + 1 is cut under the matrix instructions of position
+                // c + j - 1 (position n1 is all the producers')
+                const bool cut_next = j < PF - 1 || c + PF < n1;
                 const RawC &rn = rawc[(j + 1) % PF];
 #pragma unroll
                 for (int i = 0; i < 24; i++) {
@@ -441,7 +479,7 @@ __global__ __launch_bounds__(512, 2) void scan_tp_kernel(ScanArgs p) {
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
-        // the last of these chunks (c0 is even: its fragments are in the second set)
+        // the last of these chunks (n1 is even: its fragments are in the second set)
 #pragma unroll
         for (int i = 0; i < 24; i++) {
             S[i % 4] = mfma16(bt2[i % 4][kPa[i / 4]], vf2[kPb[i / 4]], S[i % 4]);
@@ -453,6 +491,30 @@ __global__ __launch_bounds__(512, 2) void scan_tp_kernel(ScanArgs p) {
         FTC_STAMP(13);  // first chunk cut
 #pragma unroll
         for (int i = 0; i < 18; i++) rm_frag(unit_pc, i);
+    }
+    if (exchange) {
+        // ---- the sum of this segment's rows goes out, the state before the segment comes in ----
+        const uint32_t total_units = (uint32_t)p.total_waves;
+        gfloat *const sums = (gfloat *)(hdr + kControlBytes / 4);
+        // the flag words and state slots of consumer w of the segment with ticket t are those
+        // of "ticket" w * total_units + t (as in ftc_wg_kernel.h)
+        StateExchange<1, 1> xch(flags, sums, 4u * total_units,
+                                (uint32_t)w * total_units + chain_id * nseg + (uint32_t)seg, seg,
+                                (int)nseg, p.group, lane);
+        f32x16 Sx[1][1], X[1][1];
+#pragma unroll
+        for (int dt = 0; dt < 4; dt++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) Sx[0][0][4 * dt + r] = S[dt][r];
+        if (n1 > 0) xch.publish_sum(Sx);
+        xch.gather(Sx, X);
+        if (xch.failed && lane == 0)
+            __hip_atomic_store(hdr + kHdrError, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+        for (int dt = 0; dt < 4; dt++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) S[dt][r] = X[0][0][4 * dt + r];
+        if (op.s0) add_caller_state();
     }
     // S_w as pieces in A operand order (slots 0..3 from tile 2 ks, 4..7 from tile 2 ks + 1).
     // Tiles 0 and 1 are final after phase 3 and are cut under phase 4, tiles 2 and 3 after
@@ -584,6 +646,25 @@ __global__ __launch_bounds__(512, 2) void scan_tp_kernel(ScanArgs p) {
         for (int dt = 0; dt < 4; dt++)
 #pragma unroll
             for (int r = 0; r < 4; r++) base[(int64_t)state_row(dt, r) * op.so_sd] = S[dt][r];
+    }
+    // the last consumer of the launch leaves the control block zeroed (as in ftc_wg_kernel.h)
+    if (exchange) {
+        const uint32_t total_units = (uint32_t)p.total_waves;
+        uint32_t done = 0;
+        if (lane == 0)
+            done = __hip_atomic_fetch_add(hdr + kHdrDone, 1u, __ATOMIC_RELAXED,
+                                          __HIP_MEMORY_SCOPE_AGENT);
+        done = __builtin_amdgcn_readfirstlane(done);
+        if (done == 4u * total_units - 1) {
+            for (uint32_t i = lane; i < 4u * total_units; i += kWave)
+                __hip_atomic_store(flags + i, kFlagEmpty, __ATOMIC_RELAXED,
+                                   __HIP_MEMORY_SCOPE_AGENT);
+            for (uint32_t i = lane; i < total_units / nseg; i += kWave)
+                __hip_atomic_store(flags + kMaxWaves + i, 0u, __ATOMIC_RELAXED,
+                                   __HIP_MEMORY_SCOPE_AGENT);
+            if (lane == 0)
+                __hip_atomic_store(hdr + kHdrDone, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
     }
 }
 

@@ -745,7 +745,7 @@ void launch_scan_wg_ffff(int D, int F, bool norm, void *ws, const ScanArgs &args
 bool scan_wg_covers(int D, int F);
 bool scan_wg_norm_covers(int D, int F);
 // chain-parallel form (ftc_tp_kernel.h): one workgroup per chain of a 64 x 64 all-fp32 scan
-void launch_scan_tp(const ScanArgs &args, hipStream_t stream);
+void launch_scan_tp(void *ws, const ScanArgs &args, hipStream_t stream);
 
 }  // namespace mfma
 }  // namespace ftc

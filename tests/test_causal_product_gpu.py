@@ -487,6 +487,8 @@ STATE_SHAPES = {
     "e64_m64": (2, 4, 1000, 64, 64, 51, torch.float32),
     # one segment per chain (no exchange)
     "many_chains": (40, 32, 64, 64, 64, 52, torch.float32),
+    # long chains: workgroups of the chain-parallel kernel exchange segment sums
+    "long_e64_m64": (1, 4, 5000, 64, 64, 59, torch.float32),
     "e32_m128": (2, 3, 700, 32, 128, 53, torch.float32),
     # register-fed kernel, column slices
     "e128_m128": (1, 3, 500, 128, 128, 54, torch.float32),
@@ -699,6 +701,46 @@ def test_chain_parallel_kernel(cp, shape):
     exacts = oracle.backward(Q.double(), K.double(), V.double(), G.double())
     for name, got, ref, ex in zip(("dQ", "dK", "dV"), (dq, dk, dv), refs, exacts):
         _gate_against_float64("tp %s %s" % (shape, name), got.cpu(), ref, ex)
+
+
+TPX_SHAPES = [
+    # N, H, L: long chains on few CUs: segments that exchange their sums (one and two levels
+    # of the sum, ragged last segment, a last segment shorter than the others)
+    (2, 8, 4096), (1, 3, 9000), (3, 5, 2100), (1, 2, 40000),
+]
+
+
+@pytest.mark.parametrize("shape", TPX_SHAPES, ids=lambda s: "n%d_h%d_l%d" % s)
+def test_chain_parallel_kernel_with_exchange(cp, shape):
+    """The same kernel on chains too long to walk twice from the start: every workgroup first
+    sums its own segment, the sums travel through the workspace.  Both directions,
+    (N, L, H, X) views, against the CPU checker anchored on float64; a second call finds the
+    control block as the first one left it."""
+    from fast_transformers_amd import _native
+    N, H, L = shape
+    E = M = 64
+    Q, K, V, G = oracle.make_inputs(N, H, L, E, M, seed=400 + L)
+    nlh = lambda t: t.permute(0, 2, 1, 3).contiguous().cuda().permute(0, 2, 1, 3)  # NLHE storage
+    q, k, v, g = (nlh(t) for t in (Q, K, V, G))
+    out = torch.full((N, L, H, M), float("nan"), device="cuda").permute(0, 2, 1, 3)
+    cp.causal_dot_product_hip(q, k, v, out)
+    assert _native.load().ftc_last_kernel() == b"scan_tp_kernel (exchange)"
+    dq, dk, dv = (torch.full((N, L, H, X), float("nan"), device="cuda").permute(0, 2, 1, 3)
+                  for X in (E, E, M))
+    cp.causal_dot_backward_hip(q, k, v, g, dq, dk, dv)
+    assert _native.load().ftc_last_kernel() == b"scan_tp_kernel (exchange)"
+    again = torch.empty_like(out)
+    cp.causal_dot_product_hip(q, k, v, again)
+    torch.cuda.synchronize()
+    assert torch.equal(out, again)
+    cp.check_workspaces()
+    want = oracle.forward(Q, K, V)
+    exact = oracle.forward(Q.double(), K.double(), V.double())
+    _gate_against_float64("tpx %s product" % (shape,), out.cpu(), want, exact)
+    refs = oracle.backward(Q, K, V, G)
+    exacts = oracle.backward(Q.double(), K.double(), V.double(), G.double())
+    for name, got, ref, ex in zip(("dQ", "dK", "dV"), (dq, dk, dv), refs, exacts):
+        _gate_against_float64("tpx %s %s" % (shape, name), got.cpu(), ref, ex)
 
 
 def test_rows_far_apart_leave_the_chain_parallel_kernel(cp):
