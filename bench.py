@@ -39,8 +39,8 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 matrix, published
 # carries it only while the sources are unchanged, otherwise null.
 MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {
     # workload: (bytes, kernel source hash at the time of the measurement)
-    "cfg2": (136948007, "7afd66aaa13d877c"),
-    "cfg3": (3156036879, "7afd66aaa13d877c"),
+    "cfg2": (137118429, "74a891c3d2326939"),
+    "cfg3": (3139063532, "74a891c3d2326939"),
 }
 
 WORKLOADS = {
