@@ -2,20 +2,25 @@
 //
 //   out[c, l, f] = sum_{j <= l} (a[c,l,:] . b[c,j,:]) * v[c,j,f]      (REV: j >= l)
 //
-// One workgroup walks one chain, chunk after chunk; nothing is exchanged between workgroups
-// and there is no workspace.  With enough chains a workgroup takes a whole chain and every
-// row is read once.  With fewer, a chain is cut into up to four segments, and the workgroup
-// of a segment first runs the state update alone -- step (3) below, a third of the matrix
-// work and no chunk product -- over the chunks before its own, so that it starts from the
-// same state, bit for bit, that a single walk would have reached (later segments are made
-// shorter, so that all workgroups of a chain finish together).  What makes a single chain
-// fast enough is that the work of a chunk is spread over four matrix cores: the 64 x 64 state is held as four slabs of 16
-// columns, one per consumer wavefront (one per SIMD), and the 32 x 32 chunk product Pt is
-// computed once, a quadrant per wavefront, and shared through LDS.
+// One workgroup walks one chain, chunk after chunk.  With enough chains a workgroup takes a
+// whole chain and every row is read once; nothing is exchanged between workgroups and no
+// workspace is touched.  With fewer, a chain is cut into segments, one workgroup each, and
+// the state before a segment comes about in one of two ways:
+//  * short chains: the workgroup first runs the state update alone -- step (3) below, a
+//    third of the matrix work and no chunk product -- over the chunks before its own, so
+//    that it starts from the same state, bit for bit, that a single walk would have reached
+//    (later segments are made shorter, so that all workgroups of a chain finish together);
+//  * long chains: it first runs the state update alone over its OWN chunks, publishes that
+//    sum and adds up the sums of the segments before it (StateExchange, ftc_mfma_kernel.h).
+// What makes a single chain fast enough is that the work of a chunk is spread over four
+// matrix cores: the 64 x 64 state is held as four slabs of 16 columns, one per consumer
+// wavefront (one per SIMD), and the 32 x 32 chunk product Pt is computed once, a quadrant
+// per wavefront, and shared through LDS.
 //
 //  * Wavefronts 4..7 (producers) fetch the rows of a chunk, cut every fp32 value into its
-//    three bf16 pieces and write them as row-major piece tiles into double-buffered LDS,
-//    four chunks ahead (as in ftc_wg_kernel.h).
+//    three bf16 pieces and write them as row-major piece tiles into LDS, four chunks
+//    ahead (as in ftc_wg_kernel.h).  Of the chunks that only feed the state they take rows
+//    0 .. 15 of b and v; the consumers, who have little to do there, take rows 16 .. 31.
 //  * Wavefronts 0..3 (consumers), v_mfma_f32_16x16x32_bf16 (A: row = lane % 16, B: column =
 //    lane % 16, both with k-slots t = 0..7 of lane group g = lane / 16; accumulator: column
 //    = lane % 16, rows 4 g + r).  Consumer w owns output columns 16 w .. 16 w + 15:
