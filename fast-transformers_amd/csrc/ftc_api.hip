@@ -10,6 +10,7 @@
 //   dV      = scan_rev(a=K, b=Q, v=G)      state E x M
 #include <stdarg.h>
 #include <stdio.h>
+#include <string.h>
 
 #include <algorithm>
 #include <mutex>
@@ -27,6 +28,18 @@ static thread_local char g_error[512] = "";
 
 static thread_local const char *g_kernel = "";
 void note_kernel(const char *name) { g_kernel = name; }
+static thread_local bool g_plan_only = false;
+static thread_local char g_plan[2048] = "";
+bool plan_only() { return g_plan_only; }
+void note_plan(const char *fmt, ...) {
+    const size_t used = strlen(g_plan);
+    if (used + 2 >= sizeof(g_plan)) return;
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_plan + used, sizeof(g_plan) - used - 1, fmt, ap);
+    va_end(ap);
+    strcat(g_plan, "\n");
+}
 
 int fail(int code, const char *fmt, ...) {
     va_list ap;
@@ -333,6 +346,42 @@ int ftc_causal_dot_backward(const ftc_tensor4 *queries, const ftc_tensor4 *keys,
     if (grad_values)  // dV: state E x M, walks down
         scans[n++] = ScanDesc{K, Q, G, as_operand_out(grad_values), true};
     return run_scans(scans, n, d.N, d.H, d.L, workspace, workspace_bytes, s);
+}
+
+int ftc_causal_dot_plan(const ftc_tensor4 *queries, const ftc_tensor4 *keys,
+                        const ftc_tensor4 *values, int backward, char *text, size_t text_bytes) {
+    if (!queries || !keys || !values || !text || text_bytes == 0)
+        return fail(FTC_ERR_INVALID, "null argument");
+    // data pointers are never read here: absent ones are replaced by a placeholder so that
+    // the checks of the real entry points apply unchanged
+    auto with_ptr = [](ftc_tensor4 t) {
+        if (!t.ptr) t.ptr = (void *)(uintptr_t)4096;
+        return t;
+    };
+    const ftc_tensor4 q = with_ptr(*queries), k = with_ptr(*keys), v = with_ptr(*values);
+    auto dense = [&](int64_t width, int dtype) {
+        ftc_tensor4 t;
+        t.ptr = (void *)(uintptr_t)4096;
+        t.dtype = dtype;
+        t.size[0] = q.size[0], t.size[1] = q.size[1], t.size[2] = q.size[2], t.size[3] = width;
+        t.stride[3] = 1, t.stride[2] = width, t.stride[1] = t.stride[2] * t.size[2];
+        t.stride[0] = t.stride[1] * t.size[1];
+        return t;
+    };
+    const ftc_tensor4 out = dense(v.size[3], FTC_F32);
+    g_plan[0] = 0;
+    g_plan_only = true;
+    int rc;
+    if (!backward) {
+        rc = ftc_causal_dot_product(&q, &k, &v, &out, nullptr, 0, nullptr);
+    } else {
+        const ftc_tensor4 gq = dense(q.size[3], q.dtype), gk = dense(k.size[3], k.dtype),
+                          gv = dense(v.size[3], v.dtype);
+        rc = ftc_causal_dot_backward(&q, &k, &v, &out, &gq, &gk, &gv, nullptr, 0, nullptr);
+    }
+    g_plan_only = false;
+    snprintf(text, text_bytes, "%s", g_plan);
+    return rc;
 }
 
 int64_t ftc_causal_linear_attention_workspace_bytes(int64_t N, int64_t H, int64_t L, int64_t E,

@@ -44,6 +44,10 @@ inline OperandOut as_operand_out(const ftc_tensor4 *t) {
 int fail(int code, const char *fmt, ...);
 // Records which kernel the last launch on this thread used (ftc_last_kernel()).
 void note_kernel(const char *name);
+// Plan-only mode of the calling thread (ftc_causal_dot_plan): the scan functions describe the
+// launch they would make, one line each, instead of making it, and touch no GPU.
+bool plan_only();
+void note_plan(const char *fmt, ...);
 
 // bf16 <-> fp32 with round-to-nearest-even (finite inputs; NaN stays NaN).
 __device__ __forceinline__ float bf16_to_f32(uint16_t b) {

@@ -282,6 +282,10 @@ void launch_by_width(const GenericArgs &args, int64_t wgs, hipStream_t stream) {
 int zero_rows(const OperandOut &out, int64_t N, int64_t H, int64_t L, hipStream_t stream) {
     const int64_t total = N * H * L * out.width;
     if (total == 0) return FTC_OK;
+    if (plan_only()) {
+        note_plan("zero_rows_kernel: %lld values", (long long)total);
+        return FTC_OK;
+    }
     const int64_t wgs = std::min<int64_t>((total + kThreads - 1) / kThreads, 65536);
     hipLaunchKernelGGL(zero_rows_kernel, dim3((unsigned)wgs), dim3(kThreads), 0, stream, out, H, L,
                        total);
@@ -305,6 +309,11 @@ int generic_scan(const Operand &a, const Operand &b, const Operand &v, const Ope
                     kGenericMaxDim, (long long)D, (long long)F);
     if (b.width != D || out.width != F) return fail(FTC_ERR_INVALID, "operand widths disagree");
     const GenericPlan pl = make_plan(N, H, L, D, F);
+    if (plan_only()) {
+        note_plan("generic_scan_kernel: state %lld x %lld, %s, workspace %lld bytes", (long long)D,
+                  (long long)F, reverse ? "reverse" : "forward", (long long)pl.workspace_bytes);
+        return FTC_OK;
+    }
     if (pl.workspace_bytes > 0 && (!workspace || workspace_bytes < (size_t)pl.workspace_bytes))
         return fail(FTC_ERR_WORKSPACE, "workspace of %lld bytes needed, %zu given",
                     (long long)pl.workspace_bytes, workspace_bytes);

@@ -303,11 +303,13 @@ int mfma_scan(const ScanDesc *scans, int nscans, int64_t N, int64_t H, int64_t L
         pl.waves = chains * pl.nseg;
         pl.workspace_bytes = 0;
     }
-    if (pl.workspace_bytes > 0 && (!workspace || workspace_bytes < (size_t)pl.workspace_bytes))
-        return fail(FTC_ERR_WORKSPACE, "workspace of %lld bytes needed, %zu given",
-                    (long long)pl.workspace_bytes, workspace_bytes);
-    if (pl.workspace_bytes > 0 && (uintptr_t)workspace % 256 != 0)
-        return fail(FTC_ERR_WORKSPACE, "workspace must be 256-byte aligned");
+    if (!plan_only()) {
+        if (pl.workspace_bytes > 0 && (!workspace || workspace_bytes < (size_t)pl.workspace_bytes))
+            return fail(FTC_ERR_WORKSPACE, "workspace of %lld bytes needed, %zu given",
+                        (long long)pl.workspace_bytes, workspace_bytes);
+        if (pl.workspace_bytes > 0 && (uintptr_t)workspace % 256 != 0)
+            return fail(FTC_ERR_WORKSPACE, "workspace must be 256-byte aligned");
+    }
 
     ScanArgs args;
     int64_t max_stride = 0;
@@ -375,6 +377,20 @@ int mfma_scan(const ScanDesc *scans, int nscans, int64_t N, int64_t H, int64_t L
     if (const char *env = getenv("FTC_DMA")) dma = dma && atoi(env) != 0;  // tuning aid
     note_kernel(tp ? (tpx_seg_chunks > 0 ? "scan_tp_kernel (exchange)" : "scan_tp_kernel") : wg ? (fused ? "scan_wg_kernel<NORM>" : "scan_wg_kernel")
                 : dma ? "scan_dma_kernel" : "scan_mfma_kernel");
+    if (plan_only()) {
+        char cuts[160] = "";
+        if (tp && tpx_seg_chunks == 0)
+            for (int i = 0, at = 0; i <= pl.nseg && at < 140; i++)
+                at += snprintf(cuts + at, sizeof(cuts) - at, "%s%d", i ? "," : ", cuts at chunks ",
+                               (int)args.tp_start[i]);
+        note_plan("%s: %d scan%s (%s), state %d x %d, %lld chains, %d segment%s of %d rows%s, "
+                  "%lld workgroups or wavefronts, workspace %lld bytes",
+                  ftc_last_kernel(), nscans, nscans == 1 ? "" : "s",
+                  scans[0].reverse ? "first one reverse" : "first one forward", D, F,
+                  (long long)chains, (int)pl.nseg, pl.nseg == 1 ? "" : "s", (int)pl.seg_len, cuts,
+                  (long long)args.total_waves, (long long)pl.workspace_bytes);
+        return FTC_OK;
+    }
     if (tp) {
         launch_scan_tp(workspace, args, stream);
     } else if (wg) {

@@ -22,6 +22,7 @@ EXPORTED_SYMBOLS = (
     "ftc_version",
     "ftc_last_error",
     "ftc_last_kernel",
+    "ftc_causal_dot_plan",
     "ftc_workspace_reset",
     "ftc_causal_dot_product_workspace_bytes",
     "ftc_causal_dot_product",
@@ -87,8 +88,31 @@ def load():
     lib.ftc_causal_linear_attention.argtypes = [t4] * 3 + [ctypes.c_void_p, ctypes.c_float, t4,
                                                            ctypes.c_void_p, ctypes.c_size_t,
                                                            ctypes.c_void_p]
+    lib.ftc_causal_dot_plan.restype = ctypes.c_int
+    lib.ftc_causal_dot_plan.argtypes = [t4] * 3 + [ctypes.c_int, ctypes.c_char_p, ctypes.c_size_t]
     _lib = lib
     return lib
+
+
+def plan(shape_q, shape_v, dtype=FTC_F32, backward=False, strides=None):
+    """Text of ``ftc_causal_dot_plan`` for dense (N, H, L, E) queries and keys and (N, H, L, M)
+    values (or the element strides given as three 4-tuples): what the planner would launch.
+    Needs no GPU."""
+    def dense(shape, stride):
+        d = Tensor4()
+        d.ptr = None
+        d.dtype = dtype
+        st = stride or (shape[1] * shape[2] * shape[3], shape[2] * shape[3], shape[3], 1)
+        for i in range(4):
+            d.size[i], d.stride[i] = shape[i], st[i]
+        return d
+    st = strides or (None, None, None)
+    q, k, v = dense(shape_q, st[0]), dense(shape_q, st[1]), dense(shape_v, st[2])
+    buf = ctypes.create_string_buffer(4096)
+    rc = load().ftc_causal_dot_plan(ctypes.byref(q), ctypes.byref(k), ctypes.byref(v),
+                                    1 if backward else 0, buf, len(buf))
+    check(rc, "ftc_causal_dot_plan")
+    return buf.value.decode()
 
 
 def last_error():

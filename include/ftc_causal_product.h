@@ -81,6 +81,18 @@ const char *ftc_last_error(void);
 const char *ftc_last_kernel(void);
 
 /*
+ * What ftc_causal_dot_product (backward == 0) or ftc_causal_dot_backward (backward != 0,
+ * all three gradients, dense outputs) would launch for tensors of these shapes, element
+ * types and strides: one line of text per launch (kernel, state size, chains, segments, cuts,
+ * workspace), written to `text` (at most text_bytes - 1 characters).  Nothing is launched and
+ * no GPU is needed; the data pointers are not read and may be NULL.  Returns what the real
+ * call would return for these arguments, workspace checks aside.  For tests of the planner
+ * and for tuning; no counterpart in the reference.
+ */
+int ftc_causal_dot_plan(const ftc_tensor4 *queries, const ftc_tensor4 *keys,
+                        const ftc_tensor4 *values, int backward, char *text, size_t text_bytes);
+
+/*
  * Clears the control block of a workspace (a fill kernel enqueued on `stream`; no memset, so
  * it may be captured in a graph).  No counterpart in the reference.  A workspace needs this
  * once before its first use unless it was allocated zero-filled, and again after a call whose

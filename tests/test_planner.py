@@ -1,0 +1,108 @@
+"""Host-side planning of the launches (which kernel, how chains are cut, how much workspace),
+read through ``ftc_causal_dot_plan``: nothing is launched, no GPU is needed.
+
+The figures pinned here are the planner's rules as documented where the planner lives
+(csrc/ftc_mfma.hip): one workgroup per chain segment on up to 256 CUs, chains of up to 64
+chunks cut without an exchange at multiples of four chunks with later segments shorter,
+longer chains on few CUs with an exchange, everything the MFMA kernels do not cover on the
+generic kernel."""
+import re
+
+import pytest
+
+from fast_transformers_amd import _native
+
+
+def lines(q, v, **kw):
+    return [l for l in _native.plan(q, v, **kw).split("\n") if l]
+
+
+def field(line, pattern):
+    m = re.search(pattern, line)
+    assert m, (pattern, line)
+    return m.group(1)
+
+
+def test_headline_shape():
+    fwd = lines((10, 8, 1000, 64), (10, 8, 1000, 64))
+    assert len(fwd) == 1 and fwd[0].startswith("scan_tp_kernel:")
+    assert "3 segments" in fwd[0] and "cuts at chunks 0,12,24,32" in fwd[0]
+    assert "240 workgroups" in fwd[0] and "workspace 0 bytes" in fwd[0]
+    bwd = lines((10, 8, 1000, 64), (10, 8, 1000, 64), backward=True)
+    assert len(bwd) == 1 and bwd[0].startswith("scan_tp_kernel: 3 scans")
+    assert "1 segment " in bwd[0] and "240 workgroups" in bwd[0]
+
+
+def test_long_chains_exchange_their_segment_sums():
+    fwd = lines((1, 16, 65536, 64), (1, 16, 65536, 64))
+    assert fwd[0].startswith("scan_tp_kernel (exchange):")
+    assert "16 segments of 4096 rows" in fwd[0] and "256 workgroups" in fwd[0]
+    need = int(field(fwd[0], r"workspace (\d+) bytes"))
+    lib = _native.load()
+    assert 0 < need <= lib.ftc_causal_dot_product_workspace_bytes(1, 16, 65536, 64, 64, 0)
+    # three scans of 16 chains would need segments of 412 chunks: the kernels that split L
+    bwd = lines((1, 16, 65536, 64), (1, 16, 65536, 64), backward=True)
+    assert bwd[0].startswith("scan_dma_kernel: 3 scans")
+    # config 4's operator shape
+    op = lines((10, 8, 4096, 64), (10, 8, 4096, 64))
+    assert op[0].startswith("scan_tp_kernel (exchange):") and "3 segments of 1408 rows" in op[0]
+
+
+def test_what_the_chain_parallel_kernel_leaves_to_the_others():
+    # rows that lie too far apart for one 32-bit descriptor per chain
+    far = (144 * 8192 * 65536, 8192 * 65536, 65536, 1)
+    out = lines((1, 144, 8192, 64), (1, 144, 8192, 64), strides=(far, far, far))
+    assert not out[0].startswith("scan_tp_kernel")
+    # more chains than two rounds of workgroups
+    many = lines((64, 16, 512, 64), (64, 16, 512, 64))
+    assert many[0].startswith("scan_dma_kernel")
+    # other state sizes and element types
+    assert lines((10, 8, 1000, 32), (10, 8, 1000, 32))[0].startswith("scan_dma_kernel")
+    assert lines((10, 8, 1000, 128), (10, 8, 1000, 128))[0].startswith("scan_mfma_kernel")
+    assert lines((4, 8, 1000, 64), (4, 8, 1000, 64), dtype=_native.FTC_BF16)[0] \
+        .startswith("scan_mfma_kernel")
+    assert lines((8, 16, 4096, 100), (8, 16, 4096, 100))[0].startswith("generic_scan_kernel")
+    assert lines((2, 2, 40, 10), (2, 2, 40, 3))[0].startswith("generic_scan_kernel")
+    # nothing to do
+    assert lines((0, 8, 100, 64), (0, 8, 100, 64)) == []
+
+
+@pytest.mark.parametrize("L", [33, 129, 500, 1000, 1500, 2048])
+@pytest.mark.parametrize("chains", [(2, 8), (5, 8), (10, 8), (30, 4)])
+def test_cut_chains(chains, L):
+    """Cuts at multiples of four chunks, the last one at the end, at most 256 workgroups, and
+    the longest workgroup (a chunk walked for its state alone counted as 0.4 of a full one)
+    no longer than with equal segments (of whole groups of four chunks)."""
+    N, H = chains
+    line = lines((N, H, L, 64), (N, H, L, 64))[0]
+    if not line.startswith("scan_tp_kernel:"):
+        return
+    cuts = [int(x) for x in field(line, r"cuts at chunks ([\d,]*\d)").split(",")]
+    nseg = int(field(line, r"(\d+) segments? of"))
+    assert len(cuts) == nseg + 1 and cuts[0] == 0 and cuts[-1] == (L + 31) // 32
+    assert all(c % 4 == 0 for c in cuts[:-1])
+    lengths = [b - a for a, b in zip(cuts, cuts[1:])]
+    assert all(x > 0 for x in lengths)
+    longest = max(0.4 * a + (b - a) for a, b in zip(cuts, cuts[1:]))
+    step = -(-(-(-cuts[-1] // nseg)) // 4) * 4   # equal segments of whole groups of four
+    equal = [min(i * step, cuts[-1]) for i in range(nseg + 1)]
+    assert longest <= max(0.4 * a + (b - a) for a, b in zip(equal, equal[1:])) + 1e-9
+    assert N * H * nseg <= 256 and int(field(line, r"(\d+) workgroups")) == N * H * nseg
+
+
+SWEEP = [(N, H, L, E, M) for (N, H) in [(1, 1), (1, 16), (2, 8), (10, 8), (64, 16)]
+         for L in [1, 64, 1000, 4096, 20000] for (E, M) in [(64, 64), (32, 128), (96, 64), (25, 70)]]
+
+
+@pytest.mark.parametrize("backward", [False, True])
+def test_the_workspace_query_covers_every_launch(backward):
+    lib = _native.load()
+    query = lib.ftc_causal_dot_backward_workspace_bytes if backward \
+        else lib.ftc_causal_dot_product_workspace_bytes
+    for dtype in (_native.FTC_F32, _native.FTC_BF16):
+        for N, H, L, E, M in SWEEP:
+            granted = query(N, H, L, E, M, dtype)
+            assert granted >= 0
+            for line in lines((N, H, L, E), (N, H, L, M), dtype=dtype, backward=backward):
+                need = int(field(line, r"workspace (\d+) bytes")) if "workspace" in line else 0
+                assert need <= granted, (N, H, L, E, M, dtype, line, granted)
