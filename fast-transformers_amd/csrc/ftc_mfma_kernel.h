@@ -618,11 +618,21 @@ __global__ __launch_bounds__(kWave) void scan_mfma_kernel(uint32_t *__restrict__
     // position-major operands pass through LDS in their own element type: 16-byte global
     // loads (lane = (row within the load, 16 bytes of it)), 16-byte LDS writes, element-wide
     // LDS reads by column
+    // (rows of 96 values do not divide the wavefront: the lanes left over after the last whole
+    // row of a load, and rows past the chunk in the last load, neither fetch nor store)
     constexpr int kBtLanes = D * BB / 16, kVtLanes = F * BV / 16;      // lanes per row
     constexpr int kBtRows = kWave / kBtLanes, kVtRows = kWave / kVtLanes;  // rows per load
-    constexpr int kBtLoads = kChunk / kBtRows, kVtLoads = kChunk / kVtRows;
+    constexpr int kBtLoads = (kChunk + kBtRows - 1) / kBtRows,
+                  kVtLoads = (kChunk + kVtRows - 1) / kVtRows;
     const uint32_t bt_lane = (uint32_t)(lane / kBtLanes) * b_slb + 16u * (lane % kBtLanes);
     const uint32_t vt_lane = (uint32_t)(lane / kVtLanes) * v_slb + 16u * (lane % kVtLanes);
+    constexpr uint32_t kNoRow = 0x80000000u;  // an offset outside every descriptor: reads zero
+    auto bt_row = [&](int i) -> int {
+        return lane < kBtRows * kBtLanes ? i * kBtRows + lane / kBtLanes : kChunk;
+    };
+    auto vt_row = [&](int i) -> int {
+        return lane < kVtRows * kVtLanes ? i * kVtRows + lane / kVtLanes : kChunk;
+    };
     const uint32_t o_lane = ln * o_slb + 4u * BO * g;
 
     // first row of chunk c relative to the segment (REV walks down from the end and its
@@ -660,29 +670,29 @@ __global__ __launch_bounds__(kWave) void scan_mfma_kernel(uint32_t *__restrict__
 #pragma unroll
         for (int i = 0; i < kBtLoads; i++)
             raw[i] = __builtin_amdgcn_raw_buffer_load_b128(
-                b_rs, off + (uint32_t)(i * kBtRows) * b_slb, 0, 0);
+                b_rs, bt_row(i) < kChunk ? off + (uint32_t)(i * kBtRows) * b_slb : kNoRow, 0, 0);
     };
     auto fetch_vt_into = [&](int row0, u32x4 (&raw)[kVtLoads]) {
         const uint32_t off = vt_lane + (uint32_t)row0 * v_slb;
 #pragma unroll
         for (int i = 0; i < kVtLoads; i++)
             raw[i] = __builtin_amdgcn_raw_buffer_load_b128(
-                v_rs, off + (uint32_t)(i * kVtRows) * v_slb, 0, 0);
+                v_rs, vt_row(i) < kChunk ? off + (uint32_t)(i * kVtRows) * v_slb : kNoRow, 0, 0);
     };
     // fetched rows -> LDS tile `buf` (row-major, 32 rows)
     auto stash_bt_from = [&](int buf, const u32x4 (&raw)[kBtLoads]) {
         char *tile = (char *)bt_lds[buf];
 #pragma unroll
         for (int i = 0; i < kBtLoads; i++)
-            *(lds_u32x4 *)(tile + (i * kBtRows + lane / kBtLanes) * (D * BB) +
-                           16 * (lane % kBtLanes)) = raw[i];
+            if (bt_row(i) < kChunk)
+                *(lds_u32x4 *)(tile + bt_row(i) * (D * BB) + 16 * (lane % kBtLanes)) = raw[i];
     };
     auto stash_vt_from = [&](int buf, const u32x4 (&raw)[kVtLoads]) {
         char *tile = (char *)vt_lds[buf];
 #pragma unroll
         for (int i = 0; i < kVtLoads; i++)
-            *(lds_u32x4 *)(tile + (i * kVtRows + lane / kVtLanes) * (F * BV) +
-                           16 * (lane % kVtLanes)) = raw[i];
+            if (vt_row(i) < kChunk)
+                *(lds_u32x4 *)(tile + vt_row(i) * (F * BV) + 16 * (lane % kVtLanes)) = raw[i];
     };
     auto fetch_bt = [&](int row0) { fetch_bt_into(row0, bt_raw); };
     auto fetch_vt = [&](int row0) { fetch_vt_into(row0, vt_raw); };
