@@ -10,6 +10,7 @@
 //   dV      = scan_rev(a=K, b=Q, v=G)      state E x M
 #include <stdarg.h>
 #include <stdio.h>
+#include <stdlib.h>
 #include <string.h>
 
 #include <algorithm>
@@ -91,11 +92,222 @@ int read_dims(const ftc_tensor4 *q, const ftc_tensor4 *v, Dims *d) {
     return FTC_OK;
 }
 
+// ---- odd widths on the matrix cores: dense zero-padded copies --------------------------
+//
+// A scan whose rows are not 32, 64, 96 or 128 (a, b) and a multiple of 32 (v, out) values
+// wide, or whose rows are misaligned or too far apart, is run on zero-padded dense copies
+// of its operands when the workspace has room for them: padding columns of a and b add
+// nothing to any dot product, padding columns of v produce output columns that are dropped
+// when the result is copied back.  Two extra passes over the rows, but the matrix-core
+// kernels are several times faster than the generic one.
+
+// Rows of a strided operand of width w <-> rows of a dense buffer of width wp (a multiple of
+// 32), chain after chain.  A lane moves one 16-byte group of the dense row (T: uint32_t for
+// fp32, uint16_t for bf16 elements); blockIdx.y walks the chains.
+template <typename T, bool PAD>
+__global__ __launch_bounds__(256) void pad_rows_kernel(T *strided, int64_t sn, int64_t sh, int64_t sl,
+                                                       int64_t H, int64_t L, int64_t chains, int w,
+                                                       int wp, T *dense) {
+    constexpr int PER = 16 / sizeof(T);
+    typedef T Vec __attribute__((ext_vector_type(PER)));
+    const uint32_t groups = (uint32_t)wp / PER;
+    const uint32_t j = blockIdx.x * 256u + threadIdx.x;
+    if (j >= (uint32_t)L * groups) return;
+    const uint32_t l = j / groups, c0 = (j % groups) * PER;
+    for (int64_t chain = blockIdx.y; chain < chains; chain += gridDim.y) {
+        T *row = strided + (chain / H) * sn + (chain % H) * sh + (int64_t)l * sl;
+        Vec *slot = (Vec *)(dense + (chain * L + l) * wp + c0);
+        if (PAD) {
+            Vec x;
+#pragma unroll
+            for (int e = 0; e < PER; e++) x[e] = (int)(c0 + e) < w ? row[c0 + e] : (T)0;
+            *slot = x;
+        } else {
+            const Vec x = *slot;
+#pragma unroll
+            for (int e = 0; e < PER; e++)
+                if ((int)(c0 + e) < w) row[c0 + e] = x[e];
+        }
+    }
+}
+
+template <bool PAD>
+void launch_pad_rows(void *strided, int64_t sn, int64_t sh, int64_t sl, int64_t N, int64_t H,
+                     int64_t L, int w, int wp, int esz, void *dense, hipStream_t stream) {
+    const int per = 16 / esz;
+    const dim3 grid((unsigned)((L * (wp / per) + 255) / 256), (unsigned)std::min<int64_t>(N * H, 65535));
+    if (esz == 4)
+        hipLaunchKernelGGL((pad_rows_kernel<uint32_t, PAD>), grid, dim3(256), 0, stream,
+                           (uint32_t *)strided, sn, sh, sl, H, L, N * H, w, wp, (uint32_t *)dense);
+    else
+        hipLaunchKernelGGL((pad_rows_kernel<uint16_t, PAD>), grid, dim3(256), 0, stream,
+                           (uint16_t *)strided, sn, sh, sl, H, L, N * H, w, wp, (uint16_t *)dense);
+}
+
+constexpr int64_t kPadMinRows = 8192;
+int64_t round_up(int64_t x, int64_t m) { return (x + m - 1) / m * m; }
+// padded widths of a D x F scan (0: the matrix-core kernels take no such state)
+int padded_rows(int64_t D) { return D <= 32 ? 32 : D <= 64 ? 64 : D <= 96 ? 96 : D <= 128 ? 128 : 0; }
+
+int64_t scan_workspace_bytes(int64_t N, int64_t H, int64_t L, int64_t D, int64_t F,
+                             bool with_pad = true);
+
+// workspace of the padded route of one scan: the scan's own, then dense copies of all four
+// operands (fp32 sizes: an upper bound)
+int64_t padded_scan_workspace_bytes(int64_t N, int64_t H, int64_t L, int64_t D, int64_t F) {
+    const int64_t Dp = padded_rows(D), Fp = round_up(F, 32), rows = N * H * L;
+    int widths[kMfmaMaxSlices];
+    if (Dp == 0 || (Dp == D && Fp == F) || rows < kPadMinRows ||
+        mfma_slice_widths(Dp, Fp, widths) == 0)
+        return 0;
+    return round_up(scan_workspace_bytes(N, H, L, Dp, Fp), 256) +
+           2 * round_up(rows * Dp * 4, 256) + 2 * round_up(rows * Fp * 4, 256);
+}
+
+int run_scans(const ScanDesc *scans, int n, int64_t N, int64_t H, int64_t L, void *workspace,
+              size_t workspace_bytes, hipStream_t stream, bool may_pad);
+
+// The scans of a call that the matrix-core kernels do not take as they are, run on padded
+// copies: `take[i]` says which.  An operand that several scans read is copied once; an
+// operand whose rows are fine where they lie is used in place.  Returns with *done = false
+// (nothing launched) when the workspace has no room.
+int padded_scans(const ScanDesc *scans, int n, const bool *take, int64_t N, int64_t H, int64_t L,
+                 void *workspace, size_t workspace_bytes, hipStream_t stream, bool *done) {
+    *done = false;
+    const int64_t rows = N * H * L;
+    auto esz = [](int dtype) { return dtype == FTC_F32 ? 4 : 2; };
+    struct Copy {
+        const void *ptr;  // the caller's tensor
+        int64_t sn, sh, sl;
+        int dtype, width, padded;
+        bool is_output;
+        char *dense;
+    };
+    Copy copies[4 * kMfmaMaxScans];
+    int ncopies = 0;
+    ScanDesc work[kMfmaMaxScans];
+    int nwork = 0;
+    int64_t ws_scan = 0;
+    auto copy_of = [&](const void *ptr, int64_t sn, int64_t sh, int64_t sl, int dtype, int width,
+                       int padded, bool is_output) -> int {
+        for (int i = 0; i < ncopies; i++)
+            if (copies[i].ptr == ptr && copies[i].sn == sn && copies[i].sh == sh &&
+                copies[i].sl == sl && copies[i].width == width && copies[i].padded == padded &&
+                !copies[i].is_output && !is_output)
+                return i;
+        copies[ncopies] = Copy{ptr, sn, sh, sl, dtype, width, padded, is_output, nullptr};
+        return ncopies++;
+    };
+    int which[kMfmaMaxScans][4];
+    for (int i = 0; i < n; i++) {
+        if (!take[i]) continue;
+        const ScanDesc &sc = scans[i];
+        const int Dp = padded_rows(sc.a.width), Fp = (int)round_up(sc.v.width, 32);
+        ws_scan = std::max(ws_scan, round_up(scan_workspace_bytes(N, H, L, Dp, Fp), 256));
+        const Operand *in[3] = {&sc.a, &sc.b, &sc.v};
+        const int target[3] = {Dp, Dp, Fp};
+        for (int k = 0; k < 3; k++) {
+            const Operand &o = *in[k];
+            which[nwork][k] = o.width == target[k] && mfma_operand_in_place(o.ptr, o.stride_n, o.stride_h,
+                                                                           o.stride_l, o.dtype, o.width, L)
+                                  ? -1
+                                  : copy_of(o.ptr, o.stride_n, o.stride_h, o.stride_l, o.dtype, o.width,
+                                            target[k], false);
+        }
+        const OperandOut &o = sc.out;
+        which[nwork][3] = o.width == Fp && mfma_operand_in_place(o.ptr, o.stride_n, o.stride_h, o.stride_l,
+                                                                 o.dtype, o.width, L)
+                              ? -1
+                              : copy_of(o.ptr, o.stride_n, o.stride_h, o.stride_l, o.dtype, o.width, Fp, true);
+        work[nwork++] = sc;
+    }
+    int64_t need = ws_scan;
+    for (int i = 0; i < ncopies; i++) need += round_up(rows * copies[i].padded * esz(copies[i].dtype), 256);
+    if (!plan_only() && (!workspace || (int64_t)workspace_bytes < need || (uintptr_t)workspace % 256 != 0))
+        return FTC_OK;
+    char *base = (char *)workspace + ws_scan;
+    for (int i = 0; i < ncopies; i++) {
+        copies[i].dense = base;
+        base += round_up(rows * copies[i].padded * esz(copies[i].dtype), 256);
+    }
+    for (int s = 0; s < nwork; s++) {
+        Operand *in[3] = {&work[s].a, &work[s].b, &work[s].v};
+        for (int k = 0; k < 3; k++)
+            if (which[s][k] >= 0) {
+                const Copy &c = copies[which[s][k]];
+                const int64_t w = c.padded;
+                *in[k] = Operand{c.dense, H * L * w, L * w, w, c.dtype, (int32_t)w};
+            }
+        if (which[s][3] >= 0) {
+            const Copy &c = copies[which[s][3]];
+            const int64_t w = c.padded;
+            work[s].out = OperandOut{c.dense, H * L * w, L * w, w, c.dtype, (int32_t)w};
+        }
+    }
+    int nin = 0, nout = 0;
+    for (int i = 0; i < ncopies; i++) (copies[i].is_output ? nout : nin)++;
+    if (plan_only()) {
+        note_plan("pad_rows_kernel: %d operand%s copied into zero-padded rows, %d result%s copied "
+                  "back, workspace %lld bytes", nin, nin == 1 ? "" : "s", nout, nout == 1 ? "" : "s",
+                  (long long)need);
+    } else {
+        for (int i = 0; i < ncopies; i++)
+            if (!copies[i].is_output)
+                launch_pad_rows<true>((void *)copies[i].ptr, copies[i].sn, copies[i].sh, copies[i].sl,
+                                      N, H, L, copies[i].width, copies[i].padded,
+                                      esz(copies[i].dtype), copies[i].dense, stream);
+    }
+    int rc = run_scans(work, nwork, N, H, L, workspace, (size_t)ws_scan, stream, false);
+    if (rc) return rc;
+    if (!plan_only()) {
+        for (int i = 0; i < ncopies; i++)
+            if (copies[i].is_output)
+                launch_pad_rows<false>((void *)copies[i].ptr, copies[i].sn, copies[i].sh, copies[i].sl,
+                                       N, H, L, copies[i].width, copies[i].padded,
+                                       esz(copies[i].dtype), copies[i].dense, stream);
+        hipError_t err = hipGetLastError();
+        if (err != hipSuccess)
+            return fail(FTC_ERR_HIP, "padding launch failed: %s", hipGetErrorString(err));
+    }
+    *done = true;
+    return FTC_OK;
+}
+
+// whether a scan that the matrix-core kernels do not take as it is may go the padded way
+bool pad_eligible(const ScanDesc &sc, int64_t rows) {
+    int widths[kMfmaMaxSlices];
+    const int Dp = padded_rows(sc.a.width);
+    if (sc.initial.ptr || sc.final_.ptr || Dp == 0 || rows < kPadMinRows) return false;
+    if (const char *env = getenv("FTC_PAD"))  // tuning aid
+        if (atoi(env) == 0) return false;
+    return mfma_slice_widths(Dp, round_up(sc.v.width, 32), widths) > 0;
+}
+
 // Runs a list of independent scans.  A scan whose shape the MFMA kernels cover is cut into
 // column slices; consecutive slices (of any of the scans) that share widths and element
 // types go out in one launch.  Everything else takes the generic path.
 int run_scans(const ScanDesc *scans, int n, int64_t N, int64_t H, int64_t L, void *workspace,
-              size_t workspace_bytes, hipStream_t stream) {
+              size_t workspace_bytes, hipStream_t stream, bool may_pad = true) {
+    // which scans the matrix-core kernels take as they are
+    bool native[kMfmaMaxScans], padded[kMfmaMaxScans];
+    bool any_padded = false;
+    if (n > kMfmaMaxScans) return fail(FTC_ERR_INVALID, "too many scans");
+    for (int i = 0; i < n; i++) {
+        int widths[kMfmaMaxSlices];
+        int nslices = mfma_slice_widths(scans[i].a.width, scans[i].v.width, widths);
+        for (int j = 0, col = 0; j < nslices; col += widths[j], j++)
+            if (!mfma_scan_supported(mfma_slice(scans[i], col, widths[j]), L)) nslices = 0;
+        native[i] = nslices > 0;
+        padded[i] = !native[i] && may_pad && pad_eligible(scans[i], N * H * L);
+        any_padded = any_padded || padded[i];
+    }
+    if (any_padded) {
+        bool done = false;
+        const int rc = padded_scans(scans, n, padded, N, H, L, workspace, workspace_bytes, stream, &done);
+        if (rc) return rc;
+        if (!done)
+            for (int i = 0; i < n; i++) padded[i] = false;
+    }
     ScanDesc batch[kMfmaMaxScans];
     int nbatch = 0;
     auto flush = [&]() -> int {
@@ -105,11 +317,8 @@ int run_scans(const ScanDesc *scans, int n, int64_t N, int64_t H, int64_t L, voi
         return rc;
     };
     for (int i = 0; i < n; i++) {
-        int widths[kMfmaMaxSlices];
-        int nslices = mfma_slice_widths(scans[i].a.width, scans[i].v.width, widths);
-        for (int j = 0, col = 0; j < nslices; col += widths[j], j++)
-            if (!mfma_scan_supported(mfma_slice(scans[i], col, widths[j]), L)) nslices = 0;
-        if (nslices == 0) {
+        if (padded[i]) continue;
+        if (!native[i]) {
             int rc = flush();
             if (rc) return rc;
             rc = generic_scan(scans[i].a, scans[i].b, scans[i].v, scans[i].out, N, H, L,
@@ -118,6 +327,8 @@ int run_scans(const ScanDesc *scans, int n, int64_t N, int64_t H, int64_t L, voi
             if (rc) return rc;
             continue;
         }
+        int widths[kMfmaMaxSlices];
+        const int nslices = mfma_slice_widths(scans[i].a.width, scans[i].v.width, widths);
         for (int j = 0, col = 0; j < nslices; col += widths[j], j++) {
             const ScanDesc slice = mfma_slice(scans[i], col, widths[j]);
             if (nbatch == kMfmaMaxScans || (nbatch > 0 && !mfma_scan_same_launch(batch[0], slice))) {
@@ -131,13 +342,16 @@ int run_scans(const ScanDesc *scans, int n, int64_t N, int64_t H, int64_t L, voi
 }
 
 // Upper bound over every way run_scans may slice and group scans of these widths.
-int64_t scan_workspace_bytes(int64_t N, int64_t H, int64_t L, int64_t D, int64_t F) {
+// `with_pad` = false leaves out the padded copies: what a call needs at the least (without
+// them such a scan runs on the generic kernel).
+int64_t scan_workspace_bytes(int64_t N, int64_t H, int64_t L, int64_t D, int64_t F, bool with_pad) {
     int64_t need = generic_scan_workspace_bytes(N, H, L, D, F);
     int widths[kMfmaMaxSlices];
     const int nslices = mfma_slice_widths(D, F, widths);
     for (int j = 0; j < nslices; j++)
         for (int k = 1; k <= kMfmaMaxScans; k++)
             need = std::max(need, mfma_scan_workspace_bytes(N, H, L, D, widths[j], k));
+    if (nslices == 0 && with_pad) need = std::max(need, padded_scan_workspace_bytes(N, H, L, D, F));
     return need;
 }
 
@@ -236,6 +450,9 @@ int ftc_causal_dot_product_static(const ftc_tensor4 *queries, const ftc_tensor4 
     if (d.N * d.H * d.L * d.M > 0 && d.E > 0) {
         need = ftc_causal_dot_product_workspace_bytes(d.N, d.H, d.L, d.E, d.M, queries->dtype);
         if (need < 0) return (int)need;
+        // widths that would run on padded copies do without them when the array has no room
+        if (need > (int64_t)FTC_STATIC_SCRATCH_BYTES)
+            need = scan_workspace_bytes(d.N, d.H, d.L, d.E, d.M, false);
     }
     if (need > (int64_t)FTC_STATIC_SCRATCH_BYTES)
         return fail(FTC_ERR_WORKSPACE,
@@ -300,7 +517,16 @@ int64_t ftc_causal_dot_backward_workspace_bytes(int64_t N, int64_t H, int64_t L,
     if (N * H * L == 0 || M == 0 || E == 0) return 0;
     if (E > kGenericMaxDim || M > kGenericMaxDim)
         return fail(FTC_ERR_UNSUPPORTED, "E and M must be at most %d", kGenericMaxDim);
-    return std::max(scan_workspace_bytes(N, H, L, E, M), scan_workspace_bytes(N, H, L, M, E));
+    int64_t need = std::max(scan_workspace_bytes(N, H, L, E, M), scan_workspace_bytes(N, H, L, M, E));
+    // the padded route of the three scans together: Q, K, dQ, dK and V, G, dV as dense rows
+    if (padded_scan_workspace_bytes(N, H, L, E, M) > 0 || padded_scan_workspace_bytes(N, H, L, M, E) > 0) {
+        int64_t ws = 0;
+        if (padded_rows(E)) ws = std::max(ws, scan_workspace_bytes(N, H, L, padded_rows(E), round_up(M, 32)));
+        if (padded_rows(M)) ws = std::max(ws, scan_workspace_bytes(N, H, L, padded_rows(M), round_up(E, 32)));
+        need = std::max(need, round_up(ws, 256) + 4 * round_up(N * H * L * round_up(E, 32) * 4, 256) +
+                                  3 * round_up(N * H * L * round_up(M, 32) * 4, 256));
+    }
+    return need;
 }
 
 int ftc_causal_dot_backward(const ftc_tensor4 *queries, const ftc_tensor4 *keys,
@@ -354,14 +580,17 @@ int ftc_causal_dot_plan(const ftc_tensor4 *queries, const ftc_tensor4 *keys,
         return fail(FTC_ERR_INVALID, "null argument");
     // data pointers are never read here: absent ones are replaced by a placeholder so that
     // the checks of the real entry points apply unchanged
-    auto with_ptr = [](ftc_tensor4 t) {
-        if (!t.ptr) t.ptr = (void *)(uintptr_t)4096;
+    uintptr_t placeholder = 0;  // (distinct ones: tensors are told apart by their pointers)
+    auto with_ptr = [&](ftc_tensor4 t) {
+        placeholder += 4096;
+        if (!t.ptr) t.ptr = (void *)placeholder;
         return t;
     };
     const ftc_tensor4 q = with_ptr(*queries), k = with_ptr(*keys), v = with_ptr(*values);
     auto dense = [&](int64_t width, int dtype) {
         ftc_tensor4 t;
-        t.ptr = (void *)(uintptr_t)4096;
+        placeholder += 4096;
+        t.ptr = (void *)placeholder;
         t.dtype = dtype;
         t.size[0] = q.size[0], t.size[1] = q.size[1], t.size[2] = q.size[2], t.size[3] = width;
         t.stride[3] = 1, t.stride[2] = width, t.stride[1] = t.stride[2] * t.size[2];

@@ -107,6 +107,10 @@ constexpr int kMfmaMaxSlices = 16;  // column slices per scan
 // Widths of the column slices that cover F output columns for state rows of width D;
 // returns their number (0: this shape does not go to the MFMA path).
 int mfma_slice_widths(int64_t D, int64_t F, int (&widths)[kMfmaMaxSlices]);
+// Whether the MFMA kernels can read (or write) rows of this width where they lie: 16-byte
+// aligned, at most 65536 elements apart.
+bool mfma_operand_in_place(const void *ptr, int64_t stride_n, int64_t stride_h, int64_t stride_l,
+                           int dtype, int width, int64_t L);
 // Column slice [col0, col0 + width) of a scan: same a and b rows, offset v and out rows.
 ScanDesc mfma_slice(const ScanDesc &scan, int col0, int width);
 bool mfma_scan_supported(const ScanDesc &scan, int64_t L);

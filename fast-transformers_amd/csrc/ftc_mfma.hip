@@ -227,6 +227,11 @@ bool mfma_scan_same_launch(const ScanDesc &x, const ScanDesc &y) {
     return combo_of(x) == combo_of(y) && x.a.width == y.a.width && x.v.width == y.v.width;
 }
 
+bool mfma_operand_in_place(const void *ptr, int64_t stride_n, int64_t stride_h, int64_t stride_l,
+                           int dtype, int width, int64_t L) {
+    return (L <= 1 || stride_ok(stride_l, width)) && aligned16(ptr, stride_n, stride_h, stride_l, dtype);
+}
+
 bool mfma_scan_supported(const ScanDesc &sd, int64_t L) {
     const Operand &a = sd.a, &b = sd.b, &v = sd.v;
     const OperandOut &out = sd.out;

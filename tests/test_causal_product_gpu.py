@@ -376,6 +376,11 @@ BF16_SHAPES = {
     "e40_m24": (2, 2, 300, 40, 24, 12),
     # column slices
     "e128_m128": (1, 3, 700, 128, 128, 22),
+    # 96-row states: bf16 rows of 96 values are 12 lanes of 16 bytes, which does not divide a
+    # wavefront (the row staging once left the chunk's last two rows unwritten)
+    "e64_m96": (2, 4, 1200, 64, 96, 23),
+    "e96_m64": (2, 4, 1200, 96, 64, 24),
+    "e96_m96": (1, 3, 500, 96, 96, 25),
 }
 
 
@@ -741,6 +746,78 @@ def test_chain_parallel_kernel_with_exchange(cp, shape):
     exacts = oracle.backward(Q.double(), K.double(), V.double(), G.double())
     for name, got, ref, ex in zip(("dQ", "dK", "dV"), (dq, dk, dv), refs, exacts):
         _gate_against_float64("tpx %s %s" % (shape, name), got.cpu(), ref, ex)
+
+
+ODD_SHAPES = [
+    # N, H, L, E, M, dtype: widths that the matrix-core kernels do not take as they are
+    (2, 4, 2000, 25, 64, torch.float32),     # queries and keys padded, values in place
+    (2, 4, 1100, 100, 100, torch.float32),   # everything padded, 128-row states
+    (3, 3, 1000, 10, 3, torch.float32),      # tiny widths
+    (1, 2, 5000, 70, 33, torch.float32),     # 96-row state one way, 64-row state the other
+    (2, 4, 1200, 48, 80, torch.bfloat16),    # bf16 rows
+    (1, 4, 2500, 130, 40, torch.float32),    # E beyond 128: dV stays on the generic kernel
+]
+
+
+@pytest.mark.parametrize("shape", ODD_SHAPES, ids=lambda s: "n%d_h%d_l%d_e%d_m%d_%s" % (s[:5] + (str(s[5])[6:],)))
+def test_odd_widths_run_on_padded_copies(cp, shape):
+    """Rows that are not 32/64/96/128 (a, b) or a multiple of 32 (v, out) values wide are
+    copied into zero-padded dense rows for the matrix-core kernels when there are enough of
+    them; (N, L, H, X) views; against the CPU checker (bf16: 2e-2 on identical rounded inputs)."""
+    from fast_transformers_amd import _native
+    N, H, L, E, M, dtype = shape
+    Q, K, V, G = oracle.make_inputs(N, H, L, E, M, seed=500 + E)
+    Q, K, V = (t.to(dtype) for t in (Q, K, V))
+    nlh = lambda t: t.permute(0, 2, 1, 3).contiguous().cuda().permute(0, 2, 1, 3)
+    q, k, v, g = (nlh(t) for t in (Q, K, V, G))
+    out = torch.full((N, L, H, M), float("nan"), device="cuda").permute(0, 2, 1, 3)
+    cp.causal_dot_product_hip(q, k, v, out)
+    if E <= 128:
+        assert _native.load().ftc_last_kernel() != b"generic_scan_kernel"
+    dq, dk, dv = (torch.full((N, L, H, X), float("nan"), device="cuda", dtype=dtype).permute(0, 2, 1, 3)
+                  for X in (E, E, M))
+    cp.causal_dot_backward_hip(q, k, v, g, dq, dk, dv)
+    torch.cuda.synchronize()
+    cp.check_workspaces()
+    Qf, Kf, Vf = Q.float(), K.float(), V.float()
+    want = (oracle.forward(Qf, Kf, Vf),) + tuple(oracle.backward(Qf, Kf, Vf, G))
+    tol = 1e-4 if dtype == torch.float32 else 2e-2
+    for name, got, ref in zip(("product", "dQ", "dK", "dV"), (out, dq, dk, dv), want):
+        assert torch.isfinite(got).all(), name
+        assert scale_error(got.float().cpu(), ref) <= tol, name
+
+
+def test_misaligned_rows_run_on_dense_copies(cp):
+    """Rows of a supported width that start 4 bytes off a 16-byte boundary: the matrix-core
+    kernels cannot read them where they lie; dense copies are made instead of falling back
+    to the generic kernel.  Without room in the workspace the generic kernel still serves."""
+    from fast_transformers_amd import _native
+    N, H, L, E, M = 2, 4, 1500, 64, 64
+    Q, K, V, _ = oracle.make_inputs(N, H, L, E, M, seed=77)
+    wide = torch.zeros(N, H, L, 1 + E, device="cuda")
+    wide[..., 1:] = Q.cuda()
+    q = wide[..., 1:]                                   # rows start at byte 4 of a 260-byte pitch
+    out = torch.full((N, H, L, M), float("nan"), device="cuda")
+    cp.causal_dot_product_hip(q, K.cuda(), V.cuda(), out)
+    assert _native.load().ftc_last_kernel() != b"generic_scan_kernel"
+    torch.cuda.synchronize()
+    want = oracle.forward(Q, K, V)
+    assert scale_error(out.cpu(), want) <= 1e-4
+    # the entry point without a workspace has 48 MiB of scratch: too little for the copies
+    big_n = 64
+    Qb, Kb, Vb, _ = oracle.make_inputs(big_n, H, L, 25, M, seed=78)
+    outb = torch.full((big_n, H, L, M), float("nan"), device="cuda")
+    dev = (Qb.cuda(), Kb.cuda(), Vb.cuda(), outb)
+    d = [_native.describe(t) for t in dev]
+    import ctypes
+    rc = _native.load().ftc_causal_dot_product_static(
+        ctypes.byref(d[0]), ctypes.byref(d[1]), ctypes.byref(d[2]), ctypes.byref(d[3]),
+        ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+    assert rc == 0, _native.last_error()
+    assert _native.load().ftc_last_kernel() == b"generic_scan_kernel"
+    torch.cuda.synchronize()
+    assert scale_error(outb[:2].cpu(), oracle.forward(Qb[:2], Kb[:2], Vb[:2])) <= 1e-4
+    del dev
 
 
 def test_rows_far_apart_leave_the_chain_parallel_kernel(cp):

@@ -61,8 +61,21 @@ def test_what_the_chain_parallel_kernel_leaves_to_the_others():
     assert lines((10, 8, 1000, 128), (10, 8, 1000, 128))[0].startswith("scan_mfma_kernel")
     assert lines((4, 8, 1000, 64), (4, 8, 1000, 64), dtype=_native.FTC_BF16)[0] \
         .startswith("scan_mfma_kernel")
-    assert lines((8, 16, 4096, 100), (8, 16, 4096, 100))[0].startswith("generic_scan_kernel")
+    # odd widths: zero-padded dense copies for the matrix-core kernels when there are enough
+    # rows to pay for the extra launches; states of more than 128 rows stay generic
+    # (queries and keys are copied, the values and the product stay where they are; in the
+    # backward the two copies serve all three scans, and dQ and dK are copied back)
+    odd = lines((8, 16, 4096, 25), (8, 16, 4096, 64))
+    assert odd[0].startswith("pad_rows_kernel: 2 operands") and "0 results" in odd[0]
+    assert odd[1].startswith("scan_dma_kernel") and "state 32 x 64" in odd[1]
+    odd = lines((8, 16, 4096, 25), (8, 16, 4096, 64), backward=True)
+    assert odd[0].startswith("pad_rows_kernel: 2 operands") and "2 results" in odd[0]
+    assert odd[1].startswith("scan_dma_kernel: 2 scans") and "state 64 x 32" in odd[1]
+    wide = lines((8, 16, 4096, 100), (8, 16, 4096, 100), backward=True)
+    assert wide[0].startswith("pad_rows_kernel: 4 operands") and "3 results" in wide[0]
+    assert wide[1].startswith("scan_mfma_kernel") and "state 128 x 32" in wide[1]
     assert lines((2, 2, 40, 10), (2, 2, 40, 3))[0].startswith("generic_scan_kernel")
+    assert lines((1, 2, 8192, 200), (1, 2, 8192, 64))[0].startswith("generic_scan_kernel")
     # nothing to do
     assert lines((0, 8, 100, 64), (0, 8, 100, 64)) == []
 
