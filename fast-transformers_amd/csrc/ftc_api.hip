@@ -289,10 +289,26 @@ bool pad_eligible(const ScanDesc &sc, int64_t rows) {
 int run_scans(const ScanDesc *scans, int n, int64_t N, int64_t H, int64_t L, void *workspace,
               size_t workspace_bytes, hipStream_t stream, bool may_pad = true) {
     // which scans the matrix-core kernels take as they are
-    bool native[kMfmaMaxScans], padded[kMfmaMaxScans];
+    bool native[kMfmaMaxScans], padded[kMfmaMaxScans], taken[kMfmaMaxScans] = {};
     bool any_padded = false;
     if (n > kMfmaMaxScans) return fail(FTC_ERR_INVALID, "too many scans");
+    // Wide states and widths that are multiples of 4: the scans of one shape go to the
+    // chain-parallel kernel together where it takes them (64 x 64 finds it below).
     for (int i = 0; i < n; i++) {
+        if (taken[i] || (scans[i].a.width == 64 && scans[i].v.width == 64)) continue;
+        ScanDesc group[kMfmaMaxScans];
+        int members[kMfmaMaxScans], ngroup = 0;
+        for (int j = i; j < n; j++)
+            if (!taken[j] && scans[j].a.width == scans[i].a.width && scans[j].v.width == scans[i].v.width)
+                members[ngroup] = j, group[ngroup++] = scans[j];
+        if (!mfma_tp_takes(group, ngroup, N, H, L)) continue;
+        const int rc = mfma_scan(group, ngroup, N, H, L, workspace, workspace_bytes, stream);
+        if (rc) return rc;
+        for (int k = 0; k < ngroup; k++) taken[members[k]] = true;
+    }
+    for (int i = 0; i < n; i++) {
+        native[i] = padded[i] = false;
+        if (taken[i]) continue;
         int widths[kMfmaMaxSlices];
         int nslices = mfma_slice_widths(scans[i].a.width, scans[i].v.width, widths);
         for (int j = 0, col = 0; j < nslices; col += widths[j], j++)
@@ -317,7 +333,7 @@ int run_scans(const ScanDesc *scans, int n, int64_t N, int64_t H, int64_t L, voi
         return rc;
     };
     for (int i = 0; i < n; i++) {
-        if (padded[i]) continue;
+        if (padded[i] || taken[i]) continue;
         if (!native[i]) {
             int rc = flush();
             if (rc) return rc;
@@ -352,6 +368,8 @@ int64_t scan_workspace_bytes(int64_t N, int64_t H, int64_t L, int64_t D, int64_t
         for (int k = 1; k <= kMfmaMaxScans; k++)
             need = std::max(need, mfma_scan_workspace_bytes(N, H, L, D, widths[j], k));
     if (nslices == 0 && with_pad) need = std::max(need, padded_scan_workspace_bytes(N, H, L, D, F));
+    for (int k = 1; k <= kMfmaMaxScans; k++)
+        need = std::max(need, mfma_tp_workspace_bytes(N, H, L, D, F, k));
     return need;
 }
 

@@ -119,6 +119,12 @@ bool mfma_scan_same_launch(const ScanDesc &x, const ScanDesc &y);
 // Workspace for `nscans` scans of one (D, F) run side by side in one launch.
 int64_t mfma_scan_workspace_bytes(int64_t N, int64_t H, int64_t L, int64_t D, int64_t F,
                                   int nscans);
+// The chain-parallel kernel: all-fp32 scans of one shape whose state has more than 32 and at
+// most 128 rows and columns, widths multiples of 4 (also widths that mfma_scan_supported
+// does not list).  True when mfma_scan would run these scans, side by side, on that kernel;
+// its workspace (part of mfma_scan_workspace_bytes where both apply).
+bool mfma_tp_takes(const ScanDesc *scans, int nscans, int64_t N, int64_t H, int64_t L);
+int64_t mfma_tp_workspace_bytes(int64_t N, int64_t H, int64_t L, int64_t D, int64_t F, int nscans);
 // The fused attention form of a forward scan: a and b go through the feature map
 // elu(x) + 1, rows of b at or beyond key_lengths[n] count as zero, and every output row is
 // divided by (phi(a_l) . sum_{j <= l} phi(b_j) + eps).

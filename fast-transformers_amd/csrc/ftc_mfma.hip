@@ -24,11 +24,19 @@ bool use_wg_kernel(int64_t D, int64_t F, int nscans, int64_t L, bool all_f32) {
     return nscans == 1 && L >= 128 * kChunk && D == 64 && F == 64;
 }
 
-// all-fp32 scans with a 64 x 64 state can run one workgroup per chain with no split of L
-// (ftc_tp_kernel.h)
+// Row widths that the chain-parallel kernel takes (ftc_tp_kernel.h): states of up to 128 x 128,
+// walked in blocks of 64 rows, with one workgroup per block of 64 output columns; widths
+// that are multiples of 4 (a lane's 16 bytes lie wholly inside a row or wholly outside).
+bool tp_widths(int64_t D, int64_t F) {
+    return D > 32 && D <= 128 && F > 32 && F <= 128 && D % 4 == 0 && F % 4 == 0;
+}
+int64_t tp_fblocks(int64_t F) { return (F + 63) / 64; }
+
+// all-fp32 scans can run one workgroup per chain (and block of 64 output columns) with no
+// split of L (ftc_tp_kernel.h).  `units`: chains x scans x column blocks; `wide`: a state
+// other than 64 x 64, for which the kernels that split L are half as fast as for 64 x 64.
 // Returns the number of segments per chain (0: another kernel takes the launch).
-int tp_kernel_segments(const ScanDesc *scans, int nscans, int64_t chains, int64_t L, bool all_f32) {
-    if (!all_f32 || scans[0].a.width != 64 || scans[0].v.width != 64) return 0;
+int tp_kernel_segments(int64_t units, int64_t L, bool wide) {
     // a chain is walked by one workgroup from end to end: beyond 256 chunks the split of L
     // of the other kernels is faster, and its segment sums also keep the rounding of a long
     // running state in check
@@ -37,7 +45,6 @@ int tp_kernel_segments(const ScanDesc *scans, int nscans, int64_t chains, int64_
     // once; with fewer chains than CUs a chain is cut into up to four segments whose
     // workgroups each rebuild the state before their segment by themselves (a state-only
     // chunk costs about a third of a full one), as long as that fills at least half the GPU.
-    const int64_t units = chains * nscans;
     const int64_t total_chunks = (L + kChunk - 1) / kChunk;
     int nseg = (int)std::max<int64_t>(1, std::min<int64_t>(std::min<int64_t>(4, 256 / units), total_chunks));
     if (const char *env = getenv("FTC_TP_SEGS")) nseg = std::max(1, std::min(atoi(env), 16));  // tuning aid
@@ -46,7 +53,13 @@ int tp_kernel_segments(const ScanDesc *scans, int nscans, int64_t chains, int64_
     // L and exchange states; L=3000: 75 against 84; L=4096: 100 against 108; L=8192: 201
     // against 201 -- cut chains pay off while the chunks that a workgroup walks for its
     // state alone are few.
-    if (nseg > 1 && total_chunks > 128) return 0;
+    if (nseg > 1 && total_chunks > 128) {
+        if (!wide) return 0;
+        nseg = 1;
+    }
+    // (wide states: the other kernels run them as column slices that each repeat the chunk
+    // product, and lose at any number of rounds)
+    if (wide) return units * nseg >= 64 ? nseg : 0;
     // Beyond two rounds of workgroups the other kernels win again (1024 chains of 512
     // positions: 128 / 315 us against 135 / 348): there every chain has its own wavefront,
     // all resident at once, and nothing is split either.
@@ -95,15 +108,19 @@ int tp_segment_starts(int64_t chunks, int nseg, int32_t *start) {
 // chain is cut into as many equal segments as fill the GPU (one workgroup each); a workgroup
 // walks its own chunks twice, first for their state alone.  Returns the number of chunks per
 // segment (0: not this way) and the number of segments in *nseg.
-int tp_exchange_segments(int64_t units, int64_t L, int *nseg) {
+int tp_exchange_segments(int64_t units, int64_t L, bool wide, int *nseg) {
     const int64_t total_chunks = (L + kChunk - 1) / kChunk;
     *nseg = 0;
     if (const char *env = getenv("FTC_TPX"))  // tuning aid
         if (atoi(env) == 0) return 0;
     // Up to 64 chunks the cut chains without an exchange are as fast (cfg2: 30 us either way)
     // and need no workspace.
-    if (units < 1 || units > 128 || total_chunks <= 64) return 0;
-    int64_t want = std::min<int64_t>(256 / units, total_chunks / 8);
+    if (units < 1 || (units > 128 && !wide) || total_chunks <= 64) return 0;
+    // (wide states: also with more workgroups than CUs, where chains are too long to walk whole)
+    if (units > 128 && total_chunks <= 256) return 0;
+    int64_t want = 256 / units;
+    if (wide) want = std::max<int64_t>(want, (total_chunks + 255) / 256);
+    want = std::min<int64_t>(want, total_chunks / 8);
     if (const char *env = getenv("FTC_TPX_SEGS")) want = std::max(1, atoi(env));  // tuning aid
     if (want < 2) return 0;
     const int64_t seg_chunks = ((total_chunks + want - 1) / want + kTpAhead - 1) / kTpAhead * kTpAhead;
@@ -117,9 +134,9 @@ int tp_exchange_segments(int64_t units, int64_t L, int *nseg) {
 }
 
 // workspace of the exchange: control block, then two state slots (own sum, group total) of
-// 64 x 16 floats per consumer, four consumers per segment
-int64_t tp_exchange_workspace_bytes(int64_t units, int nseg) {
-    return kControlBytes + 2 * 4 * units * nseg * (int64_t)(64 * 16 * 4);
+// D x 16 floats (D rounded up to whole blocks of 64 rows) per consumer, four consumers per segment
+int64_t tp_exchange_workspace_bytes(int64_t units, int nseg, int64_t D) {
+    return kControlBytes + 2 * 4 * units * nseg * (int64_t)((D + 63) / 64 * 64 * 16 * 4);
 }
 
 // `wg`: the plan is for workgroups of F / 32 wavefronts (each has its own flag words);
@@ -255,12 +272,43 @@ int64_t mfma_scan_workspace_bytes(int64_t N, int64_t H, int64_t L, int64_t D, in
     // whichever kernel the element types will select
     int64_t bytes = std::max(make_plan(N, H, L, D, F, nscans, false).workspace_bytes,
                              make_plan(N, H, L, D, F, nscans, true).workspace_bytes);
-    if (D == 64 && F == 64) {
-        int nseg = 0;
-        if (tp_exchange_segments(std::max<int64_t>(1, N * H) * nscans, L, &nseg) > 0)
-            bytes = std::max(bytes, tp_exchange_workspace_bytes(std::max<int64_t>(1, N * H) * nscans, nseg));
+    return std::max(bytes, mfma_tp_workspace_bytes(N, H, L, D, F, nscans));
+}
+
+int64_t mfma_tp_workspace_bytes(int64_t N, int64_t H, int64_t L, int64_t D, int64_t F, int nscans) {
+    if (!tp_widths(D, F)) return 0;
+    const int64_t units = std::max<int64_t>(1, N * H) * nscans * tp_fblocks(F);
+    int nseg = 0;
+    if (tp_exchange_segments(units, L, D != 64 || F != 64, &nseg) > 0)
+        return tp_exchange_workspace_bytes(units, nseg, D);
+    return 0;
+}
+
+bool mfma_tp_takes(const ScanDesc *scans, int nscans, int64_t N, int64_t H, int64_t L) {
+    const int D = scans[0].a.width, F = scans[0].v.width;
+    if (nscans < 1 || nscans > kMaxScans || !tp_widths(D, F)) return false;
+    int64_t widest_stride = 0;
+    for (int i = 0; i < nscans; i++) {
+        const ScanDesc &sd = scans[i];
+        if (combo_of(sd) != kFFFF || sd.a.width != D || sd.v.width != F) return false;
+        if (L > 1 && !(stride_ok(sd.a.stride_l, D) && stride_ok(sd.b.stride_l, D) &&
+                       stride_ok(sd.v.stride_l, F) && stride_ok(sd.out.stride_l, F)))
+            return false;
+        if (!(aligned16(sd.a.ptr, sd.a.stride_n, sd.a.stride_h, sd.a.stride_l, FTC_F32) &&
+              aligned16(sd.b.ptr, sd.b.stride_n, sd.b.stride_h, sd.b.stride_l, FTC_F32) &&
+              aligned16(sd.v.ptr, sd.v.stride_n, sd.v.stride_h, sd.v.stride_l, FTC_F32) &&
+              aligned16(sd.out.ptr, sd.out.stride_n, sd.out.stride_h, sd.out.stride_l, FTC_F32)))
+            return false;
+        widest_stride = std::max(widest_stride, std::max(std::max(sd.a.stride_l, sd.b.stride_l),
+                                                         std::max(sd.v.stride_l, sd.out.stride_l)));
     }
-    return bytes;
+    // the chain-parallel kernel addresses a whole chain through one 32-bit descriptor
+    if ((L + 2 * kChunk) * std::max<int64_t>(widest_stride, std::max(D, F)) * 4 >= 0x7fffffffLL)
+        return false;
+    const bool wide = D != 64 || F != 64;
+    const int64_t units = std::max<int64_t>(1, N * H) * nscans * tp_fblocks(F);
+    int nseg = 0;
+    return tp_exchange_segments(units, L, wide, &nseg) > 0 || tp_kernel_segments(units, L, wide) > 0;
 }
 
 bool fused_attention_supported(const ScanDesc &sd, int64_t L) {
@@ -280,20 +328,18 @@ int mfma_scan(const ScanDesc *scans, int nscans, int64_t N, int64_t H, int64_t L
     const Combo combo = combo_of(scans[0]);
     if (fused && (nscans != 1 || !fused_attention_supported(scans[0], L)))
         return fail(FTC_ERR_UNSUPPORTED, "no fused attention kernel for this shape or layout");
-    // the chain-parallel kernel addresses a whole chain through one 32-bit descriptor
-    int64_t widest_stride = 0;
-    for (int i = 0; i < nscans; i++)
-        widest_stride = std::max(widest_stride,
-                                 std::max(std::max(scans[i].a.stride_l, scans[i].b.stride_l),
-                                          std::max(scans[i].v.stride_l, scans[i].out.stride_l)));
-    const bool chain_fits = (L + 2 * kChunk) * widest_stride * 4 < 0x7fffffffLL;
-    const bool tp_shape = !fused && chain_fits && combo == kFFFF && D == 64 && F == 64;
+    const bool tp_shape = !fused && mfma_tp_takes(scans, nscans, N, H, L);
+    const bool wide = D != 64 || F != 64;
     const int64_t chains = std::max<int64_t>(1, N * H);
+    const int64_t fblocks = tp_shape ? tp_fblocks(F) : 1;
     int tpx_nseg = 0;
-    const int tpx_seg_chunks = tp_shape ? tp_exchange_segments(chains * nscans, L, &tpx_nseg) : 0;
+    const int tpx_seg_chunks =
+        tp_shape ? tp_exchange_segments(chains * nscans * fblocks, L, wide, &tpx_nseg) : 0;
     const int tp_nseg = tp_shape && tpx_seg_chunks == 0
-                            ? tp_kernel_segments(scans, nscans, N * H, L, combo == kFFFF) : 0;
+                            ? tp_kernel_segments(chains * nscans * fblocks, L, wide) : 0;
     const bool tp = tp_nseg > 0 || tpx_seg_chunks > 0;
+    if (!tp && !mfma_scan_supported(scans[0], L))
+        return fail(FTC_ERR_UNSUPPORTED, "no MFMA kernel takes a %d x %d state here", D, F);
     const bool wg = fused || use_wg_kernel(D, F, nscans, L, combo == kFFFF);
     MfmaPlan pl = make_plan(N, H, L, D, F, nscans, wg, fused != nullptr);
     int32_t tp_start[kMaxTpSegments + 1] = {0};
@@ -301,7 +347,7 @@ int mfma_scan(const ScanDesc *scans, int nscans, int64_t N, int64_t H, int64_t L
         pl.nseg = tpx_nseg;
         pl.seg_len = tpx_seg_chunks * kChunk;
         pl.waves = chains * pl.nseg;
-        pl.workspace_bytes = tp_exchange_workspace_bytes(chains * nscans, pl.nseg);
+        pl.workspace_bytes = tp_exchange_workspace_bytes(chains * nscans * fblocks, pl.nseg, D);
     } else if (tp) {  // one workgroup per chain segment, nothing to exchange
         pl.nseg = tp_segment_starts((L + kChunk - 1) / kChunk, tp_nseg, tp_start);
         pl.seg_len = (int)L;
@@ -360,7 +406,8 @@ int mfma_scan(const ScanDesc *scans, int nscans, int64_t N, int64_t H, int64_t L
     args.tp_seg_chunks = tpx_seg_chunks;
     args.nseg = pl.nseg;
     args.waves_per_scan = (int32_t)pl.waves;
-    args.total_waves = (int32_t)(pl.waves * nscans);
+    args.total_waves = (int32_t)(pl.waves * nscans * fblocks);
+    args.tp_d = D, args.tp_f = F, args.tp_fblocks = (int32_t)fblocks;
     // very short chains: one level (every step adds the sums of all steps before it);
     // otherwise groups of about sqrt(nseg) steps, which moves fewer states per step
     args.group = pl.nseg;

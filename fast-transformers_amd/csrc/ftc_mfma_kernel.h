@@ -468,6 +468,9 @@ struct ScanArgs {
     // ... or, with an exchange of segment sums (tp_exchange != 0), nseg segments of
     // tp_seg_chunks chunks (a multiple of kTpAhead), taken in the order of arrival
     int32_t tp_exchange, tp_seg_chunks;
+    // widths of the rows as they lie in memory (a, b: tp_d <= 128; v, out: tp_f <= 128, both
+    // multiples of 4) and the number of 64-column blocks of v and out, one workgroup each
+    int32_t tp_d, tp_f, tp_fblocks;
 };
 
 // Which (scan, chain, L-segment) a wavefront works on.

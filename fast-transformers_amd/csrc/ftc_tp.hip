@@ -5,9 +5,14 @@ namespace ftc {
 namespace mfma {
 
 void launch_scan_tp(void *ws, const ScanArgs &args, hipStream_t stream) {
-    // args.waves_per_scan counts chains, args.total_waves chains of all scans of the launch
-    hipLaunchKernelGGL(scan_tp_kernel, dim3((unsigned)args.total_waves), dim3(512), 0, stream,
-                       (uint32_t *)ws, args);
+    // args.waves_per_scan counts the workgroups of one block of 64 output columns of one scan,
+    // args.total_waves those of all blocks of all scans of the launch
+    if (args.tp_d <= 64)
+        hipLaunchKernelGGL(scan_tp_kernel<1>, dim3((unsigned)args.total_waves), dim3(512), 0, stream,
+                           (uint32_t *)ws, args);
+    else
+        hipLaunchKernelGGL(scan_tp_kernel<2>, dim3((unsigned)args.total_waves), dim3(512), 0, stream,
+                           (uint32_t *)ws, args);
 }
 
 }  // namespace mfma

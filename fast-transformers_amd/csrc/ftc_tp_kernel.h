@@ -92,8 +92,9 @@ __device__ __forceinline__ constexpr int b_tile_column(int d) {
     return 32 * (d / 32) + 16 * ((d / 4) % 2) + 4 * ((d % 32) / 8) + d % 4;
 }
 
+template <int ND>
 __global__ __launch_bounds__(512, 2) void scan_tp_kernel(uint32_t *__restrict__ ws_ptr, ScanArgs p) {
-    constexpr int D = 64, F = 64;
+    constexpr int D = 64, F = 64;              // one block of state rows and of output columns
     constexpr int T = 256;                     // producer lanes
     constexpr int PF = kTpAhead;               // chunks requested ahead
     constexpr int RBA = D * 2, RBV = F * 2;    // bytes per row of a bf16 piece tile
@@ -133,7 +134,12 @@ __global__ __launch_bounds__(512, 2) void scan_tp_kernel(uint32_t *__restrict__ 
         which = t / (chains - full);
         chain = full + t % (chains - full);
     }
-    const uint32_t scan_id = which / nseg;
+    // (a scan with more than 64 output columns counts as two, one per block of columns)
+    const uint32_t virt = which / nseg;
+    const uint32_t scan_id = virt / (uint32_t)p.tp_fblocks;
+    const int fb = (int)(virt % (uint32_t)p.tp_fblocks);
+    const int Dw = p.tp_d;                      // state rows in all: a and b are this wide
+    const int fw = min(F, p.tp_f - F * fb);     // output columns of this block
     const ScanOperands &op = p.scan[scan_id];
     const bool REV = op.rev != 0;
     const int n = (int)(chain / (uint32_t)p.H), h = (int)(chain % (uint32_t)p.H);
@@ -151,7 +157,7 @@ __global__ __launch_bounds__(512, 2) void scan_tp_kernel(uint32_t *__restrict__ 
     const bool exchange = p.tp_exchange != 0 && nseg > 1;
     gu32 *const hdr = (gu32 *)ws_ptr;
     gu32 *const flags = hdr + kHdrWords;
-    const uint32_t chain_id = scan_id * chains + chain;  // over all scans of the launch
+    const uint32_t chain_id = virt * chains + chain;  // over all scans of the launch
     int seg = (int)(which % nseg);
     __shared__ uint32_t order_sh;
     if (exchange) {
@@ -171,12 +177,16 @@ __global__ __launch_bounds__(512, 2) void scan_tp_kernel(uint32_t *__restrict__ 
     // the chunks walked for their state alone: so0 .. so0 + n1 - 1 (n1 a multiple of PF; the
     // last segment of an exchange has no reader for its sum)
     const int so0 = exchange ? c0 : 0;
-    const int n1 = exchange ? (seg + 1 < (int)nseg ? nchunks - c0 : 0) : c0;
-    // position v of the walk: v < n1: a chunk walked for its state alone; then chunk
-    // c0 + v - n1.  With an exchange the first pass runs against the direction of the second,
-    // so that the second starts with the rows that the caches saw last.
-    const int nwalk = n1 + nchunks - c0;  // (position nwalk: a chunk of zeros)
-    auto so_chunk = [&](int v) -> int { return exchange ? so0 + n1 - 1 - v : so0 + v; };
+    const int n1c = exchange ? (seg + 1 < (int)nseg ? nchunks - c0 : 0) : c0;
+    // A chunk is walked as ND positions, one per block of 64 state rows (columns of a and
+    // b): position v has block v % ND.  v < n1: a chunk walked for its state alone; then
+    // chunk c0 + (v - n1) / ND.  With an exchange the first pass runs against the direction
+    // of the second, so that the second starts with the rows that the caches saw last.
+    const int n1 = ND * n1c;
+    const int nwalk = n1 + ND * (nchunks - c0);  // (position nwalk: a chunk of zeros)
+    auto so_chunk = [&](int v) -> int { return exchange ? so0 + n1c - 1 - v / ND : so0 + v / ND; };
+    auto walk_chunk = [&](int v) -> int { return v < n1 ? so_chunk(v) : c0 + (v - n1) / ND; };
+    constexpr uint32_t kNoRow = 0x80000000u;  // an offset outside every descriptor
     auto chunk_row0 = [&](int c) -> int { return REV ? rows - kChunk * (c + 1) : kChunk * c; };
     __syncthreads();
 #ifdef FTC_TIMELINE
@@ -196,13 +206,21 @@ __global__ __launch_bounds__(512, 2) void scan_tp_kernel(uint32_t *__restrict__ 
                        v_slb = (uint32_t)op.v_sl * 4;
         const char *a_seg = (const char *)op.a + ((int64_t)n * op.a_sn + (int64_t)h * op.a_sh) * 4;
         const char *b_seg = (const char *)op.b + ((int64_t)n * op.b_sn + (int64_t)h * op.b_sh) * 4;
-        const char *v_seg = (const char *)op.v + ((int64_t)n * op.v_sn + (int64_t)h * op.v_sh) * 4;
+        const char *v_seg = (const char *)op.v +
+                            ((int64_t)n * op.v_sn + (int64_t)h * op.v_sh + F * fb) * 4;
         const __amdgpu_buffer_rsrc_t a_rs = __builtin_amdgcn_make_buffer_rsrc(
-            (void *)a_seg, 0, (rows - 1) * a_slb + D * 4, kRsrcFlags);
+            (void *)a_seg, 0, (rows - 1) * a_slb + Dw * 4, kRsrcFlags);
         const __amdgpu_buffer_rsrc_t b_rs = __builtin_amdgcn_make_buffer_rsrc(
-            (void *)b_seg, 0, (rows - 1) * b_slb + D * 4, kRsrcFlags);
+            (void *)b_seg, 0, (rows - 1) * b_slb + Dw * 4, kRsrcFlags);
         const __amdgpu_buffer_rsrc_t v_rs = __builtin_amdgcn_make_buffer_rsrc(
-            (void *)v_seg, 0, (rows - 1) * v_slb + F * 4, kRsrcFlags);
+            (void *)v_seg, 0, (rows - 1) * v_slb + fw * 4, kRsrcFlags);
+        // Widths that do not fill their last block of 64: a lane whose four columns lie
+        // beyond the width asks outside the descriptor and cuts zeros (widths are multiples
+        // of 4).  A lane has the same columns in both of its quads.
+        bool ab_in[ND];
+#pragma unroll
+        for (int hb = 0; hb < ND; hb++) ab_in[hb] = 4 * (ptid % QA) + D * hb < Dw;
+        const bool v_in = 4 * (ptid % QV) < fw;
         uint32_t a_goff[LA], b_goff[LA], v_goff[LV];
         int a_waddr[LA], b_waddr[LA], v_waddr[LV];
 #pragma unroll
@@ -230,21 +248,22 @@ __global__ __launch_bounds__(512, 2) void scan_tp_kernel(uint32_t *__restrict__ 
         // chunk the compiler can wait for the oldest ones only (s_waitcnt vmcnt(n) with n the
         // number of younger requests) instead of for all.
         static_assert(LA == 2 && LV == 2, "quad 0 of a lane: rows 0 .. 15, quad 1: rows 16 .. 31");
-        auto fetch = [&](Raw &r, int v) {  // v: position of the walk
-            const int c = v < n1 ? so_chunk(v) : c0 + v - n1;
-            const int row0 = v < nwalk ? chunk_row0(c) : -2 * kChunk;
+        auto fetch = [&](Raw &r, int v, int hb) {  // v: position of the walk, hb = v % ND
+            const int row0 = v < nwalk ? chunk_row0(walk_chunk(v)) : -2 * kChunk;
             const int row0_x = v >= n1 ? row0 : -2 * kChunk;
+            const uint32_t col = (uint32_t)(D * 4 * hb);
 #pragma unroll
             for (int q = 0; q < LA; q++) {
                 r.a[q] = __builtin_amdgcn_raw_buffer_load_b128(
-                    a_rs, a_goff[q] + (uint32_t)row0_x * a_slb, 0, 0);
+                    a_rs, ab_in[hb] ? a_goff[q] + col + (uint32_t)row0_x * a_slb : kNoRow, 0, 0);
                 r.b[q] = __builtin_amdgcn_raw_buffer_load_b128(
-                    b_rs, b_goff[q] + (uint32_t)(q == 0 ? row0 : row0_x) * b_slb, 0, 0);
+                    b_rs, ab_in[hb] ? b_goff[q] + col + (uint32_t)(q == 0 ? row0 : row0_x) * b_slb
+                                    : kNoRow, 0, 0);
             }
 #pragma unroll
             for (int q = 0; q < LV; q++)
                 r.v[q] = __builtin_amdgcn_raw_buffer_load_b128(
-                    v_rs, v_goff[q] + (uint32_t)(q == 0 ? row0 : row0_x) * v_slb, 0, 0);
+                    v_rs, v_in ? v_goff[q] + (uint32_t)(q == 0 ? row0 : row0_x) * v_slb : kNoRow, 0, 0);
         };
         // position k of the walk goes to LDS buffer k % 3 through register set k % PF.  The
         // first n1 positions (a multiple of PF) only feed the state: no piece of a, and the
@@ -264,7 +283,7 @@ __global__ __launch_bounds__(512, 2) void scan_tp_kernel(uint32_t *__restrict__ 
             if (!own) asm volatile("" ::"v"(r.a[0]), "v"(r.a[1]), "v"(r.b[1]), "v"(r.v[1]));
         };
 #pragma unroll
-        for (int j = 0; j < PF; j++) fetch(raw[j], j);
+        for (int j = 0; j < PF; j++) fetch(raw[j], j, j % ND);
         // Barrier number k (k = 0: before the first position; k >= 1: in the middle of
         // position k - 1) finds position k cut.  The last one finds a chunk of zeros.
         // Two loops whose bodies are straight-line code, so that the waits inside them count
@@ -274,7 +293,7 @@ __global__ __launch_bounds__(512, 2) void scan_tp_kernel(uint32_t *__restrict__ 
 #pragma unroll
             for (int j = 0; j < PF; j++) {
                 cut(raw[j], buf, false);
-                fetch(raw[j], v + j + PF);
+                fetch(raw[j], v + j + PF, j % ND);
                 buf = buf == 2 ? 0 : buf + 1;
                 wg_barrier();
                 __builtin_amdgcn_sched_barrier(0);  // one chunk at a time, in this order
@@ -289,7 +308,7 @@ __global__ __launch_bounds__(512, 2) void scan_tp_kernel(uint32_t *__restrict__ 
                 if (v + j == n1 + 4) FTC_STAMP(0);
                 cut(raw[j], buf, true);
                 if (v + j == n1 + 4) FTC_STAMP(1);
-                fetch(raw[j], v + j + PF);
+                fetch(raw[j], v + j + PF, j % ND);
                 buf = buf == 2 ? 0 : buf + 1;
                 if (v + j == n1 + 4) FTC_STAMP(2);
                 wg_barrier();
@@ -311,9 +330,9 @@ __global__ __launch_bounds__(512, 2) void scan_tp_kernel(uint32_t *__restrict__ 
     // =========================== consumers ===========================
     const int ln = lane & 15, g = lane >> 4;
     const uint32_t o_slb = (uint32_t)op.o_sl * 4;
-    char *o_seg = (char *)op.out + ((int64_t)n * op.o_sn + (int64_t)h * op.o_sh) * 4;
+    char *o_seg = (char *)op.out + ((int64_t)n * op.o_sn + (int64_t)h * op.o_sh + F * fb) * 4;
     const __amdgpu_buffer_rsrc_t o_rs =
-        __builtin_amdgcn_make_buffer_rsrc((void *)o_seg, 0, (rows - 1) * o_slb + F * 4, kRsrcFlags);
+        __builtin_amdgcn_make_buffer_rsrc((void *)o_seg, 0, (rows - 1) * o_slb + fw * 4, kRsrcFlags);
     // Pt quadrant of this wavefront: the two on the diagonal, the one inside the mask, and
     // (consumer 3, so that all four run the same instructions) the one outside it: zeros
     const int jh = w == 0 ? 0 : w == 1 ? 1 : ((w == 2) == REV ? 1 : 0);
@@ -368,19 +387,35 @@ __global__ __launch_bounds__(512, 2) void scan_tp_kernel(uint32_t *__restrict__ 
 #pragma unroll
     for (int x = 0; x < 2; x++)
         o_lane[x] = (uint32_t)(16 * (x ^ ih) + ln) * o_slb + 4u * (16 * w + 4 * g);
+    const bool o_in = 16 * w + 4 * g < fw;  // (columns beyond the width are not stored)
 
-    f32x4 S[4];
+    f32x4 S[ND][4];  // the slab's rows, block by block
 #pragma unroll
-    for (int dt = 0; dt < 4; dt++) S[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int hb = 0; hb < ND; hb++)
+#pragma unroll
+        for (int dt = 0; dt < 4; dt++) S[hb][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
     constexpr int kPa[6] = {0, 1, 2, 0, 1, 0}, kPb[6] = {2, 1, 0, 1, 0, 0};  // piece products
     // the caller's state: lane (f = 16 w + ln, g), tile dt, register r <-> row d below
     auto state_row = [&](int dt, int r) -> int { return 32 * (dt / 2) + 8 * g + 4 * (dt % 2) + r; };
+    const bool st_in = 16 * w + ln < fw;
     auto add_caller_state = [&]() {
-        const float *base = op.s0 + (int64_t)n * op.s0_sn + (int64_t)h * op.s0_sh + 16 * w + ln;
+        const float *base =
+            op.s0 + (int64_t)n * op.s0_sn + (int64_t)h * op.s0_sh + F * fb + 16 * w + ln;
 #pragma unroll
-        for (int dt = 0; dt < 4; dt++)
+        for (int hb = 0; hb < ND; hb++)
 #pragma unroll
-            for (int r = 0; r < 4; r++) S[dt][r] += base[(int64_t)state_row(dt, r) * op.s0_sd];
+            for (int dt = 0; dt < 4; dt++) {
+                // (rows and columns beyond the widths: nothing is read, zero is added)
+                float x[4];
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    const int d = D * hb + state_row(dt, r);
+                    const bool in = st_in && d < Dw;
+                    x[r] = *(in ? base + (int64_t)d * op.s0_sd : op.s0);
+                    x[r] = in ? x[r] : 0.f;
+                }
+                S[hb][dt] += f32x4{x[0], x[1], x[2], x[3]};
+            }
     };
     // (with an exchange the sums that travel are those of the rows alone; every segment adds
     // the caller's state on top of what it gathers)
@@ -421,11 +456,16 @@ __global__ __launch_bounds__(512, 2) void scan_tp_kernel(uint32_t *__restrict__ 
         const int cid = w * 64 + lane, crow = (T + cid) / QA, cc4 = (T + cid) % QA;
         const uint32_t b_slb = (uint32_t)op.b_sl * 4, v_slb = (uint32_t)op.v_sl * 4;
         const char *b_seg = (const char *)op.b + ((int64_t)n * op.b_sn + (int64_t)h * op.b_sh) * 4;
-        const char *v_seg = (const char *)op.v + ((int64_t)n * op.v_sn + (int64_t)h * op.v_sh) * 4;
+        const char *v_seg = (const char *)op.v +
+                            ((int64_t)n * op.v_sn + (int64_t)h * op.v_sh + F * fb) * 4;
         const __amdgpu_buffer_rsrc_t b_rs = __builtin_amdgcn_make_buffer_rsrc(
-            (void *)b_seg, 0, (rows - 1) * b_slb + D * 4, kRsrcFlags);
+            (void *)b_seg, 0, (rows - 1) * b_slb + Dw * 4, kRsrcFlags);
         const __amdgpu_buffer_rsrc_t v_rs = __builtin_amdgcn_make_buffer_rsrc(
-            (void *)v_seg, 0, (rows - 1) * v_slb + F * 4, kRsrcFlags);
+            (void *)v_seg, 0, (rows - 1) * v_slb + fw * 4, kRsrcFlags);
+        bool b_in[ND];
+#pragma unroll
+        for (int hb = 0; hb < ND; hb++) b_in[hb] = 4 * cc4 + D * hb < Dw;
+        const bool v_in = 4 * cc4 < fw;
         const uint32_t b_goff = (uint32_t)crow * b_slb + 16u * cc4,
                        v_goff = (uint32_t)crow * v_slb + 16u * cc4;
         const int b_waddr = TpSwizzle<RBA>::addr(crow, 2 * b_tile_column(4 * cc4)),
@@ -436,10 +476,12 @@ __global__ __launch_bounds__(512, 2) void scan_tp_kernel(uint32_t *__restrict__ 
         RawC rawc[PF];
         // (every request every time, as the producers do: from position n1 on outside the
         // descriptor)
-        auto cfetch = [&](RawC &r, int v) {
+        auto cfetch = [&](RawC &r, int v, int hb) {  // hb = v % ND
             const int row0 = v < n1 ? chunk_row0(so_chunk(v)) : -2 * kChunk;
-            r.b = __builtin_amdgcn_raw_buffer_load_b128(b_rs, b_goff + (uint32_t)row0 * b_slb, 0, 0);
-            r.v = __builtin_amdgcn_raw_buffer_load_b128(v_rs, v_goff + (uint32_t)row0 * v_slb, 0, 0);
+            r.b = __builtin_amdgcn_raw_buffer_load_b128(
+                b_rs, b_in[hb] ? b_goff + (uint32_t)(D * 4 * hb) + (uint32_t)row0 * b_slb : kNoRow, 0, 0);
+            r.v = __builtin_amdgcn_raw_buffer_load_b128(
+                v_rs, v_in ? v_goff + (uint32_t)row0 * v_slb : kNoRow, 0, 0);
         };
         auto ccut_b = [&](const RawC &r, int bufk) {
             split_quad_to_lds(r.b, unit_pc + bufk * kBufBytes + kOffB, kTileA, b_waddr);
@@ -448,10 +490,10 @@ __global__ __launch_bounds__(512, 2) void scan_tp_kernel(uint32_t *__restrict__ 
             split_quad_to_lds(r.v, unit_pc + bufk * kBufBytes + kOffV, kTileV, v_waddr);
         };
 #pragma unroll
-        for (int j = 0; j < PF; j++) cfetch(rawc[j], j);
+        for (int j = 0; j < PF; j++) cfetch(rawc[j], j, j % ND);
         ccut_b(rawc[0], 0);
         ccut_v(rawc[0], 0);
-        cfetch(rawc[0], PF);
+        cfetch(rawc[0], PF, 0);
         wg_barrier();
         FTC_STAMP(13);  // first chunk cut
         Frag bt2[4][3] = {}, vf2[3] = {};  // (the first round multiplies zeros)
@@ -464,30 +506,31 @@ __global__ __launch_bounds__(512, 2) void scan_tp_kernel(uint32_t *__restrict__ 
                 // c + j - 1 (position n1 is all the producers')
                 const bool cut_next = j < PF - 1 || c + PF < n1;
                 const RawC &rn = rawc[(j + 1) % PF];
+                const int hp = (j + ND - 1) % ND;  // block of the position before
 #pragma unroll
                 for (int i = 0; i < 24; i++) {
                     if (j % 2 == 0) {
-                        S[i % 4] = mfma16(bt2[i % 4][kPa[i / 4]], vf2[kPb[i / 4]], S[i % 4]);
+                        S[hp][i % 4] = mfma16(bt2[i % 4][kPa[i / 4]], vf2[kPb[i / 4]], S[hp][i % 4]);
                         if (i < 15) tr_frag_into(bt, vf, pc, i);
                     } else {
-                        S[i % 4] = mfma16(bt[i % 4][kPa[i / 4]], vf[kPb[i / 4]], S[i % 4]);
+                        S[hp][i % 4] = mfma16(bt[i % 4][kPa[i / 4]], vf[kPb[i / 4]], S[hp][i % 4]);
                         if (i < 15) tr_frag_into(bt2, vf2, pc, i);
                     }
                     if (i == 15 && cut_next) ccut_b(rn, bufn);
                     if (i == 19 && cut_next) ccut_v(rn, bufn);
                     __builtin_amdgcn_sched_barrier(0);
                 }
-                cfetch(rawc[(j + 1) % PF], c + j + 1 + PF);
+                cfetch(rawc[(j + 1) % PF], c + j + 1 + PF, (j + 1) % ND);
                 buf = bufn;
                 bufn = next_buf(bufn);
                 wg_barrier();
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
-        // the last of these chunks (n1 is even: its fragments are in the second set)
+        // the last of these positions (n1 is even: its fragments are in the second set)
 #pragma unroll
         for (int i = 0; i < 24; i++) {
-            S[i % 4] = mfma16(bt2[i % 4][kPa[i / 4]], vf2[kPb[i / 4]], S[i % 4]);
+            S[ND - 1][i % 4] = mfma16(bt2[i % 4][kPa[i / 4]], vf2[kPb[i / 4]], S[ND - 1][i % 4]);
             if (i < 18) rm_frag(unit_pc + buf * kBufBytes, i);  // our own first chunk is cut
             __builtin_amdgcn_sched_barrier(0);
         }
@@ -503,36 +546,40 @@ __global__ __launch_bounds__(512, 2) void scan_tp_kernel(uint32_t *__restrict__ 
         gfloat *const sums = (gfloat *)(hdr + kControlBytes / 4);
         // the flag words and state slots of consumer w of the segment with ticket t are those
         // of "ticket" w * total_units + t (as in ftc_wg_kernel.h)
-        StateExchange<1, 1> xch(flags, sums, 4u * total_units,
+        StateExchange<ND, 1> xch(flags, sums, 4u * total_units,
                                 (uint32_t)w * total_units + chain_id * nseg + (uint32_t)seg, seg,
                                 (int)nseg, p.group, lane);
-        f32x16 Sx[1][1], X[1][1];
+        f32x16 Sx[ND][1], X[ND][1];
 #pragma unroll
-        for (int dt = 0; dt < 4; dt++)
+        for (int hb = 0; hb < ND; hb++)
 #pragma unroll
-            for (int r = 0; r < 4; r++) Sx[0][0][4 * dt + r] = S[dt][r];
+            for (int dt = 0; dt < 4; dt++)
+#pragma unroll
+                for (int r = 0; r < 4; r++) Sx[hb][0][4 * dt + r] = S[hb][dt][r];
         if (n1 > 0) xch.publish_sum(Sx);
         xch.gather(Sx, X);
         if (xch.failed && lane == 0)
             __hip_atomic_store(hdr + kHdrError, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 #pragma unroll
-        for (int dt = 0; dt < 4; dt++)
+        for (int hb = 0; hb < ND; hb++)
 #pragma unroll
-            for (int r = 0; r < 4; r++) S[dt][r] = X[0][0][4 * dt + r];
+            for (int dt = 0; dt < 4; dt++)
+#pragma unroll
+                for (int r = 0; r < 4; r++) S[hb][dt][r] = X[hb][0][4 * dt + r];
         if (op.s0) add_caller_state();
     }
     // S_w as pieces in A operand order (slots 0..3 from tile 2 ks, 4..7 from tile 2 ks + 1).
     // Tiles 0 and 1 are final after phase 3 and are cut under phase 4, tiles 2 and 3 after
     // phase 4 and are cut under phase 1 of the next chunk.
     Frag sf[2][3];
-    auto cut_s = [&](int ks, int q) {
+    auto cut_s = [&](int hb, int ks, int q) {
         uint32_t o[3];
-        split_pair_under_mfma(S[2 * ks + q / 2][2 * (q % 2)], S[2 * ks + q / 2][2 * (q % 2) + 1], o);
+        split_pair_under_mfma(S[hb][2 * ks + q / 2][2 * (q % 2)], S[hb][2 * ks + q / 2][2 * (q % 2) + 1], o);
 #pragma unroll
         for (int k = 0; k < 3; k++) sf[ks][k].w[q] = o[k];
     };
 #pragma unroll
-    for (int q = 0; q < 4; q++) cut_s(0, q);
+    for (int q = 0; q < 4; q++) cut_s(0, 0, q);
 
     // A matrix instruction that accumulates into the result of the one before it waits for
     // that result (about twice the issue interval of independent ones), so every phase
@@ -547,110 +594,119 @@ __global__ __launch_bounds__(512, 2) void scan_tp_kernel(uint32_t *__restrict__ 
     // lane (i = 16 (x ^ ih) + ln, g) holds f = 16 w + 4 g + 0..3
     auto store_rows = [&](int x) {
         const f32x4 o = O4[x][0] + O4[x][1];
-        buffer_store4(o_rs, o_off + o_lane[x], o[0], o[1], o[2], o[3]);
+        buffer_store4(o_rs, o_in ? o_off + o_lane[x] : kNoRow, o[0], o[1], o[2], o[3]);
     };
     for (int c = c0; c < nchunks; c++) {
-        const lds_char *pc = unit_pc + buf * kBufBytes;
-        lds_char *const ptc = pt_pc + (c & 1) * (3 * kTileP);
-        Frag pf[2][3];
-        f32x4 P4[4];
-        const f32x4 zero = {0.f, 0.f, 0.f, 0.f};  // (the first product of a sum adds to a constant)
-        if (c == c0 + 4) FTC_STAMP(0);
-        __builtin_amdgcn_sched_barrier(0);
-        // phase 1: (1) the quadrant; underneath: tiles 2, 3 of S_w cut into pieces, the
-        // first position-major reads, and the rows of the chunk before go out (their last
-        // matrix instructions have long finished by now; at the end of their own chunk the
-        // wavefront would wait for them)
 #pragma unroll
-        for (int i = 0; i < 12; i++) {
-            const int ks = i % 2, m = i / 2;
-            P4[i % 4] = mfma16(bfr[ks][kPa[m]], af[0][ks][kPb[m]], i < 4 ? zero : P4[i % 4]);
-            if (i < 4) cut_s(1, i);
-            tr_frag(pc, i);
-            if (i == 5 || i == 7) store_rows(i == 5 ? 0 : 1);
+        for (int hb = 0; hb < ND; hb++) {  // block hb of the state rows
+            const lds_char *pc = unit_pc + buf * kBufBytes;
+            lds_char *const ptc = pt_pc + ((ND * c + hb) & 1) * (3 * kTileP);
+            Frag pf[2][3];
+            f32x4 P4[4];
+            const f32x4 zero = {0.f, 0.f, 0.f, 0.f};  // (the first product of a sum adds to a constant)
+            if (c == c0 + 4) FTC_STAMP(0);
             __builtin_amdgcn_sched_barrier(0);
-        }
-        if (c == c0 + 4) FTC_STAMP(1);
-        // phase 2: first half of (2b) Ot_w = S_w^T a^T; underneath: the last position-major
-        // reads, then the quadrant is added up, masked, cut and handed to the others
-        f32x4 P;
-        uint32_t plo[3], phi[3];
+            // phase 1: (1) the quadrant; underneath: tiles 2, 3 of S_w cut into pieces, the
+            // first position-major reads, and the rows of the chunk before go out (their last
+            // matrix instructions have long finished by now; at the end of their own chunk the
+            // wavefront would wait for them)
 #pragma unroll
-        for (int i = 0; i < 12; i++) {
-            const int x = i % 2, ks = (i / 2) % 2, m = i / 4;  // piece products 0..2
-            O4[x][ks] = mfma16(sf[ks][kPa[m]], af[x][ks][kPb[m]], i < 4 ? zero : O4[x][ks]);
-            if (i < 3) tr_frag(pc, 12 + i);
-            if (i == 4) P = (P4[0] + P4[1]) + (P4[2] + P4[3]);
-            if (i == 6)
-                split_pair_under_mfma(__uint_as_float(__float_as_uint(P[0]) & keep[0]),
-                                      __uint_as_float(__float_as_uint(P[1]) & keep[1]), plo);
-            if (i == 8)
-                split_pair_under_mfma(__uint_as_float(__float_as_uint(P[2]) & keep[2]),
-                                      __uint_as_float(__float_as_uint(P[3]) & keep[3]), phi);
-            if (i == 10) {
+            for (int i = 0; i < 12; i++) {
+                const int ks = i % 2, m = i / 2;
+                P4[i % 4] = mfma16(bfr[ks][kPa[m]], af[0][ks][kPb[m]], i < 4 ? zero : P4[i % 4]);
+                if (i < 4) cut_s(hb, 1, i);
+                tr_frag(pc, i);
+                if (hb == 0 && (i == 5 || i == 7)) store_rows(i == 5 ? 0 : 1);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            if (c == c0 + 4) FTC_STAMP(1);
+            // phase 2: first half of (2b) Ot_w = S_w^T a^T; underneath: the last position-major
+            // reads, then the quadrant is added up, masked, cut and handed to the others
+            f32x4 P;
+            uint32_t plo[3], phi[3];
 #pragma unroll
-                for (int k = 0; k < 3; k++) {
-                    const u32x2 xk = {plo[k], phi[k]};
-                    *(lds_vec2 *)(ptc + k * kTileP + pt_waddr) = xk;
+            for (int i = 0; i < 12; i++) {
+                const int x = i % 2, ks = (i / 2) % 2, m = i / 4;  // piece products 0..2
+                O4[x][ks] = mfma16(sf[ks][kPa[m]], af[x][ks][kPb[m]], i < 4 && hb == 0 ? zero : O4[x][ks]);
+                if (i < 3) tr_frag(pc, 12 + i);
+                if (i == 4) P = (P4[0] + P4[1]) + (P4[2] + P4[3]);
+                if (i == 6)
+                    split_pair_under_mfma(__uint_as_float(__float_as_uint(P[0]) & keep[0]),
+                                          __uint_as_float(__float_as_uint(P[1]) & keep[1]), plo);
+                if (i == 8)
+                    split_pair_under_mfma(__uint_as_float(__float_as_uint(P[2]) & keep[2]),
+                                          __uint_as_float(__float_as_uint(P[3]) & keep[3]), phi);
+                if (i == 10) {
+#pragma unroll
+                    for (int k = 0; k < 3; k++) {
+                        const u32x2 xk = {plo[k], phi[k]};
+                        *(lds_vec2 *)(ptc + k * kTileP + pt_waddr) = xk;
+                    }
                 }
+                __builtin_amdgcn_sched_barrier(0);
             }
-            __builtin_amdgcn_sched_barrier(0);
-        }
-        if (c == c0 + 4) FTC_STAMP(2);
-        // phase 3: second half of (2b) in turn with (3) S_w += b^T v_w for tiles 0 and 1
+            if (c == c0 + 4) FTC_STAMP(2);
+            // phase 3: second half of (2b) in turn with (3) S_w += b^T v_w for tiles 0 and 1
 #pragma unroll
-        for (int i = 0; i < 12; i++) {
-            const int x = i % 2, ks = (i / 2) % 2, m = 3 + i / 4;  // piece products 3..5
-            O4[x][ks] = mfma16(sf[ks][kPa[m]], af[x][ks][kPb[m]], O4[x][ks]);
-            S[i % 2] = mfma16(bt[i % 2][kPa[i / 2]], vf[kPb[i / 2]], S[i % 2]);
-            __builtin_amdgcn_sched_barrier(0);
-        }
-        if (c == c0 + 4) FTC_STAMP(3);
-        buf = next_buf(buf);
-        wg_barrier();
-        if (c == c0 + 4) FTC_STAMP(4);
-        // All of Pt is in LDS and the next chunk is cut: its row-major fragments are
-        // requested under what follows.
-        // phase 4: (3) for tiles 2 and 3 in turn with (2a) Ot_w += v_w^T Pt; underneath:
-        // tiles 0, 1 of S_w cut into pieces
-        const lds_char *pn = unit_pc + buf * kBufBytes;
-#pragma unroll
-        for (int x = 0; x < 2; x++)
-#pragma unroll
-            for (int k = 0; k < 3; k++) pf[x][k] = lds_frag16(ptc + k * kTileP + pt_raddr[x]);
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            S[2 + i % 2] = mfma16(bt[2 + i % 2][kPa[i / 2]], vf[kPb[i / 2]], S[2 + i % 2]);
-            cut_s(0, i);
-            rm_frag(pn, i);  // (past the last chunk: a buffer of zeros)
-            __builtin_amdgcn_sched_barrier(0);
-        }
-#pragma unroll
-        for (int i = 0; i < 12; i++) {
-            if (i < 8) {
-                const int t = 4 + i;
-                S[2 + t % 2] = mfma16(bt[2 + t % 2][kPa[t / 2]], vf[kPb[t / 2]], S[2 + t % 2]);
+            for (int i = 0; i < 12; i++) {
+                const int x = i % 2, ks = (i / 2) % 2, m = 3 + i / 4;  // piece products 3..5
+                O4[x][ks] = mfma16(sf[ks][kPa[m]], af[x][ks][kPb[m]], O4[x][ks]);
+                S[hb][i % 2] = mfma16(bt[i % 2][kPa[i / 2]], vf[kPb[i / 2]], S[hb][i % 2]);
+                __builtin_amdgcn_sched_barrier(0);
             }
-            const int x = i % 2, m = i / 2;
-            O4[x][m % 2] = mfma16(vf[kPa[m]], pf[x][kPb[m]], O4[x][m % 2]);
-            rm_frag(pn, 4 + i);
-            if (i < 2) rm_frag(pn, 16 + i);
+            if (c == c0 + 4) FTC_STAMP(3);
+            buf = next_buf(buf);
+            wg_barrier();
+            if (c == c0 + 4) FTC_STAMP(4);
+            // All of Pt is in LDS and the next chunk is cut: its row-major fragments are
+            // requested under what follows.
+            // phase 4: (3) for tiles 2 and 3 in turn with (2a) Ot_w += v_w^T Pt; underneath:
+            // tiles 0, 1 of S_w cut into pieces
+            const lds_char *pn = unit_pc + buf * kBufBytes;
+#pragma unroll
+            for (int x = 0; x < 2; x++)
+#pragma unroll
+                for (int k = 0; k < 3; k++) pf[x][k] = lds_frag16(ptc + k * kTileP + pt_raddr[x]);
             __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                S[hb][2 + i % 2] = mfma16(bt[2 + i % 2][kPa[i / 2]], vf[kPb[i / 2]], S[hb][2 + i % 2]);
+                cut_s((hb + 1) % ND, 0, i);
+                rm_frag(pn, i);  // (past the last chunk: a buffer of zeros)
+                __builtin_amdgcn_sched_barrier(0);
+            }
+#pragma unroll
+            for (int i = 0; i < 12; i++) {
+                if (i < 8) {
+                    const int t = 4 + i;
+                    S[hb][2 + t % 2] = mfma16(bt[2 + t % 2][kPa[t / 2]], vf[kPb[t / 2]], S[hb][2 + t % 2]);
+                }
+                const int x = i % 2, m = i / 2;
+                O4[x][m % 2] = mfma16(vf[kPa[m]], pf[x][kPb[m]], O4[x][m % 2]);
+                rm_frag(pn, 4 + i);
+                if (i < 2) rm_frag(pn, 16 + i);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            if (c == c0 + 4) FTC_STAMP(5);
+            o_off = (uint32_t)chunk_row0(c) * o_slb;
+            if (c == c0 + 4) FTC_STAMP(6);
         }
-        if (c == c0 + 4) FTC_STAMP(5);
-        o_off = (uint32_t)chunk_row0(c) * o_slb;
-        if (c == c0 + 4) FTC_STAMP(6);
     }
     store_rows(0);
     store_rows(1);
     FTC_STAMP(15);  // last rows on their way
     if (op.s_out && seg == (int)nseg - 1) {
-        float *base = op.s_out + (int64_t)n * op.so_sn + (int64_t)h * op.so_sh + 16 * w + ln;
+        float *base =
+            op.s_out + (int64_t)n * op.so_sn + (int64_t)h * op.so_sh + F * fb + 16 * w + ln;
 #pragma unroll
-        for (int dt = 0; dt < 4; dt++)
+        for (int hb = 0; hb < ND; hb++)
 #pragma unroll
-            for (int r = 0; r < 4; r++) base[(int64_t)state_row(dt, r) * op.so_sd] = S[dt][r];
+            for (int dt = 0; dt < 4; dt++)
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    const int d = D * hb + state_row(dt, r);
+                    if (st_in && d < Dw) base[(int64_t)d * op.so_sd] = S[hb][dt][r];
+                }
     }
     // the last consumer of the launch leaves the control block zeroed (as in ftc_wg_kernel.h)
     if (exchange) {

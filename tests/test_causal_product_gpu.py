@@ -494,6 +494,10 @@ STATE_SHAPES = {
     "many_chains": (40, 32, 64, 64, 64, 52, torch.float32),
     # long chains: workgroups of the chain-parallel kernel exchange segment sums
     "long_e64_m64": (1, 4, 5000, 64, 64, 59, torch.float32),
+    # the chain-parallel kernel on wider states: rows and columns beyond the widths are
+    # neither read nor written
+    "tp_e100_m72": (8, 8, 700, 100, 72, 60, torch.float32),
+    "tp_long_e128_m128": (1, 8, 5000, 128, 128, 61, torch.float32),
     "e32_m128": (2, 3, 700, 32, 128, 53, torch.float32),
     # register-fed kernel, column slices
     "e128_m128": (1, 3, 500, 128, 128, 54, torch.float32),
@@ -674,20 +678,24 @@ def test_dirty_control_block_is_reported_and_healed(cp):
 
 
 TP_SHAPES = [
-    # N, H, L: enough chains for one workgroup per chain (and scan), or few enough that a
-    # chain is cut into segments whose workgroups rebuild their starting state
-    (16, 8, 1), (16, 8, 31), (20, 8, 33), (3, 16, 1000), (40, 4, 97), (2, 32, 2048), (9, 7, 640),
+    # N, H, L, E, M: enough chains for one workgroup per chain (and scan), or few enough that
+    # a chain is cut into segments whose workgroups rebuild their starting state
+    (16, 8, 1, 64, 64), (16, 8, 31, 64, 64), (20, 8, 33, 64, 64), (3, 16, 1000, 64, 64),
+    (40, 4, 97, 64, 64), (2, 32, 2048, 64, 64), (9, 7, 640, 64, 64),
+    # states of more than 64 rows (walked in two blocks) or columns (a workgroup per block of
+    # 64), widths that leave the last block partly empty
+    (10, 8, 1000, 128, 128), (8, 8, 333, 96, 96), (16, 4, 97, 100, 100), (4, 4, 640, 48, 80),
+    (2, 32, 33, 68, 36), (16, 8, 1, 128, 36), (4, 8, 700, 64, 128),
 ]
 
 
-@pytest.mark.parametrize("shape", TP_SHAPES, ids=lambda s: "n%d_h%d_l%d" % s)
+@pytest.mark.parametrize("shape", TP_SHAPES, ids=lambda s: "n%d_h%d_l%d_e%d_m%d" % s)
 def test_chain_parallel_kernel(cp, shape):
-    """The kernel that walks a chain with one workgroup (64 x 64 states, fp32): whole chains
-    and cut chains, ragged ends, both directions, (N, L, H, X) views, against the CPU checker
-    anchored on float64."""
+    """The kernel that walks a chain with one workgroup (fp32, states of up to 128 x 128,
+    widths multiples of 4): whole chains and cut chains, ragged ends, both directions,
+    (N, L, H, X) views, against the CPU checker anchored on float64."""
     from fast_transformers_amd import _native
-    N, H, L = shape
-    E = M = 64
+    N, H, L, E, M = shape
     Q, K, V, G = oracle.make_inputs(N, H, L, E, M, seed=300 + L)
     nlh = lambda t: t.permute(0, 2, 1, 3).contiguous().cuda().permute(0, 2, 1, 3)  # NLHE storage
     q, k, v, g = (nlh(t) for t in (Q, K, V, G))
@@ -709,21 +717,23 @@ def test_chain_parallel_kernel(cp, shape):
 
 
 TPX_SHAPES = [
-    # N, H, L: long chains on few CUs: segments that exchange their sums (one and two levels
-    # of the sum, ragged last segment, a last segment shorter than the others)
-    (2, 8, 4096), (1, 3, 9000), (3, 5, 2100), (1, 2, 40000),
+    # N, H, L, E, M: long chains on few CUs: segments that exchange their sums (one and two
+    # levels of the sum, ragged last segment, a last segment shorter than the others)
+    (2, 8, 4096, 64, 64), (1, 3, 9000, 64, 64), (3, 5, 2100, 64, 64), (1, 2, 40000, 64, 64),
+    # wider states; the last one has more workgroups than the GPU has CUs (a workgroup only
+    # ever waits for workgroups that started before it)
+    (1, 8, 5000, 128, 128), (2, 4, 9000, 100, 68), (1, 130, 8200, 36, 36),
 ]
 
 
-@pytest.mark.parametrize("shape", TPX_SHAPES, ids=lambda s: "n%d_h%d_l%d" % s)
+@pytest.mark.parametrize("shape", TPX_SHAPES, ids=lambda s: "n%d_h%d_l%d_e%d_m%d" % s)
 def test_chain_parallel_kernel_with_exchange(cp, shape):
     """The same kernel on chains too long to walk twice from the start: every workgroup first
     sums its own segment, the sums travel through the workspace.  Both directions,
     (N, L, H, X) views, against the CPU checker anchored on float64; a second call finds the
     control block as the first one left it."""
     from fast_transformers_amd import _native
-    N, H, L = shape
-    E = M = 64
+    N, H, L, E, M = shape
     Q, K, V, G = oracle.make_inputs(N, H, L, E, M, seed=400 + L)
     nlh = lambda t: t.permute(0, 2, 1, 3).contiguous().cuda().permute(0, 2, 1, 3)  # NLHE storage
     q, k, v, g = (nlh(t) for t in (Q, K, V, G))
@@ -751,7 +761,7 @@ def test_chain_parallel_kernel_with_exchange(cp, shape):
 ODD_SHAPES = [
     # N, H, L, E, M, dtype: widths that the matrix-core kernels do not take as they are
     (2, 4, 2000, 25, 64, torch.float32),     # queries and keys padded, values in place
-    (2, 4, 1100, 100, 100, torch.float32),   # everything padded, 128-row states
+    (2, 4, 1100, 99, 101, torch.float32),    # everything padded, 128-row states
     (3, 3, 1000, 10, 3, torch.float32),      # tiny widths
     (1, 2, 5000, 70, 33, torch.float32),     # 96-row state one way, 64-row state the other
     (2, 4, 1200, 48, 80, torch.bfloat16),    # bf16 rows
@@ -841,18 +851,20 @@ def test_rows_far_apart_leave_the_chain_parallel_kernel(cp):
     del wide
 
 
-def test_chain_parallel_kernel_cut_chains_equal_whole_chains(cp):
+@pytest.mark.parametrize("widths", [(64, 64), (100, 72)], ids=lambda w: "e%d_m%d" % w)
+def test_chain_parallel_kernel_cut_chains_equal_whole_chains(cp, widths):
     """A chain cut into segments starts every segment from the state a single walk reaches,
     computed in the same order: the results are the same bit for bit however it is cut."""
     N, H, L = 6, 8, 1500
-    Q, K, V, G = (t.cuda() for t in oracle.make_inputs(N, H, L, 64, 64, seed=17))
+    E, M = widths
+    Q, K, V, G = (t.cuda() for t in oracle.make_inputs(N, H, L, E, M, seed=17))
     outs = []
     for segs in ("1", "2", "4"):
         os.environ["FTC_TP"], os.environ["FTC_TP_SEGS"] = "1", segs
         try:
-            out = torch.empty(N, H, L, 64, device="cuda")
+            out = torch.empty(N, H, L, M, device="cuda")
             cp.causal_dot_product_hip(Q, K, V, out)
-            grads = [torch.empty(N, H, L, 64, device="cuda") for _ in range(3)]
+            grads = [torch.empty(N, H, L, X, device="cuda") for X in (E, E, M)]
             cp.causal_dot_backward_hip(Q, K, V, G, *grads)
             torch.cuda.synchronize()
             outs.append([out] + grads)

@@ -58,7 +58,8 @@ def test_what_the_chain_parallel_kernel_leaves_to_the_others():
     assert many[0].startswith("scan_dma_kernel")
     # other state sizes and element types
     assert lines((10, 8, 1000, 32), (10, 8, 1000, 32))[0].startswith("scan_dma_kernel")
-    assert lines((10, 8, 1000, 128), (10, 8, 1000, 128))[0].startswith("scan_mfma_kernel")
+    assert lines((10, 8, 1000, 32), (10, 8, 1000, 128))[0].startswith("scan_dma_kernel")
+    assert lines((1, 3, 500, 128), (1, 3, 500, 128))[0].startswith("scan_mfma_kernel")  # few chains
     assert lines((4, 8, 1000, 64), (4, 8, 1000, 64), dtype=_native.FTC_BF16)[0] \
         .startswith("scan_mfma_kernel")
     # odd widths: zero-padded dense copies for the matrix-core kernels when there are enough
@@ -71,9 +72,9 @@ def test_what_the_chain_parallel_kernel_leaves_to_the_others():
     odd = lines((8, 16, 4096, 25), (8, 16, 4096, 64), backward=True)
     assert odd[0].startswith("pad_rows_kernel: 2 operands") and "2 results" in odd[0]
     assert odd[1].startswith("scan_dma_kernel: 2 scans") and "state 64 x 32" in odd[1]
-    wide = lines((8, 16, 4096, 100), (8, 16, 4096, 100), backward=True)
+    wide = lines((8, 16, 4096, 99), (8, 16, 4096, 101), backward=True)
     assert wide[0].startswith("pad_rows_kernel: 4 operands") and "3 results" in wide[0]
-    assert wide[1].startswith("scan_mfma_kernel") and "state 128 x 32" in wide[1]
+    assert wide[1].startswith("scan_tp_kernel: 3 scans") and "state 128 x 128" in wide[1]
     assert lines((2, 2, 40, 10), (2, 2, 40, 3))[0].startswith("generic_scan_kernel")
     assert lines((1, 2, 8192, 200), (1, 2, 8192, 64))[0].startswith("generic_scan_kernel")
     # nothing to do
@@ -103,8 +104,33 @@ def test_cut_chains(chains, L):
     assert N * H * nseg <= 256 and int(field(line, r"(\d+) workgroups")) == N * H * nseg
 
 
+def test_wide_states_on_the_chain_parallel_kernel():
+    """fp32 states of more than 32 and up to 128 rows and columns, widths multiples of 4: two
+    blocks of rows per chunk, a workgroup per block of 64 output columns."""
+    fwd = lines((8, 16, 4096, 128), (8, 16, 4096, 128))
+    assert len(fwd) == 1 and fwd[0].startswith("scan_tp_kernel: 1 scan")
+    assert "state 128 x 128" in fwd[0] and "256 workgroups" in fwd[0] and "workspace 0 bytes" in fwd[0]
+    bwd = lines((8, 16, 4096, 128), (8, 16, 4096, 128), backward=True)
+    assert len(bwd) == 1 and bwd[0].startswith("scan_tp_kernel: 3 scans") and "768 workgroups" in bwd[0]
+    # widths that leave the last block partly empty need no copies
+    odd = lines((8, 16, 4096, 100), (8, 16, 4096, 68), backward=True)
+    assert [l.split(":")[0] for l in odd] == ["scan_tp_kernel", "scan_tp_kernel"]
+    assert "2 scans" in odd[0] and "state 68 x 100" in odd[0] and "state 100 x 68" in odd[1]
+    # one block of columns: as many workgroups as chains
+    assert "256 workgroups" in lines((16, 16, 4000, 128), (16, 16, 4000, 64))[0]
+    # long chains: segment sums are exchanged, also with more workgroups than CUs
+    long = lines((4, 16, 16384, 128), (4, 16, 16384, 128), backward=True)
+    assert long[0].startswith("scan_tp_kernel (exchange): 3 scans") and "2 segments of 8192 rows" in long[0]
+    need = int(field(long[0], r"workspace (\d+) bytes"))
+    assert need == 65536 + 2 * 4 * 768 * 128 * 16 * 4
+    # bf16 rows and widths that are not multiples of 4 go the other ways
+    assert lines((8, 16, 4096, 128), (8, 16, 4096, 128), dtype=_native.FTC_BF16)[0] \
+        .startswith("scan_mfma_kernel")
+    assert lines((8, 16, 4096, 98), (8, 16, 4096, 128))[0].startswith("pad_rows_kernel")
+
+
 SWEEP = [(N, H, L, E, M) for (N, H) in [(1, 1), (1, 16), (2, 8), (10, 8), (64, 16)]
-         for L in [1, 64, 1000, 4096, 20000] for (E, M) in [(64, 64), (32, 128), (96, 64), (25, 70)]]
+         for L in [1, 64, 1000, 4096, 20000] for (E, M) in [(64, 64), (32, 128), (96, 64), (25, 70), (128, 128), (100, 36)]]
 
 
 @pytest.mark.parametrize("backward", [False, True])
