@@ -126,7 +126,9 @@ int ftc_causal_dot_product(const ftc_tensor4 *queries, const ftc_tensor4 *keys,
  * starting a graph capture).  The call itself allocates and frees nothing and enqueues
  * kernels only.  Sizes whose scratch need
  * (ftc_causal_dot_product_workspace_bytes) exceeds the array are refused with
- * FTC_ERR_WORKSPACE.  All calls on one GPU share that GPU's array: two calls whose work
+ * FTC_ERR_WORKSPACE -- except that widths which would otherwise run on zero-padded copies
+ * in the workspace then run without them, on the slower shape-agnostic kernel, if the
+ * array holds what that needs.  All calls on one GPU share that GPU's array: two calls whose work
  * overlaps in time on one GPU (different streams, different threads) race; calls on one
  * stream are safe.
  */
