@@ -160,7 +160,8 @@ int64_t padded_scan_workspace_bytes(int64_t N, int64_t H, int64_t L, int64_t D, 
     if (Dp == 0 || (Dp == D && Fp == F) || rows < kPadMinRows ||
         mfma_slice_widths(Dp, Fp, widths) == 0)
         return 0;
-    return round_up(scan_workspace_bytes(N, H, L, Dp, Fp), 256) +
+    return std::max<int64_t>(round_up(scan_workspace_bytes(N, H, L, Dp, Fp), 256),
+                             FTC_WORKSPACE_CONTROL_BYTES) +
            2 * round_up(rows * Dp * 4, 256) + 2 * round_up(rows * Fp * 4, 256);
 }
 
@@ -221,6 +222,8 @@ int padded_scans(const ScanDesc *scans, int n, const bool *take, int64_t N, int6
                               : copy_of(o.ptr, o.stride_n, o.stride_h, o.stride_l, o.dtype, o.width, Fp, true);
         work[nwork++] = sc;
     }
+    // the copies never lie on the control block, which every call must leave zeroed
+    ws_scan = std::max<int64_t>(ws_scan, FTC_WORKSPACE_CONTROL_BYTES);
     int64_t need = ws_scan;
     for (int i = 0; i < ncopies; i++) need += round_up(rows * copies[i].padded * esz(copies[i].dtype), 256);
     if (!plan_only() && (!workspace || (int64_t)workspace_bytes < need || (uintptr_t)workspace % 256 != 0))
@@ -541,7 +544,8 @@ int64_t ftc_causal_dot_backward_workspace_bytes(int64_t N, int64_t H, int64_t L,
         int64_t ws = 0;
         if (padded_rows(E)) ws = std::max(ws, scan_workspace_bytes(N, H, L, padded_rows(E), round_up(M, 32)));
         if (padded_rows(M)) ws = std::max(ws, scan_workspace_bytes(N, H, L, padded_rows(M), round_up(E, 32)));
-        need = std::max(need, round_up(ws, 256) + 4 * round_up(N * H * L * round_up(E, 32) * 4, 256) +
+        need = std::max(need, std::max<int64_t>(round_up(ws, 256), FTC_WORKSPACE_CONTROL_BYTES) +
+                                  4 * round_up(N * H * L * round_up(E, 32) * 4, 256) +
                                   3 * round_up(N * H * L * round_up(M, 32) * 4, 256));
     }
     return need;

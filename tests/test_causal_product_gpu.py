@@ -766,6 +766,9 @@ ODD_SHAPES = [
     (1, 2, 5000, 70, 33, torch.float32),     # 96-row state one way, 64-row state the other
     (2, 4, 1200, 48, 80, torch.bfloat16),    # bf16 rows
     (1, 4, 2500, 130, 40, torch.float32),    # E beyond 128: dV stays on the generic kernel
+    # many short chains: the scans on the copies need no workspace of their own, and the
+    # copies must still keep off the control block
+    (33, 12, 64, 48, 33, torch.float32),
 ]
 
 
