@@ -32,11 +32,18 @@ bool tp_widths(int64_t D, int64_t F) {
 }
 int64_t tp_fblocks(int64_t F) { return (F + 63) / 64; }
 
+// whether the kernels that split L take fp32 rows of these widths (as column slices, if need be)
+bool mfma_scan_supported_widths(int64_t D, int64_t F) {
+    int widths[kMfmaMaxSlices];
+    return mfma_slice_widths(D, F, widths) > 0;
+}
+
 // all-fp32 scans can run one workgroup per chain (and block of 64 output columns) with no
 // split of L (ftc_tp_kernel.h).  `units`: chains x scans x column blocks; `wide`: a state
-// other than 64 x 64, for which the kernels that split L are half as fast as for 64 x 64.
+// other than 64 x 64, for which the kernels that split L are half as fast as for 64 x 64;
+// `others`: one of those kernels takes this shape (else the choice is the VALU kernel).
 // Returns the number of segments per chain (0: another kernel takes the launch).
-int tp_kernel_segments(int64_t units, int64_t L, bool wide) {
+int tp_kernel_segments(int64_t units, int64_t L, bool wide, bool others) {
     // a chain is walked by one workgroup from end to end: beyond 256 chunks the split of L
     // of the other kernels is faster, and its segment sums also keep the rounding of a long
     // running state in check
@@ -58,8 +65,9 @@ int tp_kernel_segments(int64_t units, int64_t L, bool wide) {
         nseg = 1;
     }
     // (wide states: the other kernels run them as column slices that each repeat the chunk
-    // product, and lose at any number of rounds)
-    if (wide) return units * nseg >= 64 ? nseg : 0;
+    // product, and lose at any number of rounds; on a quarter of the CUs they still win, N=1,
+    // H=8, L=2048, 128 x 128 forward: 52 against 91 us.  The VALU kernel loses always.)
+    if (wide) return !others || units * nseg >= 128 ? nseg : 0;
     // Beyond two rounds of workgroups the other kernels win again (1024 chains of 512
     // positions: 128 / 315 us against 135 / 348): there every chain has its own wavefront,
     // all resident at once, and nothing is split either.
@@ -119,7 +127,18 @@ int tp_exchange_segments(int64_t units, int64_t L, bool wide, int *nseg) {
     // (wide states: also with more workgroups than CUs, where chains are too long to walk whole)
     if (units > 128 && total_chunks <= 256) return 0;
     int64_t want = 256 / units;
-    if (wide) want = std::max<int64_t>(want, (total_chunks + 255) / 256);
+    if (wide && units * want != 256) {
+        // Workgroups that do not fill whole rounds of 256: the number of segments with the
+        // shortest estimated time -- rounds x (a segment walked twice, the first time at 0.4
+        // of the cost, plus about six chunks' time for the exchange and the start).
+        double best = 1e30;
+        for (int64_t n = std::max<int64_t>(2, (total_chunks + 255) / 256); n <= 64; n++) {
+            const int64_t c = ((total_chunks + n - 1) / n + kTpAhead - 1) / kTpAhead * kTpAhead;
+            const int64_t rounds = (units * ((total_chunks + c - 1) / c) + 255) / 256;
+            const double t = (double)rounds * (1.4 * (double)c + 6.0);
+            if (t < best - 1e-9) best = t, want = n;
+        }
+    }
     want = std::min<int64_t>(want, total_chunks / 8);
     if (const char *env = getenv("FTC_TPX_SEGS")) want = std::max(1, atoi(env));  // tuning aid
     if (want < 2) return 0;
@@ -308,7 +327,7 @@ bool mfma_tp_takes(const ScanDesc *scans, int nscans, int64_t N, int64_t H, int6
     const bool wide = D != 64 || F != 64;
     const int64_t units = std::max<int64_t>(1, N * H) * nscans * tp_fblocks(F);
     int nseg = 0;
-    return tp_exchange_segments(units, L, wide, &nseg) > 0 || tp_kernel_segments(units, L, wide) > 0;
+    return tp_exchange_segments(units, L, wide, &nseg) > 0 || tp_kernel_segments(units, L, wide, mfma_scan_supported_widths(D, F)) > 0;
 }
 
 bool fused_attention_supported(const ScanDesc &sd, int64_t L) {
@@ -336,7 +355,8 @@ int mfma_scan(const ScanDesc *scans, int nscans, int64_t N, int64_t H, int64_t L
     const int tpx_seg_chunks =
         tp_shape ? tp_exchange_segments(chains * nscans * fblocks, L, wide, &tpx_nseg) : 0;
     const int tp_nseg = tp_shape && tpx_seg_chunks == 0
-                            ? tp_kernel_segments(chains * nscans * fblocks, L, wide) : 0;
+                            ? tp_kernel_segments(chains * nscans * fblocks, L, wide,
+                                                 mfma_scan_supported_widths(D, F)) : 0;
     const bool tp = tp_nseg > 0 || tpx_seg_chunks > 0;
     if (!tp && !mfma_scan_supported(scans[0], L))
         return fail(FTC_ERR_UNSUPPORTED, "no MFMA kernel takes a %d x %d state here", D, F);

@@ -123,6 +123,13 @@ def test_wide_states_on_the_chain_parallel_kernel():
     assert long[0].startswith("scan_tp_kernel (exchange): 3 scans") and "2 segments of 8192 rows" in long[0]
     need = int(field(long[0], r"workspace (\d+) bytes"))
     assert need == 65536 + 2 * 4 * 768 * 128 * 16 * 4
+    # more workgroups than CUs: segments chosen so that the rounds of 256 are full
+    rounds = lines((1, 16, 20000, 128), (1, 16, 20000, 128), backward=True)
+    assert "8 segments of 2560 rows" in rounds[0] and "768 workgroups" in rounds[0]
+    # few chains: shapes that the kernels which split L also take go to those below half
+    # the CUs, the others go to the chain-parallel kernel at any size
+    assert lines((1, 8, 2048, 128), (1, 8, 2048, 128))[0].startswith("scan_mfma_kernel")
+    assert lines((1, 4, 1000, 100), (1, 4, 1000, 100))[0].startswith("scan_tp_kernel: 1 scan")
     # bf16 rows and widths that are not multiples of 4 go the other ways
     assert lines((8, 16, 4096, 128), (8, 16, 4096, 128), dtype=_native.FTC_BF16)[0] \
         .startswith("scan_mfma_kernel")
