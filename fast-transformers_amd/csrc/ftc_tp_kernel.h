@@ -1,4 +1,9 @@
-// Chain-parallel form of the MFMA causal scan for gfx950, all-fp32 rows, 64 x 64 state.
+// Chain-parallel form of the MFMA causal scan for gfx950, all-fp32 rows, states of up to
+// 128 x 128.  Described for a 64 x 64 state; a state of more rows is walked in two blocks of
+// 64 (ND = 2: two positions of the walk per chunk, each on its own 64 columns of a and b and
+// its own rows of the slabs; their quadrants of Pt are added before the cut, the result rows
+// are stored after the second, and both read one v tile), output columns beyond 64 have a
+// workgroup of their own, and widths that do not fill the last block are clipped.
 //
 //   out[c, l, f] = sum_{j <= l} (a[c,l,:] . b[c,j,:]) * v[c,j,f]      (REV: j >= l)
 //
@@ -260,27 +265,34 @@ __global__ __launch_bounds__(512, 2) void scan_tp_kernel(uint32_t *__restrict__ 
                     b_rs, ab_in[hb] ? b_goff[q] + col + (uint32_t)(q == 0 ? row0 : row0_x) * b_slb
                                     : kNoRow, 0, 0);
             }
+            // (the second block of a chunk multiplies the v tile of the first: no second copy)
+            if (hb == 0) {
 #pragma unroll
-            for (int q = 0; q < LV; q++)
-                r.v[q] = __builtin_amdgcn_raw_buffer_load_b128(
-                    v_rs, v_in ? v_goff[q] + (uint32_t)(q == 0 ? row0 : row0_x) * v_slb : kNoRow, 0, 0);
+                for (int q = 0; q < LV; q++)
+                    r.v[q] = __builtin_amdgcn_raw_buffer_load_b128(
+                        v_rs, v_in ? v_goff[q] + (uint32_t)(q == 0 ? row0 : row0_x) * v_slb : kNoRow,
+                        0, 0);
+            }
         };
         // position k of the walk goes to LDS buffer k % 3 through register set k % PF.  The
         // first n1 positions (a multiple of PF) only feed the state: no piece of a, and the
         // consumers, who have little to do there, cut rows 16 .. 31 of b and v themselves.
-        auto cut = [&](const Raw &r, int buf, bool own) {
+        auto cut = [&](const Raw &r, int buf, bool own, int hb) {
             lds_char *const pc = unit_pc + buf * kBufBytes;
 #pragma unroll
             for (int q = 0; q < LA; q++) {
                 if (own) split_quad_to_lds(r.a[q], pc, kTileA, a_waddr[q]);
                 if (own || q == 0) split_quad_to_lds(r.b[q], pc + kOffB, kTileA, b_waddr[q]);
             }
+            if (hb == 0) {
 #pragma unroll
-            for (int q = 0; q < LV; q++)
-                if (own || q == 0) split_quad_to_lds(r.v[q], pc + kOffV, kTileV, v_waddr[q]);
+                for (int q = 0; q < LV; q++)
+                    if (own || q == 0) split_quad_to_lds(r.v[q], pc + kOffV, kTileV, v_waddr[q]);
+            }
             // (a request whose answer is not used would be moved out of the loop: the waits
             // are the same either way)
-            if (!own) asm volatile("" ::"v"(r.a[0]), "v"(r.a[1]), "v"(r.b[1]), "v"(r.v[1]));
+            if (!own) asm volatile("" ::"v"(r.a[0]), "v"(r.a[1]), "v"(r.b[1]));
+            if (!own && hb == 0) asm volatile("" ::"v"(r.v[1]));
         };
 #pragma unroll
         for (int j = 0; j < PF; j++) fetch(raw[j], j, j % ND);
@@ -292,7 +304,7 @@ __global__ __launch_bounds__(512, 2) void scan_tp_kernel(uint32_t *__restrict__ 
         for (int v = 0; v < n1; v += PF) {
 #pragma unroll
             for (int j = 0; j < PF; j++) {
-                cut(raw[j], buf, false);
+                cut(raw[j], buf, false, j % ND);
                 fetch(raw[j], v + j + PF, j % ND);
                 buf = buf == 2 ? 0 : buf + 1;
                 wg_barrier();
@@ -306,7 +318,7 @@ __global__ __launch_bounds__(512, 2) void scan_tp_kernel(uint32_t *__restrict__ 
 #pragma unroll
             for (int j = 0; j < PF; j++) {
                 if (v + j == n1 + 4) FTC_STAMP(0);
-                cut(raw[j], buf, true);
+                cut(raw[j], buf, true, j % ND);
                 if (v + j == n1 + 4) FTC_STAMP(1);
                 fetch(raw[j], v + j + PF, j % ND);
                 buf = buf == 2 ? 0 : buf + 1;
@@ -319,7 +331,7 @@ __global__ __launch_bounds__(512, 2) void scan_tp_kernel(uint32_t *__restrict__ 
 #pragma unroll
         for (int j = 0; j < PF - 1; j++) {
             if (v + j > nwalk) return;
-            cut(raw[j], buf, true);
+            cut(raw[j], buf, true, j % ND);
             buf = buf == 2 ? 0 : buf + 1;
             wg_barrier();
             __builtin_amdgcn_sched_barrier(0);
@@ -434,15 +446,17 @@ __global__ __launch_bounds__(512, 2) void scan_tp_kernel(uint32_t *__restrict__ 
             af[x - 1][ks][k] = lds_frag16(pc + k * kTileA + a_addr[x - 1][ks]);
     };
     // position-major fragment number i of a chunk (15: v first, then b^T tile by tile)
-    auto tr_frag_into = [&](Frag (&btx)[4][3], Frag (&vfx)[3], const lds_char *pc, int i) {
+    // (pcv: the buffer that holds the chunk's v tile, which is the one of its first block)
+    auto tr_frag_into = [&](Frag (&btx)[4][3], Frag (&vfx)[3], const lds_char *pc,
+                            const lds_char *pcv, int i) {
         if (i < 3)
-            vfx[i] = lds_frag_tr(pc + i * kTileV + vt_addr[0], pc + i * kTileV + vt_addr[1]);
+            vfx[i] = lds_frag_tr(pcv + i * kTileV + vt_addr[0], pcv + i * kTileV + vt_addr[1]);
         else {
             const int dt = (i - 3) / 3, k = (i - 3) % 3;
             btx[dt][k] = lds_frag_tr(pc + k * kTileA + bt_addr[dt][0], pc + k * kTileA + bt_addr[dt][1]);
         }
     };
-    auto tr_frag = [&](const lds_char *pc, int i) { tr_frag_into(bt, vf, pc, i); };
+    auto prev_buf = [](int b) -> int { return b == 0 ? 2 : b - 1; };
 
     auto next_buf = [](int b) -> int { return b == 2 ? 0 : b + 1; };
     int buf = 0;  // LDS buffer of the chunk at hand
@@ -480,8 +494,9 @@ __global__ __launch_bounds__(512, 2) void scan_tp_kernel(uint32_t *__restrict__ 
             const int row0 = v < n1 ? chunk_row0(so_chunk(v)) : -2 * kChunk;
             r.b = __builtin_amdgcn_raw_buffer_load_b128(
                 b_rs, b_in[hb] ? b_goff + (uint32_t)(D * 4 * hb) + (uint32_t)row0 * b_slb : kNoRow, 0, 0);
-            r.v = __builtin_amdgcn_raw_buffer_load_b128(
-                v_rs, v_in ? v_goff + (uint32_t)row0 * v_slb : kNoRow, 0, 0);
+            if (hb == 0)
+                r.v = __builtin_amdgcn_raw_buffer_load_b128(
+                    v_rs, v_in ? v_goff + (uint32_t)row0 * v_slb : kNoRow, 0, 0);
         };
         auto ccut_b = [&](const RawC &r, int bufk) {
             split_quad_to_lds(r.b, unit_pc + bufk * kBufBytes + kOffB, kTileA, b_waddr);
@@ -502,6 +517,7 @@ __global__ __launch_bounds__(512, 2) void scan_tp_kernel(uint32_t *__restrict__ 
 #pragma unroll
             for (int j = 0; j < PF; j++) {
                 const lds_char *pc = unit_pc + buf * kBufBytes;
+                const lds_char *pcv = j % ND == 0 ? pc : unit_pc + prev_buf(buf) * kBufBytes;
                 // position c + j + 1 is cut under the matrix instructions of position
                 // c + j - 1 (position n1 is all the producers')
                 const bool cut_next = j < PF - 1 || c + PF < n1;
@@ -511,13 +527,13 @@ __global__ __launch_bounds__(512, 2) void scan_tp_kernel(uint32_t *__restrict__ 
                 for (int i = 0; i < 24; i++) {
                     if (j % 2 == 0) {
                         S[hp][i % 4] = mfma16(bt2[i % 4][kPa[i / 4]], vf2[kPb[i / 4]], S[hp][i % 4]);
-                        if (i < 15) tr_frag_into(bt, vf, pc, i);
+                        if (i < 15) tr_frag_into(bt, vf, pc, pcv, i);
                     } else {
                         S[hp][i % 4] = mfma16(bt[i % 4][kPa[i / 4]], vf[kPb[i / 4]], S[hp][i % 4]);
-                        if (i < 15) tr_frag_into(bt2, vf2, pc, i);
+                        if (i < 15) tr_frag_into(bt2, vf2, pc, pcv, i);
                     }
                     if (i == 15 && cut_next) ccut_b(rn, bufn);
-                    if (i == 19 && cut_next) ccut_v(rn, bufn);
+                    if (i == 19 && cut_next && (j + 1) % ND == 0) ccut_v(rn, bufn);
                     __builtin_amdgcn_sched_barrier(0);
                 }
                 cfetch(rawc[(j + 1) % PF], c + j + 1 + PF, (j + 1) % ND);
@@ -596,11 +612,16 @@ __global__ __launch_bounds__(512, 2) void scan_tp_kernel(uint32_t *__restrict__ 
         const f32x4 o = O4[x][0] + O4[x][1];
         buffer_store4(o_rs, o_in ? o_off + o_lane[x] : kNoRow, o[0], o[1], o[2], o[3]);
     };
+    f32x4 Pkeep = {0.f, 0.f, 0.f, 0.f};  // the quadrant summed over the blocks so far
     for (int c = c0; c < nchunks; c++) {
 #pragma unroll
         for (int hb = 0; hb < ND; hb++) {  // block hb of the state rows
             const lds_char *pc = unit_pc + buf * kBufBytes;
-            lds_char *const ptc = pt_pc + ((ND * c + hb) & 1) * (3 * kTileP);
+            const lds_char *pcv = hb == 0 ? pc : unit_pc + prev_buf(buf) * kBufBytes;
+            lds_char *const ptc = pt_pc + (c & 1) * (3 * kTileP);
+            // The quadrants of a chunk's blocks are added up before they are cut: only the
+            // last block of a chunk hands Pt to the others and multiplies it with v.
+            const bool last_block = hb == ND - 1;
             Frag pf[2][3];
             f32x4 P4[4];
             const f32x4 zero = {0.f, 0.f, 0.f, 0.f};  // (the first product of a sum adds to a constant)
@@ -615,7 +636,7 @@ __global__ __launch_bounds__(512, 2) void scan_tp_kernel(uint32_t *__restrict__ 
                 const int ks = i % 2, m = i / 2;
                 P4[i % 4] = mfma16(bfr[ks][kPa[m]], af[0][ks][kPb[m]], i < 4 ? zero : P4[i % 4]);
                 if (i < 4) cut_s(hb, 1, i);
-                tr_frag(pc, i);
+                tr_frag_into(bt, vf, pc, pcv, i);
                 if (hb == 0 && (i == 5 || i == 7)) store_rows(i == 5 ? 0 : 1);
                 __builtin_amdgcn_sched_barrier(0);
             }
@@ -628,15 +649,19 @@ __global__ __launch_bounds__(512, 2) void scan_tp_kernel(uint32_t *__restrict__ 
             for (int i = 0; i < 12; i++) {
                 const int x = i % 2, ks = (i / 2) % 2, m = i / 4;  // piece products 0..2
                 O4[x][ks] = mfma16(sf[ks][kPa[m]], af[x][ks][kPb[m]], i < 4 && hb == 0 ? zero : O4[x][ks]);
-                if (i < 3) tr_frag(pc, 12 + i);
-                if (i == 4) P = (P4[0] + P4[1]) + (P4[2] + P4[3]);
-                if (i == 6)
+                if (i < 3) tr_frag_into(bt, vf, pc, pcv, 12 + i);
+                if (i == 4) {
+                    P = (P4[0] + P4[1]) + (P4[2] + P4[3]);
+                    if (hb > 0) P += Pkeep;
+                    if (!last_block) Pkeep = P;
+                }
+                if (i == 6 && last_block)
                     split_pair_under_mfma(__uint_as_float(__float_as_uint(P[0]) & keep[0]),
                                           __uint_as_float(__float_as_uint(P[1]) & keep[1]), plo);
-                if (i == 8)
+                if (i == 8 && last_block)
                     split_pair_under_mfma(__uint_as_float(__float_as_uint(P[2]) & keep[2]),
                                           __uint_as_float(__float_as_uint(P[3]) & keep[3]), phi);
-                if (i == 10) {
+                if (i == 10 && last_block) {
 #pragma unroll
                     for (int k = 0; k < 3; k++) {
                         const u32x2 xk = {plo[k], phi[k]};
@@ -663,10 +688,12 @@ __global__ __launch_bounds__(512, 2) void scan_tp_kernel(uint32_t *__restrict__ 
             // phase 4: (3) for tiles 2 and 3 in turn with (2a) Ot_w += v_w^T Pt; underneath:
             // tiles 0, 1 of S_w cut into pieces
             const lds_char *pn = unit_pc + buf * kBufBytes;
+            if (last_block) {
 #pragma unroll
-            for (int x = 0; x < 2; x++)
+                for (int x = 0; x < 2; x++)
 #pragma unroll
-                for (int k = 0; k < 3; k++) pf[x][k] = lds_frag16(ptc + k * kTileP + pt_raddr[x]);
+                    for (int k = 0; k < 3; k++) pf[x][k] = lds_frag16(ptc + k * kTileP + pt_raddr[x]);
+            }
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int i = 0; i < 4; i++) {
@@ -682,7 +709,7 @@ __global__ __launch_bounds__(512, 2) void scan_tp_kernel(uint32_t *__restrict__ 
                     S[hb][2 + t % 2] = mfma16(bt[2 + t % 2][kPa[t / 2]], vf[kPb[t / 2]], S[hb][2 + t % 2]);
                 }
                 const int x = i % 2, m = i / 2;
-                O4[x][m % 2] = mfma16(vf[kPa[m]], pf[x][kPb[m]], O4[x][m % 2]);
+                if (last_block) O4[x][m % 2] = mfma16(vf[kPa[m]], pf[x][kPb[m]], O4[x][m % 2]);
                 rm_frag(pn, 4 + i);
                 if (i < 2) rm_frag(pn, 16 + i);
                 __builtin_amdgcn_sched_barrier(0);
