@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the causal linear-attention product on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg2|cfg3|cfg5|cfg4op]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg2|cfg3|cfg5|cfg4op|cfg4|wide]
 
 A step is one forward + backward of ``causal_dot_product`` over one batch of synthetic input,
 called through the C ABI with outputs and workspace pre-allocated and every input already in
@@ -49,6 +49,9 @@ WORKLOADS = {
     "cfg3": (1, 16, 65536, 64, 64, "f32", 3),
     "cfg4op": (10, 8, 4096, 64, 64, "f32", 4),
     "cfg5": (4, 32, 16384, 32, 128, "bf16", 5),
+    # not one of the reference's configurations: a 128 x 128 state, for the profiles of the
+    # chain-parallel kernel's wide form
+    "wide": (8, 16, 4096, 128, 128, "f32", 6),
 }
 
 
