@@ -97,7 +97,9 @@ __device__ __forceinline__ constexpr int b_tile_column(int d) {
     return 32 * (d / 32) + 16 * ((d / 4) % 2) + 4 * ((d % 32) / 8) + d % 4;
 }
 
-template <int ND>
+// KS2: groups of 32 rows in the state's last block (1: a state of 65 .. 96 rows, whose last
+// block skips the matrix instructions and fragment reads of its empty half)
+template <int ND, int KS2>
 __global__ __launch_bounds__(512, 2) void scan_tp_kernel(uint32_t *__restrict__ ws_ptr, ScanArgs p) {
     constexpr int D = 64, F = 64;              // one block of state rows and of output columns
     constexpr int T = 256;                     // producer lanes
@@ -192,6 +194,8 @@ __global__ __launch_bounds__(512, 2) void scan_tp_kernel(uint32_t *__restrict__ 
     auto so_chunk = [&](int v) -> int { return exchange ? so0 + n1c - 1 - v / ND : so0 + v / ND; };
     auto walk_chunk = [&](int v) -> int { return v < n1 ? so_chunk(v) : c0 + (v - n1) / ND; };
     constexpr uint32_t kNoRow = 0x80000000u;  // an offset outside every descriptor
+    // groups of 32 rows of block hb
+    auto block_ks = [](int hb) -> int { return hb == ND - 1 ? KS2 : 2; };
     auto chunk_row0 = [&](int c) -> int { return REV ? rows - kChunk * (c + 1) : kChunk * c; };
     __syncthreads();
 #ifdef FTC_TIMELINE
@@ -438,8 +442,9 @@ __global__ __launch_bounds__(512, 2) void scan_tp_kernel(uint32_t *__restrict__ 
     // scheduling barriers keep the compiler from regrouping them.
     Frag af[2][2][3], bfr[2][3], bt[4][3], vf[3];
     // row-major fragment number i of a chunk (18: b for the quadrant first, then a)
-    auto rm_frag = [&](const lds_char *pc, int i) {
+    auto rm_frag = [&](const lds_char *pc, int i, int hb) {  // hb: the block of that position
         const int k = i % 3, ks = (i / 3) % 2, x = i / 6;
+        if (ks >= block_ks(hb)) return;
         if (x == 0)
             bfr[ks][k] = lds_frag8x2(pc + k * kTileA + b_addr[ks][0], pc + k * kTileA + b_addr[ks][1]);
         else
@@ -448,7 +453,8 @@ __global__ __launch_bounds__(512, 2) void scan_tp_kernel(uint32_t *__restrict__ 
     // position-major fragment number i of a chunk (15: v first, then b^T tile by tile)
     // (pcv: the buffer that holds the chunk's v tile, which is the one of its first block)
     auto tr_frag_into = [&](Frag (&btx)[4][3], Frag (&vfx)[3], const lds_char *pc,
-                            const lds_char *pcv, int i) {
+                            const lds_char *pcv, int i, int hb) {
+        if (i >= 3 && (i - 3) / 6 >= block_ks(hb)) return;  // tiles 2, 3: rows 32 .. 63
         if (i < 3)
             vfx[i] = lds_frag_tr(pcv + i * kTileV + vt_addr[0], pcv + i * kTileV + vt_addr[1]);
         else {
@@ -525,12 +531,15 @@ __global__ __launch_bounds__(512, 2) void scan_tp_kernel(uint32_t *__restrict__ 
                 const int hp = (j + ND - 1) % ND;  // block of the position before
 #pragma unroll
                 for (int i = 0; i < 24; i++) {
+                    const bool rows_exist = (i % 4) / 2 < block_ks(hp);
                     if (j % 2 == 0) {
-                        S[hp][i % 4] = mfma16(bt2[i % 4][kPa[i / 4]], vf2[kPb[i / 4]], S[hp][i % 4]);
-                        if (i < 15) tr_frag_into(bt, vf, pc, pcv, i);
+                        if (rows_exist)
+                            S[hp][i % 4] = mfma16(bt2[i % 4][kPa[i / 4]], vf2[kPb[i / 4]], S[hp][i % 4]);
+                        if (i < 15) tr_frag_into(bt, vf, pc, pcv, i, j % ND);
                     } else {
-                        S[hp][i % 4] = mfma16(bt[i % 4][kPa[i / 4]], vf[kPb[i / 4]], S[hp][i % 4]);
-                        if (i < 15) tr_frag_into(bt2, vf2, pc, pcv, i);
+                        if (rows_exist)
+                            S[hp][i % 4] = mfma16(bt[i % 4][kPa[i / 4]], vf[kPb[i / 4]], S[hp][i % 4]);
+                        if (i < 15) tr_frag_into(bt2, vf2, pc, pcv, i, j % ND);
                     }
                     if (i == 15 && cut_next) ccut_b(rn, bufn);
                     if (i == 19 && cut_next && (j + 1) % ND == 0) ccut_v(rn, bufn);
@@ -546,15 +555,16 @@ __global__ __launch_bounds__(512, 2) void scan_tp_kernel(uint32_t *__restrict__ 
         // the last of these positions (n1 is even: its fragments are in the second set)
 #pragma unroll
         for (int i = 0; i < 24; i++) {
-            S[ND - 1][i % 4] = mfma16(bt2[i % 4][kPa[i / 4]], vf2[kPb[i / 4]], S[ND - 1][i % 4]);
-            if (i < 18) rm_frag(unit_pc + buf * kBufBytes, i);  // our own first chunk is cut
+            if ((i % 4) / 2 < KS2)
+                S[ND - 1][i % 4] = mfma16(bt2[i % 4][kPa[i / 4]], vf2[kPb[i / 4]], S[ND - 1][i % 4]);
+            if (i < 18) rm_frag(unit_pc + buf * kBufBytes, i, 0);  // our own first chunk is cut
             __builtin_amdgcn_sched_barrier(0);
         }
     } else {
         wg_barrier();
         FTC_STAMP(13);  // first chunk cut
 #pragma unroll
-        for (int i = 0; i < 18; i++) rm_frag(unit_pc, i);
+        for (int i = 0; i < 18; i++) rm_frag(unit_pc, i, 0);
     }
     if (exchange) {
         // ---- the sum of this segment's rows goes out, the state before the segment comes in ----
@@ -634,9 +644,12 @@ __global__ __launch_bounds__(512, 2) void scan_tp_kernel(uint32_t *__restrict__ 
 #pragma unroll
             for (int i = 0; i < 12; i++) {
                 const int ks = i % 2, m = i / 2;
-                P4[i % 4] = mfma16(bfr[ks][kPa[m]], af[0][ks][kPb[m]], i < 4 ? zero : P4[i % 4]);
-                if (i < 4) cut_s(hb, 1, i);
-                tr_frag_into(bt, vf, pc, pcv, i);
+                if (ks < block_ks(hb))
+                    P4[i % 4] = mfma16(bfr[ks][kPa[m]], af[0][ks][kPb[m]], i < 4 ? zero : P4[i % 4]);
+                else if (i < 4)
+                    P4[i % 4] = zero;
+                if (i < 4 && block_ks(hb) > 1) cut_s(hb, 1, i);
+                tr_frag_into(bt, vf, pc, pcv, i, hb);
                 if (hb == 0 && (i == 5 || i == 7)) store_rows(i == 5 ? 0 : 1);
                 __builtin_amdgcn_sched_barrier(0);
             }
@@ -648,8 +661,11 @@ __global__ __launch_bounds__(512, 2) void scan_tp_kernel(uint32_t *__restrict__ 
 #pragma unroll
             for (int i = 0; i < 12; i++) {
                 const int x = i % 2, ks = (i / 2) % 2, m = i / 4;  // piece products 0..2
-                O4[x][ks] = mfma16(sf[ks][kPa[m]], af[x][ks][kPb[m]], i < 4 && hb == 0 ? zero : O4[x][ks]);
-                if (i < 3) tr_frag_into(bt, vf, pc, pcv, 12 + i);
+                if (ks < block_ks(hb))
+                    O4[x][ks] = mfma16(sf[ks][kPa[m]], af[x][ks][kPb[m]], i < 4 && hb == 0 ? zero : O4[x][ks]);
+                else if (i < 4 && hb == 0)
+                    O4[x][ks] = zero;
+                if (i < 3) tr_frag_into(bt, vf, pc, pcv, 12 + i, hb);
                 if (i == 4) {
                     P = (P4[0] + P4[1]) + (P4[2] + P4[3]);
                     if (hb > 0) P += Pkeep;
@@ -675,7 +691,7 @@ __global__ __launch_bounds__(512, 2) void scan_tp_kernel(uint32_t *__restrict__ 
 #pragma unroll
             for (int i = 0; i < 12; i++) {
                 const int x = i % 2, ks = (i / 2) % 2, m = 3 + i / 4;  // piece products 3..5
-                O4[x][ks] = mfma16(sf[ks][kPa[m]], af[x][ks][kPb[m]], O4[x][ks]);
+                if (ks < block_ks(hb)) O4[x][ks] = mfma16(sf[ks][kPa[m]], af[x][ks][kPb[m]], O4[x][ks]);
                 S[hb][i % 2] = mfma16(bt[i % 2][kPa[i / 2]], vf[kPb[i / 2]], S[hb][i % 2]);
                 __builtin_amdgcn_sched_barrier(0);
             }
@@ -697,21 +713,22 @@ __global__ __launch_bounds__(512, 2) void scan_tp_kernel(uint32_t *__restrict__ 
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int i = 0; i < 4; i++) {
-                S[hb][2 + i % 2] = mfma16(bt[2 + i % 2][kPa[i / 2]], vf[kPb[i / 2]], S[hb][2 + i % 2]);
+                if (block_ks(hb) > 1)
+                    S[hb][2 + i % 2] = mfma16(bt[2 + i % 2][kPa[i / 2]], vf[kPb[i / 2]], S[hb][2 + i % 2]);
                 cut_s((hb + 1) % ND, 0, i);
-                rm_frag(pn, i);  // (past the last chunk: a buffer of zeros)
+                rm_frag(pn, i, (hb + 1) % ND);  // (past the last chunk: a buffer of zeros)
                 __builtin_amdgcn_sched_barrier(0);
             }
 #pragma unroll
             for (int i = 0; i < 12; i++) {
-                if (i < 8) {
+                if (i < 8 && block_ks(hb) > 1) {
                     const int t = 4 + i;
                     S[hb][2 + t % 2] = mfma16(bt[2 + t % 2][kPa[t / 2]], vf[kPb[t / 2]], S[hb][2 + t % 2]);
                 }
                 const int x = i % 2, m = i / 2;
                 if (last_block) O4[x][m % 2] = mfma16(vf[kPa[m]], pf[x][kPb[m]], O4[x][m % 2]);
-                rm_frag(pn, 4 + i);
-                if (i < 2) rm_frag(pn, 16 + i);
+                rm_frag(pn, 4 + i, (hb + 1) % ND);
+                if (i < 2) rm_frag(pn, 16 + i, (hb + 1) % ND);
                 __builtin_amdgcn_sched_barrier(0);
             }
             if (c == c0 + 4) FTC_STAMP(5);
