@@ -295,15 +295,16 @@ int run_scans(const ScanDesc *scans, int n, int64_t N, int64_t H, int64_t L, voi
     bool native[kMfmaMaxScans], padded[kMfmaMaxScans], taken[kMfmaMaxScans] = {};
     bool any_padded = false;
     if (n > kMfmaMaxScans) return fail(FTC_ERR_INVALID, "too many scans");
-    // Wide states and widths that are multiples of 4: the scans of one shape go to the
-    // chain-parallel kernel together where it takes them (64 x 64 finds it below).
+    // The scans of one shape go to the chain-parallel kernel together where it takes them
+    // (whole scans: a column slice made below is never offered to it).
+    bool offered[kMfmaMaxScans] = {};
     for (int i = 0; i < n; i++) {
-        if (taken[i] || (scans[i].a.width == 64 && scans[i].v.width == 64)) continue;
+        if (offered[i]) continue;
         ScanDesc group[kMfmaMaxScans];
         int members[kMfmaMaxScans], ngroup = 0;
         for (int j = i; j < n; j++)
-            if (!taken[j] && scans[j].a.width == scans[i].a.width && scans[j].v.width == scans[i].v.width)
-                members[ngroup] = j, group[ngroup++] = scans[j];
+            if (!offered[j] && scans[j].a.width == scans[i].a.width && scans[j].v.width == scans[i].v.width)
+                offered[j] = true, members[ngroup] = j, group[ngroup++] = scans[j];
         if (!mfma_tp_takes(group, ngroup, N, H, L)) continue;
         const int rc = mfma_scan(group, ngroup, N, H, L, workspace, workspace_bytes, stream);
         if (rc) return rc;
@@ -331,7 +332,8 @@ int run_scans(const ScanDesc *scans, int n, int64_t N, int64_t H, int64_t L, voi
     int nbatch = 0;
     auto flush = [&]() -> int {
         if (nbatch == 0) return FTC_OK;
-        const int rc = mfma_scan(batch, nbatch, N, H, L, workspace, workspace_bytes, stream);
+        const int rc = mfma_scan(batch, nbatch, N, H, L, workspace, workspace_bytes, stream, nullptr,
+                                 false);
         nbatch = 0;
         return rc;
     };

@@ -119,8 +119,8 @@ bool mfma_scan_same_launch(const ScanDesc &x, const ScanDesc &y);
 // Workspace for `nscans` scans of one (D, F) run side by side in one launch.
 int64_t mfma_scan_workspace_bytes(int64_t N, int64_t H, int64_t L, int64_t D, int64_t F,
                                   int nscans);
-// The chain-parallel kernel: all-fp32 scans of one shape whose state has more than 32 and at
-// most 128 rows and columns, widths multiples of 4 (also widths that mfma_scan_supported
+// The chain-parallel kernel: all-fp32 scans of one shape whose state has 16 to 128 rows and
+// columns, widths multiples of 4 (also widths that mfma_scan_supported
 // does not list).  True when mfma_scan would run these scans, side by side, on that kernel;
 // its workspace (part of mfma_scan_workspace_bytes where both apply).
 bool mfma_tp_takes(const ScanDesc *scans, int nscans, int64_t N, int64_t H, int64_t L);
@@ -135,10 +135,11 @@ struct FusedAttention {
 bool fused_attention_supported(const ScanDesc &scan, int64_t L);
 int64_t fused_attention_workspace_bytes(int64_t N, int64_t H, int64_t L, int64_t D, int64_t F);
 // Runs scans[0..nscans) (all of the same row widths) in one launch.  `fused`: a single
-// forward scan in its fused attention form.
+// forward scan in its fused attention form.  `may_chain_parallel` = false keeps the launch
+// off the chain-parallel kernel (column slices of a scan that it has declined as a whole).
 int mfma_scan(const ScanDesc *scans, int nscans, int64_t N, int64_t H, int64_t L,
               void *workspace, size_t workspace_bytes, hipStream_t stream,
-              const FusedAttention *fused = nullptr);
+              const FusedAttention *fused = nullptr, bool may_chain_parallel = true);
 
 // Fill every row of `out` with zeros (used for empty contractions).
 int zero_rows(const OperandOut &out, int64_t N, int64_t H, int64_t L, hipStream_t stream);

@@ -24,11 +24,11 @@ bool use_wg_kernel(int64_t D, int64_t F, int nscans, int64_t L, bool all_f32) {
     return nscans == 1 && L >= 128 * kChunk && D == 64 && F == 64;
 }
 
-// Row widths that the chain-parallel kernel takes (ftc_tp_kernel.h): states of up to 128 x 128,
-// walked in blocks of 64 rows, with one workgroup per block of 64 output columns; widths
-// that are multiples of 4 (a lane's 16 bytes lie wholly inside a row or wholly outside).
+// Row widths that the chain-parallel kernel takes (ftc_tp_kernel.h): states of 16 x 16 to
+// 128 x 128, walked in blocks of 64 rows, with one workgroup per block of 64 output columns;
+// widths that are multiples of 4 (a lane's 16 bytes lie wholly inside a row or wholly outside).
 bool tp_widths(int64_t D, int64_t F) {
-    return D > 32 && D <= 128 && F > 32 && F <= 128 && D % 4 == 0 && F % 4 == 0;
+    return D >= 16 && D <= 128 && F >= 16 && F <= 128 && D % 4 == 0 && F % 4 == 0;
 }
 int64_t tp_fblocks(int64_t F) { return (F + 63) / 64; }
 
@@ -150,6 +150,26 @@ int tp_exchange_segments(int64_t units, int64_t L, bool wide, int *nseg) {
     if (n < 2 || seg_chunks > 256 || n > 4096 || 4 * units * n > kMaxWaves) return 0;
     *nseg = (int)n;
     return (int)seg_chunks;
+}
+
+// The chain-parallel kernel's plan for `nscans` scans of a D x F state over chains x L rows:
+// *seg_chunks > 0: an exchange with *nseg segments of that many chunks; else *nseg > 0: chains
+// cut into *nseg segments that need no exchange; both 0: another kernel takes the launch.
+void tp_plan(int64_t D, int64_t F, int64_t chains, int nscans, int64_t L, int *nseg, int *seg_chunks) {
+    *nseg = *seg_chunks = 0;
+    if (!tp_widths(D, F)) return;
+    const bool wide = D != 64 || F != 64;
+    const bool others = mfma_scan_supported_widths(D, F);
+    const int64_t units = chains * nscans * tp_fblocks(F);
+    // Shapes of the other kernels with 32 rows or columns (a workgroup here has half of its
+    // matrix work or half of its consumers to spare for them): measured at N=8, H=16, L=4096,
+    // forward + backward, 32 x 128 0.62 against 0.80 ms and 128 x 32 0.76 against 0.78 on whole
+    // chains, but 32 x 32 0.34 against 0.28, and with an exchange (N=4, H=16, L=16384)
+    // 128 x 32 1.73 against 1.58 and 32 x 128 1.70 against 1.59: those stay where they were.
+    const bool narrow = others && (D <= 32 || F <= 32);
+    if (narrow && D <= 32 && F <= 32) return;
+    if (!narrow) *seg_chunks = tp_exchange_segments(units, L, wide, nseg);
+    if (*seg_chunks == 0) *nseg = tp_kernel_segments(units, L, wide, others);
 }
 
 // workspace of the exchange: control block, then two state slots (own sum, group total) of
@@ -295,12 +315,10 @@ int64_t mfma_scan_workspace_bytes(int64_t N, int64_t H, int64_t L, int64_t D, in
 }
 
 int64_t mfma_tp_workspace_bytes(int64_t N, int64_t H, int64_t L, int64_t D, int64_t F, int nscans) {
-    if (!tp_widths(D, F)) return 0;
-    const int64_t units = std::max<int64_t>(1, N * H) * nscans * tp_fblocks(F);
-    int nseg = 0;
-    if (tp_exchange_segments(units, L, D != 64 || F != 64, &nseg) > 0)
-        return tp_exchange_workspace_bytes(units, nseg, D);
-    return 0;
+    int nseg = 0, seg_chunks = 0;
+    const int64_t chains = std::max<int64_t>(1, N * H);
+    tp_plan(D, F, chains, nscans, L, &nseg, &seg_chunks);
+    return seg_chunks > 0 ? tp_exchange_workspace_bytes(chains * nscans * tp_fblocks(F), nseg, D) : 0;
 }
 
 bool mfma_tp_takes(const ScanDesc *scans, int nscans, int64_t N, int64_t H, int64_t L) {
@@ -324,10 +342,9 @@ bool mfma_tp_takes(const ScanDesc *scans, int nscans, int64_t N, int64_t H, int6
     // the chain-parallel kernel addresses a whole chain through one 32-bit descriptor
     if ((L + 2 * kChunk) * std::max<int64_t>(widest_stride, std::max(D, F)) * 4 >= 0x7fffffffLL)
         return false;
-    const bool wide = D != 64 || F != 64;
-    const int64_t units = std::max<int64_t>(1, N * H) * nscans * tp_fblocks(F);
-    int nseg = 0;
-    return tp_exchange_segments(units, L, wide, &nseg) > 0 || tp_kernel_segments(units, L, wide, mfma_scan_supported_widths(D, F)) > 0;
+    int nseg = 0, seg_chunks = 0;
+    tp_plan(D, F, std::max<int64_t>(1, N * H), nscans, L, &nseg, &seg_chunks);
+    return nseg > 0;
 }
 
 bool fused_attention_supported(const ScanDesc &sd, int64_t L) {
@@ -341,22 +358,20 @@ int64_t fused_attention_workspace_bytes(int64_t N, int64_t H, int64_t L, int64_t
 
 int mfma_scan(const ScanDesc *scans, int nscans, int64_t N, int64_t H, int64_t L,
               void *workspace, size_t workspace_bytes, hipStream_t stream,
-              const FusedAttention *fused) {
+              const FusedAttention *fused, bool may_chain_parallel) {
     if (nscans < 1 || nscans > kMaxScans) return fail(FTC_ERR_INVALID, "bad scan count");
     const int D = scans[0].a.width, F = scans[0].v.width;
     const Combo combo = combo_of(scans[0]);
     if (fused && (nscans != 1 || !fused_attention_supported(scans[0], L)))
         return fail(FTC_ERR_UNSUPPORTED, "no fused attention kernel for this shape or layout");
-    const bool tp_shape = !fused && mfma_tp_takes(scans, nscans, N, H, L);
-    const bool wide = D != 64 || F != 64;
+    const bool tp_shape = !fused && may_chain_parallel && mfma_tp_takes(scans, nscans, N, H, L);
     const int64_t chains = std::max<int64_t>(1, N * H);
     const int64_t fblocks = tp_shape ? tp_fblocks(F) : 1;
-    int tpx_nseg = 0;
-    const int tpx_seg_chunks =
-        tp_shape ? tp_exchange_segments(chains * nscans * fblocks, L, wide, &tpx_nseg) : 0;
-    const int tp_nseg = tp_shape && tpx_seg_chunks == 0
-                            ? tp_kernel_segments(chains * nscans * fblocks, L, wide,
-                                                 mfma_scan_supported_widths(D, F)) : 0;
+    int tpx_nseg = 0, tpx_seg_chunks = 0, tp_nseg = 0;
+    if (tp_shape) {
+        tp_plan(D, F, chains, nscans, L, &tpx_nseg, &tpx_seg_chunks);
+        if (tpx_seg_chunks == 0) tp_nseg = tpx_nseg, tpx_nseg = 0;
+    }
     const bool tp = tp_nseg > 0 || tpx_seg_chunks > 0;
     if (!tp && !mfma_scan_supported(scans[0], L))
         return fail(FTC_ERR_UNSUPPORTED, "no MFMA kernel takes a %d x %d state here", D, F);

@@ -686,6 +686,8 @@ TP_SHAPES = [
     # 64), widths that leave the last block partly empty
     (10, 8, 1000, 128, 128), (8, 8, 333, 96, 96), (16, 4, 97, 100, 100), (4, 4, 640, 48, 80),
     (2, 32, 33, 68, 36), (16, 8, 1, 128, 36), (4, 8, 700, 64, 128),
+    # 32 rows or columns (half a block of rows; consumers without columns), narrower still
+    (10, 8, 300, 32, 128), (10, 8, 300, 128, 32), (8, 8, 200, 16, 16), (8, 8, 200, 20, 40),
 ]
 
 

@@ -58,7 +58,10 @@ def test_what_the_chain_parallel_kernel_leaves_to_the_others():
     assert many[0].startswith("scan_dma_kernel")
     # other state sizes and element types
     assert lines((10, 8, 1000, 32), (10, 8, 1000, 32))[0].startswith("scan_dma_kernel")
-    assert lines((10, 8, 1000, 32), (10, 8, 1000, 128))[0].startswith("scan_dma_kernel")
+    # (32 rows or columns: the chain-parallel kernel on whole chains unless both are 32,
+    # the kernels that split L where it would need an exchange)
+    assert lines((10, 8, 1000, 32), (10, 8, 1000, 128))[0].startswith("scan_tp_kernel:")
+    assert lines((4, 16, 16384, 32), (4, 16, 16384, 128))[0].startswith("scan_dma_kernel")
     assert lines((1, 3, 500, 128), (1, 3, 500, 128))[0].startswith("scan_mfma_kernel")  # few chains
     assert lines((4, 8, 1000, 64), (4, 8, 1000, 64), dtype=_native.FTC_BF16)[0] \
         .startswith("scan_mfma_kernel")
@@ -68,10 +71,10 @@ def test_what_the_chain_parallel_kernel_leaves_to_the_others():
     # backward the two copies serve all three scans, and dQ and dK are copied back)
     odd = lines((8, 16, 4096, 25), (8, 16, 4096, 64))
     assert odd[0].startswith("pad_rows_kernel: 2 operands") and "0 results" in odd[0]
-    assert odd[1].startswith("scan_dma_kernel") and "state 32 x 64" in odd[1]
+    assert odd[1].startswith("scan_tp_kernel") and "state 32 x 64" in odd[1]
     odd = lines((8, 16, 4096, 25), (8, 16, 4096, 64), backward=True)
     assert odd[0].startswith("pad_rows_kernel: 2 operands") and "2 results" in odd[0]
-    assert odd[1].startswith("scan_dma_kernel: 2 scans") and "state 64 x 32" in odd[1]
+    assert odd[1].startswith("scan_tp_kernel: 2 scans") and "state 64 x 32" in odd[1]
     wide = lines((8, 16, 4096, 99), (8, 16, 4096, 101), backward=True)
     assert wide[0].startswith("pad_rows_kernel: 4 operands") and "3 results" in wide[0]
     assert wide[1].startswith("scan_tp_kernel: 3 scans") and "state 128 x 128" in wide[1]
