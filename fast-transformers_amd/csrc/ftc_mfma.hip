@@ -168,6 +168,12 @@ void tp_plan(int64_t D, int64_t F, int64_t chains, int nscans, int64_t L, int *n
     // 128 x 32 1.73 against 1.58 and 32 x 128 1.70 against 1.59: those stay where they were.
     const bool narrow = others && (D <= 32 || F <= 32);
     if (narrow && D <= 32 && F <= 32) return;
+    // ... and so do thousands of chains of one or two chunks with a state of at most 64 x 64,
+    // where a workgroup's start costs more than its chunks (8192 chains, L=64: 32 x 128 1.17
+    // against 0.60 ms, 20 x 20 0.63 against 0.46 on padded copies), and 32-wide shapes on more
+    // than two rounds of workgroups, as for 64 x 64.
+    if (narrow && units > 512) return;
+    if (D <= 64 && F <= 64 && units > 512 && L <= 2 * kChunk) return;
     if (!narrow) *seg_chunks = tp_exchange_segments(units, L, wide, nseg);
     if (*seg_chunks == 0) *nseg = tp_kernel_segments(units, L, wide, others);
 }

@@ -133,6 +133,11 @@ def test_wide_states_on_the_chain_parallel_kernel():
     # the CUs, the others go to the chain-parallel kernel at any size
     assert lines((1, 8, 2048, 128), (1, 8, 2048, 128))[0].startswith("scan_mfma_kernel")
     assert lines((1, 4, 1000, 100), (1, 4, 1000, 100))[0].startswith("scan_tp_kernel: 1 scan")
+    # thousands of chains of one or two chunks with a small state, 32-wide shapes on more
+    # than two rounds of workgroups: the other routes
+    assert lines((512, 16, 64, 20), (512, 16, 64, 20))[0].startswith("pad_rows_kernel")
+    assert lines((512, 16, 64, 32), (512, 16, 64, 128))[0].startswith("scan_dma_kernel")
+    assert lines((512, 16, 64, 100), (512, 16, 64, 100))[0].startswith("scan_tp_kernel")
     # bf16 rows and widths that are not multiples of 4 go the other ways
     assert lines((8, 16, 4096, 128), (8, 16, 4096, 128), dtype=_native.FTC_BF16)[0] \
         .startswith("scan_mfma_kernel")
