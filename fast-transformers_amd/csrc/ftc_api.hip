@@ -144,7 +144,9 @@ void launch_pad_rows(void *strided, int64_t sn, int64_t sh, int64_t sl, int64_t 
                            (uint16_t *)strided, sn, sh, sl, H, L, N * H, w, wp, (uint16_t *)dense);
 }
 
-constexpr int64_t kPadMinRows = 8192;
+// (measured down to 512 rows: E = 25, M = 33, one chain of 512 positions, forward + backward
+// 0.10 ms on the copies against 0.30 ms on the VALU kernel)
+constexpr int64_t kPadMinRows = 512;
 int64_t round_up(int64_t x, int64_t m) { return (x + m - 1) / m * m; }
 // padded widths of a D x F scan (0: the matrix-core kernels take no such state)
 int padded_rows(int64_t D) { return D <= 32 ? 32 : D <= 64 ? 64 : D <= 96 ? 96 : D <= 128 ? 128 : 0; }
