@@ -39,9 +39,9 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 matrix, published
 # carries it only while the sources are unchanged, otherwise null.
 MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {
     # workload: (bytes, kernel source hash at the time of the measurement)
-    "cfg2": (137379788, "d997f4187d07b389"),
-    "cfg3": (3140189445, "d997f4187d07b389"),
-    "wide": (1877441753, "d997f4187d07b389"),
+    "cfg2": (137328454, "a99269205501b99a"),
+    "cfg3": (3140108459, "a99269205501b99a"),
+    "wide": (1877023479, "a99269205501b99a"),
 }
 
 WORKLOADS = {
