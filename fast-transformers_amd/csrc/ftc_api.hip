@@ -102,12 +102,13 @@ int read_dims(const ftc_tensor4 *q, const ftc_tensor4 *v, Dims *d) {
 // kernels are several times faster than the generic one.
 
 // Rows of a strided operand of width w <-> rows of a dense buffer of width wp (a multiple of
-// 32), chain after chain.  A lane moves one 16-byte group of the dense row (T: uint32_t for
-// fp32, uint16_t for bf16 elements); blockIdx.y walks the chains.
+// 32), chain after chain, Lp >= L dense rows per chain (more than L for a state whose rows
+// are padded as well; those rows are not touched here).  A lane moves one 16-byte group of
+// the dense row (T: uint32_t for fp32, uint16_t for bf16 elements); blockIdx.y walks the chains.
 template <typename T, bool PAD>
 __global__ __launch_bounds__(256) void pad_rows_kernel(T *strided, int64_t sn, int64_t sh, int64_t sl,
-                                                       int64_t H, int64_t L, int64_t chains, int w,
-                                                       int wp, T *dense) {
+                                                       int64_t H, int64_t L, int64_t Lp, int64_t chains,
+                                                       int w, int wp, T *dense) {
     constexpr int PER = 16 / sizeof(T);
     typedef T Vec __attribute__((ext_vector_type(PER)));
     const uint32_t groups = (uint32_t)wp / PER;
@@ -116,7 +117,7 @@ __global__ __launch_bounds__(256) void pad_rows_kernel(T *strided, int64_t sn, i
     const uint32_t l = j / groups, c0 = (j % groups) * PER;
     for (int64_t chain = blockIdx.y; chain < chains; chain += gridDim.y) {
         T *row = strided + (chain / H) * sn + (chain % H) * sh + (int64_t)l * sl;
-        Vec *slot = (Vec *)(dense + (chain * L + l) * wp + c0);
+        Vec *slot = (Vec *)(dense + (chain * Lp + l) * wp + c0);
         if (PAD) {
             Vec x;
 #pragma unroll
@@ -133,21 +134,24 @@ __global__ __launch_bounds__(256) void pad_rows_kernel(T *strided, int64_t sn, i
 
 template <bool PAD>
 void launch_pad_rows(void *strided, int64_t sn, int64_t sh, int64_t sl, int64_t N, int64_t H,
-                     int64_t L, int w, int wp, int esz, void *dense, hipStream_t stream) {
+                     int64_t L, int w, int wp, int esz, void *dense, hipStream_t stream,
+                     int64_t Lp = 0) {
+    if (Lp == 0) Lp = L;
     const int per = 16 / esz;
     const dim3 grid((unsigned)((L * (wp / per) + 255) / 256), (unsigned)std::min<int64_t>(N * H, 65535));
     if (esz == 4)
         hipLaunchKernelGGL((pad_rows_kernel<uint32_t, PAD>), grid, dim3(256), 0, stream,
-                           (uint32_t *)strided, sn, sh, sl, H, L, N * H, w, wp, (uint32_t *)dense);
+                           (uint32_t *)strided, sn, sh, sl, H, L, Lp, N * H, w, wp, (uint32_t *)dense);
     else
         hipLaunchKernelGGL((pad_rows_kernel<uint16_t, PAD>), grid, dim3(256), 0, stream,
-                           (uint16_t *)strided, sn, sh, sl, H, L, N * H, w, wp, (uint16_t *)dense);
+                           (uint16_t *)strided, sn, sh, sl, H, L, Lp, N * H, w, wp, (uint16_t *)dense);
 }
 
 // (measured down to 512 rows: E = 25, M = 33, one chain of 512 positions, forward + backward
 // 0.10 ms on the copies against 0.30 ms on the VALU kernel)
 constexpr int64_t kPadMinRows = 512;
 int64_t round_up(int64_t x, int64_t m) { return (x + m - 1) / m * m; }
+__global__ void zero_words_kernel(uint32_t *p, uint32_t words);
 // padded widths of a D x F scan (0: the matrix-core kernels take no such state)
 int padded_rows(int64_t D) { return D <= 32 ? 32 : D <= 64 ? 64 : D <= 96 ? 96 : D <= 128 ? 128 : 0; }
 
@@ -164,7 +168,8 @@ int64_t padded_scan_workspace_bytes(int64_t N, int64_t H, int64_t L, int64_t D, 
         return 0;
     return std::max<int64_t>(round_up(scan_workspace_bytes(N, H, L, Dp, Fp), 256),
                              FTC_WORKSPACE_CONTROL_BYTES) +
-           2 * round_up(rows * Dp * 4, 256) + 2 * round_up(rows * Fp * 4, 256);
+           2 * round_up(rows * Dp * 4, 256) + 2 * round_up(rows * Fp * 4, 256) +
+           2 * round_up(N * H * Dp * Fp * 4, 256);  // (the states handed in and out)
 }
 
 int run_scans(const ScanDesc *scans, int n, int64_t N, int64_t H, int64_t L, void *workspace,
@@ -201,11 +206,26 @@ int padded_scans(const ScanDesc *scans, int n, const bool *take, int64_t N, int6
         copies[ncopies] = Copy{ptr, sn, sh, sl, dtype, width, padded, is_output, nullptr};
         return ncopies++;
     };
+    // the states handed in and out, padded the same way (rows and columns)
+    struct StateCopy {
+        StateRef ref;
+        int D, F, Dp, Fp, scan;
+        bool is_output;
+        char *dense;
+    };
+    StateCopy states[2 * kMfmaMaxScans];
+    int nstates = 0;
     int which[kMfmaMaxScans][4];
     for (int i = 0; i < n; i++) {
         if (!take[i]) continue;
         const ScanDesc &sc = scans[i];
         const int Dp = padded_rows(sc.a.width), Fp = (int)round_up(sc.v.width, 32);
+        if (Dp != sc.a.width || Fp != sc.v.width) {
+            if (sc.initial.ptr)
+                states[nstates++] = StateCopy{sc.initial, sc.a.width, sc.v.width, Dp, Fp, nwork, false, nullptr};
+            if (sc.final_.ptr)
+                states[nstates++] = StateCopy{sc.final_, sc.a.width, sc.v.width, Dp, Fp, nwork, true, nullptr};
+        }
         ws_scan = std::max(ws_scan, round_up(scan_workspace_bytes(N, H, L, Dp, Fp), 256));
         const Operand *in[3] = {&sc.a, &sc.b, &sc.v};
         const int target[3] = {Dp, Dp, Fp};
@@ -228,12 +248,24 @@ int padded_scans(const ScanDesc *scans, int n, const bool *take, int64_t N, int6
     ws_scan = std::max<int64_t>(ws_scan, FTC_WORKSPACE_CONTROL_BYTES);
     int64_t need = ws_scan;
     for (int i = 0; i < ncopies; i++) need += round_up(rows * copies[i].padded * esz(copies[i].dtype), 256);
+    for (int i = 0; i < nstates; i++) {
+        if (N * H * states[i].Dp * states[i].Fp >= 0x7fffffffLL) return FTC_OK;  // (fill kernel: 32-bit count)
+        need += round_up(N * H * states[i].Dp * states[i].Fp * 4, 256);
+    }
     if (!plan_only() && (!workspace || (int64_t)workspace_bytes < need || (uintptr_t)workspace % 256 != 0))
         return FTC_OK;
     char *base = (char *)workspace + ws_scan;
     for (int i = 0; i < ncopies; i++) {
         copies[i].dense = base;
         base += round_up(rows * copies[i].padded * esz(copies[i].dtype), 256);
+    }
+    for (int i = 0; i < nstates; i++) {
+        StateCopy &st = states[i];
+        st.dense = base;
+        base += round_up(N * H * st.Dp * st.Fp * 4, 256);
+        const StateRef dense_ref{(float *)st.dense, H * (int64_t)st.Dp * st.Fp, (int64_t)st.Dp * st.Fp,
+                                 (int64_t)st.Fp};
+        (st.is_output ? work[st.scan].final_ : work[st.scan].initial) = dense_ref;
     }
     for (int s = 0; s < nwork; s++) {
         Operand *in[3] = {&work[s].a, &work[s].b, &work[s].v};
@@ -261,6 +293,15 @@ int padded_scans(const ScanDesc *scans, int n, const bool *take, int64_t N, int6
                 launch_pad_rows<true>((void *)copies[i].ptr, copies[i].sn, copies[i].sh, copies[i].sl,
                                       N, H, L, copies[i].width, copies[i].padded,
                                       esz(copies[i].dtype), copies[i].dense, stream);
+        for (int i = 0; i < nstates; i++) {
+            const StateCopy &st = states[i];
+            if (st.is_output) continue;
+            // zeros first (the rows beyond D are not written by the copy), then the D x F part
+            hipLaunchKernelGGL(zero_words_kernel, dim3(256), dim3(256), 0, stream, (uint32_t *)st.dense,
+                               (uint32_t)(N * H * st.Dp * st.Fp));
+            launch_pad_rows<true>((void *)st.ref.ptr, st.ref.stride_n, st.ref.stride_h, st.ref.stride_d,
+                                  N, H, st.D, st.F, st.Fp, 4, st.dense, stream, st.Dp);
+        }
     }
     int rc = run_scans(work, nwork, N, H, L, workspace, (size_t)ws_scan, stream, false);
     if (rc) return rc;
@@ -270,6 +311,13 @@ int padded_scans(const ScanDesc *scans, int n, const bool *take, int64_t N, int6
                 launch_pad_rows<false>((void *)copies[i].ptr, copies[i].sn, copies[i].sh, copies[i].sl,
                                        N, H, L, copies[i].width, copies[i].padded,
                                        esz(copies[i].dtype), copies[i].dense, stream);
+        for (int i = 0; i < nstates; i++) {
+            const StateCopy &st = states[i];
+            if (st.is_output)
+                launch_pad_rows<false>((void *)st.ref.ptr, st.ref.stride_n, st.ref.stride_h,
+                                       st.ref.stride_d, N, H, st.D, st.F, st.Fp, 4, st.dense, stream,
+                                       st.Dp);
+        }
         hipError_t err = hipGetLastError();
         if (err != hipSuccess)
             return fail(FTC_ERR_HIP, "padding launch failed: %s", hipGetErrorString(err));
@@ -282,7 +330,7 @@ int padded_scans(const ScanDesc *scans, int n, const bool *take, int64_t N, int6
 bool pad_eligible(const ScanDesc &sc, int64_t rows) {
     int widths[kMfmaMaxSlices];
     const int Dp = padded_rows(sc.a.width);
-    if (sc.initial.ptr || sc.final_.ptr || Dp == 0 || rows < kPadMinRows) return false;
+    if (Dp == 0 || rows < kPadMinRows) return false;
     if (const char *env = getenv("FTC_PAD"))  // tuning aid
         if (atoi(env) == 0) return false;
     return mfma_slice_widths(Dp, round_up(sc.v.width, 32), widths) > 0;
