@@ -39,9 +39,9 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 matrix, published
 # carries it only while the sources are unchanged, otherwise null.
 MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {
     # workload: (bytes, kernel source hash at the time of the measurement)
-    "cfg2": (137328454, "a99269205501b99a"),
-    "cfg3": (3140108459, "a99269205501b99a"),
-    "wide": (1877023479, "a99269205501b99a"),
+    "cfg2": (137166199, "cd44218d8e9cc022"),
+    "cfg3": (3135362736, "cd44218d8e9cc022"),
+    "wide": (1877448239, "cd44218d8e9cc022"),
 }
 
 WORKLOADS = {
