@@ -273,6 +273,55 @@ def test_full_config5_size_properties(cp):
         assert s <= 2e-2, key
 
 
+def test_wide_states_at_a_large_size_properties(cp):
+    """128 x 128 and 100 x 68 states at N=8, H=16, L=4096 (the chain-parallel kernel's wide
+    form: two blocks of state rows, a workgroup per block of 64 columns, clipped widths; 768
+    workgroups in the backward): prefix property and linearity over all chains, two chains
+    against the CPU checker."""
+    from fast_transformers_amd import _native
+    N, H, L = 8, 16, 4096
+    for E, M in ((128, 128), (100, 68)):
+        Q, K, V, G = oracle.make_inputs(N, H, L, E, M, seed=600 + E)
+        q, k, v, g = (t.cuda() for t in (Q, K, V, G))
+
+        def fwd(q_, k_, v_):
+            o = torch.empty(q_.shape[:3] + (v_.shape[3],), device="cuda")
+            cp.causal_dot_product_hip(q_, k_, v_, o)
+            return o
+
+        def bwd(g_):
+            outs = [torch.empty_like(t) for t in (q, k, v)]
+            cp.causal_dot_backward_hip(q, k, v, g_, *outs)
+            return outs
+
+        out = fwd(q, k, v)
+        assert _native.load().ftc_last_kernel() == b"scan_tp_kernel"
+        assert torch.isfinite(out).all()
+        Lp = L // 2 + 13   # (another cut of the chains: not bit for bit, but to rounding)
+        outp = fwd(q[:, :, :Lp], k[:, :, :Lp], v[:, :, :Lp])
+        assert scale_error(outp.cpu(), out[:, :, :Lp].cpu()) <= 1e-5
+        V2 = torch.randn(N, H, L, M, generator=torch.Generator().manual_seed(61)).cuda()
+        err = scale_error(fwd(q, k, v + 0.37 * V2).cpu(), (out + 0.37 * fwd(q, k, V2)).cpu())
+        print("wide %dx%d product linear in V: %.3e" % (E, M, err), flush=True)
+        assert err <= 1e-5
+        grads = bwd(g)
+        assert _native.load().ftc_last_kernel() == b"scan_tp_kernel"
+        G2 = torch.randn(N, H, L, M, generator=torch.Generator().manual_seed(62)).cuda()
+        errs = _linear_in(bwd, g, G2)
+        print("wide %dx%d dQ, dK, dV linear in G: %.3e %.3e %.3e" % ((E, M) + tuple(errs)), flush=True)
+        assert max(errs) <= 1e-5
+        sl = (slice(5, 6), slice(3, 5))
+        cut = lambda t: t[sl].cpu().contiguous()
+        s, _ = report("wide chains (5,3-4) product", out[sl].cpu(), oracle.forward(cut(q), cut(k), cut(v)))
+        assert s <= 1e-5
+        for key, got, ref in zip(("dQ", "dK", "dV"), grads,
+                                 oracle.backward(cut(q), cut(k), cut(v), cut(g))):
+            s, _ = report("wide chains (5,3-4) " + key, got[sl].cpu(), ref)
+            assert s <= 1e-5, key
+        del out, outp, grads, q, k, v, g, V2, G2
+        torch.cuda.empty_cache()
+
+
 def test_config4_operator_shape_through_nlhe_strides(cp):
     """The operator as the config-4 encoder calls it: N=10, H=8, L=4096, E=M=64, with Q, K, V
     and the product living in (N, L, H, X) storage and seen as (N, H, L, X) views.  Prefix
