@@ -152,8 +152,105 @@ void launch_pad_rows(void *strided, int64_t sn, int64_t sh, int64_t sl, int64_t 
 constexpr int64_t kPadMinRows = 512;
 int64_t round_up(int64_t x, int64_t m) { return (x + m - 1) / m * m; }
 __global__ void zero_words_kernel(uint32_t *p, uint32_t words);
+
+// ---- states of 129 .. 256 rows: two scans over a split of the rows ------------------------
+//
+// out_l = sum_d a[l, d] (sum_{j <= l} b[j, d] v[j, :]) is a sum over d: a scan whose a and b
+// are wider than the 128 columns that the chain-parallel kernel takes is run as two scans, on
+// columns 0 .. 127 and on the rest, the second one into a buffer in the workspace that is then
+// added to the first one's rows (add_rows_kernel).  fp32 rows, widths multiples of 4.
+bool split_widths(int64_t D, int64_t F) {
+    if (const char *env = getenv("FTC_SPLIT"))  // tuning aid
+        if (atoi(env) == 0) return false;
+    return D > 128 && D <= 256 && F >= 4 && F <= 256 && D % 4 == 0 && F % 4 == 0;
+}
+
+// rows of a strided fp32 tensor of width w (a multiple of 4, rows 16-byte aligned) += rows of a
+// dense one, chain after chain; blockIdx.y walks the chains
+__global__ __launch_bounds__(256) void add_rows_kernel(float *strided, int64_t sn, int64_t sh,
+                                                       int64_t sl, int64_t H, int64_t L,
+                                                       int64_t chains, int w, const float *dense) {
+    typedef float Vec __attribute__((ext_vector_type(4)));
+    const uint32_t groups = (uint32_t)w / 4;
+    const uint32_t j = blockIdx.x * 256u + threadIdx.x;
+    if (j >= (uint32_t)L * groups) return;
+    const uint32_t l = j / groups, c0 = (j % groups) * 4;
+    for (int64_t chain = blockIdx.y; chain < chains; chain += gridDim.y) {
+        Vec *row = (Vec *)(strided + (chain / H) * sn + (chain % H) * sh + (int64_t)l * sl + c0);
+        *row += *(const Vec *)(dense + (chain * L + l) * w + c0);
+    }
+}
+
+// workspace of the two launches of a split (the larger of the two) and of the buffers of the
+// second halves of up to kMfmaMaxScans scans
+int64_t split_scan_workspace_bytes(int64_t N, int64_t H, int64_t L, int64_t D, int64_t F,
+                                   int64_t *launch_bytes) {
+    int64_t ws = FTC_WORKSPACE_CONTROL_BYTES;
+    for (int k = 1; k <= kMfmaMaxScans; k++) {
+        ws = std::max(ws, mfma_tp_workspace_bytes(N, H, L, 128, F, k, true));
+        ws = std::max(ws, mfma_tp_workspace_bytes(N, H, L, D - 128, F, k, true));
+    }
+    ws = round_up(ws, 256);
+    if (launch_bytes) *launch_bytes = ws;
+    return ws + kMfmaMaxScans * round_up(N * H * L * F * 4, 256);
+}
+
+int run_scans(const ScanDesc *scans, int n, int64_t N, int64_t H, int64_t L, void *workspace,
+              size_t workspace_bytes, hipStream_t stream, bool may_pad);
+
+// Runs scans[0 .. n) of one shape (split_widths) as described above.  *done = false (nothing
+// launched) when the chain-parallel kernel does not take the halves or the workspace has no room.
+int split_scans(const ScanDesc *scans, int n, int64_t N, int64_t H, int64_t L, void *workspace,
+                size_t workspace_bytes, hipStream_t stream, bool *done) {
+    *done = false;
+    const int D = scans[0].a.width, F = scans[0].v.width;
+    const int64_t rows = N * H * L, tmp_bytes = round_up(rows * F * 4, 256);
+    int64_t ws_launch = 0;
+    split_scan_workspace_bytes(N, H, L, D, F, &ws_launch);
+    const int64_t need = ws_launch + n * tmp_bytes;
+    ScanDesc lo[kMfmaMaxScans], hi[kMfmaMaxScans];
+    for (int i = 0; i < n; i++) {
+        lo[i] = hi[i] = scans[i];
+        lo[i].a.width = lo[i].b.width = 128;
+        hi[i].a.width = hi[i].b.width = D - 128;
+        hi[i].a.ptr = (const char *)scans[i].a.ptr + 128 * 4;
+        hi[i].b.ptr = (const char *)scans[i].b.ptr + 128 * 4;
+        if (hi[i].initial.ptr) hi[i].initial.ptr += 128 * hi[i].initial.stride_d;
+        if (hi[i].final_.ptr) hi[i].final_.ptr += 128 * hi[i].final_.stride_d;
+        hi[i].out = OperandOut{(char *)workspace + ws_launch + i * tmp_bytes, H * L * (int64_t)F,
+                               L * (int64_t)F, (int64_t)F, FTC_F32, (int32_t)F};
+    }
+    if (!mfma_tp_takes(lo, n, N, H, L, true) || !mfma_tp_takes(hi, n, N, H, L, true)) return FTC_OK;
+    if (!plan_only() && (!workspace || (int64_t)workspace_bytes < need || (uintptr_t)workspace % 256 != 0))
+        return FTC_OK;
+    int rc = mfma_scan(lo, n, N, H, L, workspace, (size_t)ws_launch, stream, nullptr, true, true);
+    if (rc) return rc;
+    rc = mfma_scan(hi, n, N, H, L, workspace, (size_t)ws_launch, stream, nullptr, true, true);
+    if (rc) return rc;
+    if (plan_only()) {
+        note_plan("add_rows_kernel: %d result%s of the second halves added to the first, workspace %lld bytes",
+                  n, n == 1 ? "" : "s", (long long)need);
+    } else {
+        const dim3 grid((unsigned)((L * (F / 4) + 255) / 256), (unsigned)std::min<int64_t>(N * H, 65535));
+        for (int i = 0; i < n; i++)
+            hipLaunchKernelGGL(add_rows_kernel, grid, dim3(256), 0, stream, (float *)scans[i].out.ptr,
+                               scans[i].out.stride_n, scans[i].out.stride_h, scans[i].out.stride_l, H, L,
+                               N * H, F, (const float *)hi[i].out.ptr);
+        const hipError_t err = hipGetLastError();
+        if (err != hipSuccess) return fail(FTC_ERR_HIP, "add launch failed: %s", hipGetErrorString(err));
+    }
+    *done = true;
+    return FTC_OK;
+}
 // padded widths of a D x F scan (0: the matrix-core kernels take no such state)
-int padded_rows(int64_t D) { return D <= 32 ? 32 : D <= 64 ? 64 : D <= 96 ? 96 : D <= 128 ? 128 : 0; }
+// (129 .. 256: for the split above; multiples of 32 like the output widths, so that a tensor
+// that is state rows in one scan and output columns in another needs one copy)
+int padded_rows(int64_t D) { return D <= 256 ? (int)round_up(D, 32) : 0; }
+// whether the matrix-core kernels take a padded D x F state
+bool padded_shape_ok(int64_t Dp, int64_t Fp) {
+    int widths[kMfmaMaxSlices];
+    return Fp <= 256 && (split_widths(Dp, Fp) || (Dp <= 128 && mfma_slice_widths(Dp, Fp, widths) > 0));
+}
 
 int64_t scan_workspace_bytes(int64_t N, int64_t H, int64_t L, int64_t D, int64_t F,
                              bool with_pad = true);
@@ -162,10 +259,7 @@ int64_t scan_workspace_bytes(int64_t N, int64_t H, int64_t L, int64_t D, int64_t
 // operands (fp32 sizes: an upper bound)
 int64_t padded_scan_workspace_bytes(int64_t N, int64_t H, int64_t L, int64_t D, int64_t F) {
     const int64_t Dp = padded_rows(D), Fp = round_up(F, 32), rows = N * H * L;
-    int widths[kMfmaMaxSlices];
-    if (Dp == 0 || (Dp == D && Fp == F) || rows < kPadMinRows ||
-        mfma_slice_widths(Dp, Fp, widths) == 0)
-        return 0;
+    if (Dp == 0 || (Dp == D && Fp == F) || rows < kPadMinRows || !padded_shape_ok(Dp, Fp)) return 0;
     return std::max<int64_t>(round_up(scan_workspace_bytes(N, H, L, Dp, Fp), 256),
                              FTC_WORKSPACE_CONTROL_BYTES) +
            2 * round_up(rows * Dp * 4, 256) + 2 * round_up(rows * Fp * 4, 256) +
@@ -328,12 +422,15 @@ int padded_scans(const ScanDesc *scans, int n, const bool *take, int64_t N, int6
 
 // whether a scan that the matrix-core kernels do not take as it is may go the padded way
 bool pad_eligible(const ScanDesc &sc, int64_t rows) {
-    int widths[kMfmaMaxSlices];
     const int Dp = padded_rows(sc.a.width);
     if (Dp == 0 || rows < kPadMinRows) return false;
     if (const char *env = getenv("FTC_PAD"))  // tuning aid
         if (atoi(env) == 0) return false;
-    return mfma_slice_widths(Dp, round_up(sc.v.width, 32), widths) > 0;
+    // (the split of states beyond 128 rows is for fp32 rows only)
+    if (Dp > 128 && !(sc.a.dtype == FTC_F32 && sc.b.dtype == FTC_F32 && sc.v.dtype == FTC_F32 &&
+                      sc.out.dtype == FTC_F32))
+        return false;
+    return padded_shape_ok(Dp, round_up(sc.v.width, 32));
 }
 
 // Runs a list of independent scans.  A scan whose shape the MFMA kernels cover is cut into
@@ -355,6 +452,13 @@ int run_scans(const ScanDesc *scans, int n, int64_t N, int64_t H, int64_t L, voi
         for (int j = i; j < n; j++)
             if (!offered[j] && scans[j].a.width == scans[i].a.width && scans[j].v.width == scans[i].v.width)
                 offered[j] = true, members[ngroup] = j, group[ngroup++] = scans[j];
+        if (split_widths(group[0].a.width, group[0].v.width)) {
+            bool done = false;
+            const int rc = split_scans(group, ngroup, N, H, L, workspace, workspace_bytes, stream, &done);
+            if (rc) return rc;
+            for (int k = 0; k < ngroup && done; k++) taken[members[k]] = true;
+            continue;
+        }
         if (!mfma_tp_takes(group, ngroup, N, H, L)) continue;
         const int rc = mfma_scan(group, ngroup, N, H, L, workspace, workspace_bytes, stream);
         if (rc) return rc;
@@ -425,6 +529,7 @@ int64_t scan_workspace_bytes(int64_t N, int64_t H, int64_t L, int64_t D, int64_t
     if (nslices == 0 && with_pad) need = std::max(need, padded_scan_workspace_bytes(N, H, L, D, F));
     for (int k = 1; k <= kMfmaMaxScans; k++)
         need = std::max(need, mfma_tp_workspace_bytes(N, H, L, D, F, k));
+    if (split_widths(D, F)) need = std::max(need, split_scan_workspace_bytes(N, H, L, D, F, nullptr));
     return need;
 }
 

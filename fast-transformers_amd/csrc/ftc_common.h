@@ -123,8 +123,12 @@ int64_t mfma_scan_workspace_bytes(int64_t N, int64_t H, int64_t L, int64_t D, in
 // columns, widths multiples of 4 (also widths that mfma_scan_supported
 // does not list).  True when mfma_scan would run these scans, side by side, on that kernel;
 // its workspace (part of mfma_scan_workspace_bytes where both apply).
-bool mfma_tp_takes(const ScanDesc *scans, int nscans, int64_t N, int64_t H, int64_t L);
-int64_t mfma_tp_workspace_bytes(int64_t N, int64_t H, int64_t L, int64_t D, int64_t F, int nscans);
+// `forced`: these scans are parts of scans that the caller has split by state rows because
+// only this kernel can take them (any multiple of 4 will do, at any size).
+bool mfma_tp_takes(const ScanDesc *scans, int nscans, int64_t N, int64_t H, int64_t L,
+                   bool forced = false);
+int64_t mfma_tp_workspace_bytes(int64_t N, int64_t H, int64_t L, int64_t D, int64_t F, int nscans,
+                                bool forced = false);
 // The fused attention form of a forward scan: a and b go through the feature map
 // elu(x) + 1, rows of b at or beyond key_lengths[n] count as zero, and every output row is
 // divided by (phi(a_l) . sum_{j <= l} phi(b_j) + eps).
@@ -139,7 +143,8 @@ int64_t fused_attention_workspace_bytes(int64_t N, int64_t H, int64_t L, int64_t
 // off the chain-parallel kernel (column slices of a scan that it has declined as a whole).
 int mfma_scan(const ScanDesc *scans, int nscans, int64_t N, int64_t H, int64_t L,
               void *workspace, size_t workspace_bytes, hipStream_t stream,
-              const FusedAttention *fused = nullptr, bool may_chain_parallel = true);
+              const FusedAttention *fused = nullptr, bool may_chain_parallel = true,
+              bool forced = false);
 
 // Fill every row of `out` with zeros (used for empty contractions).
 int zero_rows(const OperandOut &out, int64_t N, int64_t H, int64_t L, hipStream_t stream);

@@ -27,8 +27,11 @@ bool use_wg_kernel(int64_t D, int64_t F, int nscans, int64_t L, bool all_f32) {
 // Row widths that the chain-parallel kernel takes (ftc_tp_kernel.h): states of 16 x 16 to
 // 128 x 128, walked in blocks of 64 rows, with one workgroup per block of 64 output columns;
 // widths that are multiples of 4 (a lane's 16 bytes lie wholly inside a row or wholly outside).
-bool tp_widths(int64_t D, int64_t F) {
-    return D >= 16 && D <= 128 && F >= 16 && F <= 128 && D % 4 == 0 && F % 4 == 0;
+// (`forced`: a part of a scan that the caller has split because only this kernel takes it;
+// then any multiple of 4 will do)
+bool tp_widths(int64_t D, int64_t F, bool forced = false) {
+    const int64_t least = forced ? 4 : 16;
+    return D >= least && D <= 128 && F >= least && F <= 256 && D % 4 == 0 && F % 4 == 0;
 }
 int64_t tp_fblocks(int64_t F) { return (F + 63) / 64; }
 
@@ -155,11 +158,12 @@ int tp_exchange_segments(int64_t units, int64_t L, bool wide, int *nseg) {
 // The chain-parallel kernel's plan for `nscans` scans of a D x F state over chains x L rows:
 // *seg_chunks > 0: an exchange with *nseg segments of that many chunks; else *nseg > 0: chains
 // cut into *nseg segments that need no exchange; both 0: another kernel takes the launch.
-void tp_plan(int64_t D, int64_t F, int64_t chains, int nscans, int64_t L, int *nseg, int *seg_chunks) {
+void tp_plan(int64_t D, int64_t F, int64_t chains, int nscans, int64_t L, int *nseg, int *seg_chunks,
+             bool forced = false) {
     *nseg = *seg_chunks = 0;
-    if (!tp_widths(D, F)) return;
-    const bool wide = D != 64 || F != 64;
-    const bool others = mfma_scan_supported_widths(D, F);
+    if (!tp_widths(D, F, forced)) return;
+    const bool wide = D != 64 || F != 64 || forced;
+    const bool others = !forced && mfma_scan_supported_widths(D, F);
     const int64_t units = chains * nscans * tp_fblocks(F);
     // Shapes of the other kernels with 32 rows or columns (a workgroup here has half of its
     // matrix work or half of its consumers to spare for them): measured at N=8, H=16, L=4096,
@@ -173,7 +177,7 @@ void tp_plan(int64_t D, int64_t F, int64_t chains, int nscans, int64_t L, int *n
     // against 0.60 ms, 20 x 20 0.63 against 0.46 on padded copies), and 32-wide shapes on more
     // than two rounds of workgroups, as for 64 x 64.
     if (narrow && units > 512) return;
-    if (D <= 64 && F <= 64 && units > 512 && L <= 2 * kChunk) return;
+    if (!forced && D <= 64 && F <= 64 && units > 512 && L <= 2 * kChunk) return;
     if (!narrow) *seg_chunks = tp_exchange_segments(units, L, wide, nseg);
     if (*seg_chunks == 0) *nseg = tp_kernel_segments(units, L, wide, others);
 }
@@ -320,16 +324,17 @@ int64_t mfma_scan_workspace_bytes(int64_t N, int64_t H, int64_t L, int64_t D, in
     return std::max(bytes, mfma_tp_workspace_bytes(N, H, L, D, F, nscans));
 }
 
-int64_t mfma_tp_workspace_bytes(int64_t N, int64_t H, int64_t L, int64_t D, int64_t F, int nscans) {
+int64_t mfma_tp_workspace_bytes(int64_t N, int64_t H, int64_t L, int64_t D, int64_t F, int nscans,
+                                bool forced) {
     int nseg = 0, seg_chunks = 0;
     const int64_t chains = std::max<int64_t>(1, N * H);
-    tp_plan(D, F, chains, nscans, L, &nseg, &seg_chunks);
+    tp_plan(D, F, chains, nscans, L, &nseg, &seg_chunks, forced);
     return seg_chunks > 0 ? tp_exchange_workspace_bytes(chains * nscans * tp_fblocks(F), nseg, D) : 0;
 }
 
-bool mfma_tp_takes(const ScanDesc *scans, int nscans, int64_t N, int64_t H, int64_t L) {
+bool mfma_tp_takes(const ScanDesc *scans, int nscans, int64_t N, int64_t H, int64_t L, bool forced) {
     const int D = scans[0].a.width, F = scans[0].v.width;
-    if (nscans < 1 || nscans > kMaxScans || !tp_widths(D, F)) return false;
+    if (nscans < 1 || nscans > kMaxScans || !tp_widths(D, F, forced)) return false;
     int64_t widest_stride = 0;
     for (int i = 0; i < nscans; i++) {
         const ScanDesc &sd = scans[i];
@@ -349,7 +354,7 @@ bool mfma_tp_takes(const ScanDesc *scans, int nscans, int64_t N, int64_t H, int6
     if ((L + 2 * kChunk) * std::max<int64_t>(widest_stride, std::max(D, F)) * 4 >= 0x7fffffffLL)
         return false;
     int nseg = 0, seg_chunks = 0;
-    tp_plan(D, F, std::max<int64_t>(1, N * H), nscans, L, &nseg, &seg_chunks);
+    tp_plan(D, F, std::max<int64_t>(1, N * H), nscans, L, &nseg, &seg_chunks, forced);
     return nseg > 0;
 }
 
@@ -364,18 +369,18 @@ int64_t fused_attention_workspace_bytes(int64_t N, int64_t H, int64_t L, int64_t
 
 int mfma_scan(const ScanDesc *scans, int nscans, int64_t N, int64_t H, int64_t L,
               void *workspace, size_t workspace_bytes, hipStream_t stream,
-              const FusedAttention *fused, bool may_chain_parallel) {
+              const FusedAttention *fused, bool may_chain_parallel, bool forced) {
     if (nscans < 1 || nscans > kMaxScans) return fail(FTC_ERR_INVALID, "bad scan count");
     const int D = scans[0].a.width, F = scans[0].v.width;
     const Combo combo = combo_of(scans[0]);
     if (fused && (nscans != 1 || !fused_attention_supported(scans[0], L)))
         return fail(FTC_ERR_UNSUPPORTED, "no fused attention kernel for this shape or layout");
-    const bool tp_shape = !fused && may_chain_parallel && mfma_tp_takes(scans, nscans, N, H, L);
+    const bool tp_shape = !fused && may_chain_parallel && mfma_tp_takes(scans, nscans, N, H, L, forced);
     const int64_t chains = std::max<int64_t>(1, N * H);
     const int64_t fblocks = tp_shape ? tp_fblocks(F) : 1;
     int tpx_nseg = 0, tpx_seg_chunks = 0, tp_nseg = 0;
     if (tp_shape) {
-        tp_plan(D, F, chains, nscans, L, &tpx_nseg, &tpx_seg_chunks);
+        tp_plan(D, F, chains, nscans, L, &tpx_nseg, &tpx_seg_chunks, forced);
         if (tpx_seg_chunks == 0) tp_nseg = tpx_nseg, tpx_nseg = 0;
     }
     const bool tp = tp_nseg > 0 || tpx_seg_chunks > 0;

@@ -547,6 +547,10 @@ STATE_SHAPES = {
     # neither read nor written
     "tp_e100_m72": (8, 8, 700, 100, 72, 60, torch.float32),
     "tp_long_e128_m128": (1, 8, 5000, 128, 128, 61, torch.float32),
+    # more than 128 state rows: two scans over a split of the rows, each with its rows of
+    # the state
+    "split_e160_m72": (4, 8, 600, 160, 72, 62, torch.float32),
+    "split_e255_m33": (2, 4, 900, 255, 33, 63, torch.float32),
     "e32_m128": (2, 3, 700, 32, 128, 53, torch.float32),
     # register-fed kernel, column slices
     "e128_m128": (1, 3, 500, 128, 128, 54, torch.float32),
@@ -822,7 +826,12 @@ ODD_SHAPES = [
     (3, 3, 1000, 10, 3, torch.float32),      # tiny widths
     (1, 2, 5000, 70, 33, torch.float32),     # 96-row state one way, 64-row state the other
     (2, 4, 1200, 48, 80, torch.bfloat16),    # bf16 rows
-    (1, 4, 2500, 130, 40, torch.float32),    # E beyond 128: dV stays on the generic kernel
+    (1, 4, 2500, 130, 40, torch.float32),    # E beyond 128: two scans over a split of the state rows
+    (2, 4, 700, 255, 129, torch.float32),    # ... on padded copies, both ways
+    (4, 8, 300, 200, 200, torch.float32),    # ... where the rows lie (multiples of 4)
+    (10, 10, 100, 250, 17, torch.float32),   # the reference's own test sizes
+    (2, 4, 600, 132, 36, torch.float32),     # a second part of four rows
+    (1, 4, 1000, 160, 40, torch.bfloat16),   # bf16 rows beyond 128: the generic kernel
     # many short chains: the scans on the copies need no workspace of their own, and the
     # copies must still keep off the control block
     (33, 12, 64, 48, 33, torch.float32),
@@ -842,8 +851,8 @@ def test_odd_widths_run_on_padded_copies(cp, shape):
     q, k, v, g = (nlh(t) for t in (Q, K, V, G))
     out = torch.full((N, L, H, M), float("nan"), device="cuda").permute(0, 2, 1, 3)
     cp.causal_dot_product_hip(q, k, v, out)
-    if E <= 128:
-        assert _native.load().ftc_last_kernel() != b"generic_scan_kernel"
+    on_matrix_cores = E <= 128 or (dtype == torch.float32 and E <= 256 and M <= 256)
+    assert (_native.load().ftc_last_kernel() != b"generic_scan_kernel") == on_matrix_cores
     dq, dk, dv = (torch.full((N, L, H, X), float("nan"), device="cuda", dtype=dtype).permute(0, 2, 1, 3)
                   for X in (E, E, M))
     cp.causal_dot_backward_hip(q, k, v, g, dq, dk, dv)

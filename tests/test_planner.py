@@ -79,7 +79,18 @@ def test_what_the_chain_parallel_kernel_leaves_to_the_others():
     assert wide[0].startswith("pad_rows_kernel: 4 operands") and "3 results" in wide[0]
     assert wide[1].startswith("scan_tp_kernel: 3 scans") and "state 128 x 128" in wide[1]
     assert lines((2, 2, 40, 10), (2, 2, 40, 3))[0].startswith("generic_scan_kernel")
-    assert lines((1, 2, 8192, 200), (1, 2, 8192, 64))[0].startswith("generic_scan_kernel")
+    assert lines((1, 2, 8192, 300), (1, 2, 8192, 64))[0].startswith("generic_scan_kernel")
+    # states of 129 to 256 rows: two scans over a split of the rows, the second one's rows
+    # added to the first one's
+    two = lines((1, 2, 8192, 200), (1, 2, 8192, 64))
+    assert "state 128 x 64" in two[0] and "state 72 x 64" in two[1] and two[2].startswith("add_rows_kernel: 1 result")
+    two = lines((4, 8, 1000, 200), (4, 8, 1000, 200), backward=True)
+    assert two[0].startswith("scan_tp_kernel: 3 scans") and "state 128 x 200" in two[0]
+    assert "state 72 x 200" in two[1] and two[2].startswith("add_rows_kernel: 3 results")
+    odd = lines((2, 4, 700, 255), (2, 4, 700, 129))
+    assert odd[0].startswith("pad_rows_kernel: 3 operands") and "state 128 x 160" in odd[1]
+    odd = lines((2, 4, 700, 255), (2, 4, 700, 129), backward=True)
+    assert odd[0].startswith("pad_rows_kernel: 4 operands") and "3 results" in odd[0]
     # nothing to do
     assert lines((0, 8, 100, 64), (0, 8, 100, 64)) == []
 
@@ -145,7 +156,7 @@ def test_wide_states_on_the_chain_parallel_kernel():
 
 
 SWEEP = [(N, H, L, E, M) for (N, H) in [(1, 1), (1, 16), (2, 8), (10, 8), (64, 16)]
-         for L in [1, 64, 1000, 4096, 20000] for (E, M) in [(64, 64), (32, 128), (96, 64), (25, 70), (128, 128), (100, 36)]]
+         for L in [1, 64, 1000, 4096, 20000] for (E, M) in [(64, 64), (32, 128), (96, 64), (25, 70), (128, 128), (100, 36), (200, 64), (255, 129)]]
 
 
 @pytest.mark.parametrize("backward", [False, True])
