@@ -39,9 +39,9 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 matrix, published
 # carries it only while the sources are unchanged, otherwise null.
 MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {
     # workload: (bytes, kernel source hash at the time of the measurement)
-    "cfg2": (137166199, "cd44218d8e9cc022"),
-    "cfg3": (3135362736, "cd44218d8e9cc022"),
-    "wide": (1877448239, "cd44218d8e9cc022"),
+    "cfg2": (137381497, "fa1332bb6ad7d504"),
+    "cfg3": (3141841000, "fa1332bb6ad7d504"),
+    "wide": (1877425462, "fa1332bb6ad7d504"),
 }
 
 WORKLOADS = {

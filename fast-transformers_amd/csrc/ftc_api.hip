@@ -517,8 +517,8 @@ int run_scans(const ScanDesc *scans, int n, int64_t N, int64_t H, int64_t L, voi
 }
 
 // Upper bound over every way run_scans may slice and group scans of these widths.
-// `with_pad` = false leaves out the padded copies: what a call needs at the least (without
-// them such a scan runs on the generic kernel).
+// `with_pad` = false leaves out the padded copies and the buffers of split scans: what a call
+// needs at the least (without them such a scan runs on the generic kernel).
 int64_t scan_workspace_bytes(int64_t N, int64_t H, int64_t L, int64_t D, int64_t F, bool with_pad) {
     int64_t need = generic_scan_workspace_bytes(N, H, L, D, F);
     int widths[kMfmaMaxSlices];
@@ -529,7 +529,8 @@ int64_t scan_workspace_bytes(int64_t N, int64_t H, int64_t L, int64_t D, int64_t
     if (nslices == 0 && with_pad) need = std::max(need, padded_scan_workspace_bytes(N, H, L, D, F));
     for (int k = 1; k <= kMfmaMaxScans; k++)
         need = std::max(need, mfma_tp_workspace_bytes(N, H, L, D, F, k));
-    if (split_widths(D, F)) need = std::max(need, split_scan_workspace_bytes(N, H, L, D, F, nullptr));
+    if (with_pad && split_widths(D, F))
+        need = std::max(need, split_scan_workspace_bytes(N, H, L, D, F, nullptr));
     return need;
 }
 
