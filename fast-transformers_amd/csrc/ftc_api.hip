@@ -153,16 +153,17 @@ constexpr int64_t kPadMinRows = 512;
 int64_t round_up(int64_t x, int64_t m) { return (x + m - 1) / m * m; }
 __global__ void zero_words_kernel(uint32_t *p, uint32_t words);
 
-// ---- states of 129 .. 256 rows: two scans over a split of the rows ------------------------
+// ---- states of 129 .. 512 rows: several scans over a split of the rows --------------------
 //
 // out_l = sum_d a[l, d] (sum_{j <= l} b[j, d] v[j, :]) is a sum over d: a scan whose a and b
-// are wider than the 128 columns that the chain-parallel kernel takes is run as two scans, on
-// columns 0 .. 127 and on the rest, the second one into a buffer in the workspace that is then
-// added to the first one's rows (add_rows_kernel).  fp32 rows, widths multiples of 4.
+// are wider than the 128 columns that the chain-parallel kernel takes is run as up to four
+// scans, on columns 0 .. 127, 128 .. 255 and so on, all but the first one into a buffer in the
+// workspace that is then added to the first one's rows (add_rows_kernel).  fp32 rows, widths
+// multiples of 4.
 bool split_widths(int64_t D, int64_t F) {
     if (const char *env = getenv("FTC_SPLIT"))  // tuning aid
         if (atoi(env) == 0) return false;
-    return D > 128 && D <= 256 && F >= 4 && F <= 256 && D % 4 == 0 && F % 4 == 0;
+    return D > 128 && D <= 512 && F >= 4 && F <= 512 && D % 4 == 0 && F % 4 == 0;
 }
 
 // rows of a strided fp32 tensor of width w (a multiple of 4, rows 16-byte aligned) += rows of a
@@ -188,7 +189,7 @@ int64_t split_scan_workspace_bytes(int64_t N, int64_t H, int64_t L, int64_t D, i
     int64_t ws = FTC_WORKSPACE_CONTROL_BYTES;
     for (int k = 1; k <= kMfmaMaxScans; k++) {
         ws = std::max(ws, mfma_tp_workspace_bytes(N, H, L, 128, F, k, true));
-        ws = std::max(ws, mfma_tp_workspace_bytes(N, H, L, D - 128, F, k, true));
+        if (D % 128) ws = std::max(ws, mfma_tp_workspace_bytes(N, H, L, D % 128, F, k, true));
     }
     ws = round_up(ws, 256);
     if (launch_bytes) *launch_bytes = ws;
@@ -208,34 +209,44 @@ int split_scans(const ScanDesc *scans, int n, int64_t N, int64_t H, int64_t L, v
     int64_t ws_launch = 0;
     split_scan_workspace_bytes(N, H, L, D, F, &ws_launch);
     const int64_t need = ws_launch + n * tmp_bytes;
-    ScanDesc lo[kMfmaMaxScans], hi[kMfmaMaxScans];
-    for (int i = 0; i < n; i++) {
-        lo[i] = hi[i] = scans[i];
-        lo[i].a.width = lo[i].b.width = 128;
-        hi[i].a.width = hi[i].b.width = D - 128;
-        hi[i].a.ptr = (const char *)scans[i].a.ptr + 128 * 4;
-        hi[i].b.ptr = (const char *)scans[i].b.ptr + 128 * 4;
-        if (hi[i].initial.ptr) hi[i].initial.ptr += 128 * hi[i].initial.stride_d;
-        if (hi[i].final_.ptr) hi[i].final_.ptr += 128 * hi[i].final_.stride_d;
-        hi[i].out = OperandOut{(char *)workspace + ws_launch + i * tmp_bytes, H * L * (int64_t)F,
-                               L * (int64_t)F, (int64_t)F, FTC_F32, (int32_t)F};
+    // part p: columns 128 p .. of a and b, rows 128 p .. of the states
+    const int nparts = (D + 127) / 128;
+    auto part = [&](int p, ScanDesc (&ps)[kMfmaMaxScans]) {
+        const int w = std::min(128, D - 128 * p);
+        for (int i = 0; i < n; i++) {
+            ps[i] = scans[i];
+            ps[i].a.width = ps[i].b.width = w;
+            ps[i].a.ptr = (const char *)scans[i].a.ptr + 128 * p * 4;
+            ps[i].b.ptr = (const char *)scans[i].b.ptr + 128 * p * 4;
+            if (ps[i].initial.ptr) ps[i].initial.ptr += 128 * p * ps[i].initial.stride_d;
+            if (ps[i].final_.ptr) ps[i].final_.ptr += 128 * p * ps[i].final_.stride_d;
+            if (p > 0)
+                ps[i].out = OperandOut{(char *)workspace + ws_launch + i * tmp_bytes, H * L * (int64_t)F,
+                                       L * (int64_t)F, (int64_t)F, FTC_F32, (int32_t)F};
+        }
+    };
+    ScanDesc ps[kMfmaMaxScans];
+    for (int p = 0; p < nparts; p++) {
+        part(p, ps);
+        if (!mfma_tp_takes(ps, n, N, H, L, true)) return FTC_OK;
     }
-    if (!mfma_tp_takes(lo, n, N, H, L, true) || !mfma_tp_takes(hi, n, N, H, L, true)) return FTC_OK;
     if (!plan_only() && (!workspace || (int64_t)workspace_bytes < need || (uintptr_t)workspace % 256 != 0))
         return FTC_OK;
-    int rc = mfma_scan(lo, n, N, H, L, workspace, (size_t)ws_launch, stream, nullptr, true, true);
-    if (rc) return rc;
-    rc = mfma_scan(hi, n, N, H, L, workspace, (size_t)ws_launch, stream, nullptr, true, true);
-    if (rc) return rc;
-    if (plan_only()) {
-        note_plan("add_rows_kernel: %d result%s of the second halves added to the first, workspace %lld bytes",
-                  n, n == 1 ? "" : "s", (long long)need);
-    } else {
+    for (int p = 0; p < nparts; p++) {
+        part(p, ps);
+        const int rc = mfma_scan(ps, n, N, H, L, workspace, (size_t)ws_launch, stream, nullptr, true, true);
+        if (rc) return rc;
+        if (p == 0) continue;
+        if (plan_only()) {
+            note_plan("add_rows_kernel: %d result%s of part %d added to the first part's, workspace %lld bytes",
+                      n, n == 1 ? "" : "s", p + 1, (long long)need);
+            continue;
+        }
         const dim3 grid((unsigned)((L * (F / 4) + 255) / 256), (unsigned)std::min<int64_t>(N * H, 65535));
         for (int i = 0; i < n; i++)
             hipLaunchKernelGGL(add_rows_kernel, grid, dim3(256), 0, stream, (float *)scans[i].out.ptr,
                                scans[i].out.stride_n, scans[i].out.stride_h, scans[i].out.stride_l, H, L,
-                               N * H, F, (const float *)hi[i].out.ptr);
+                               N * H, F, (const float *)ps[i].out.ptr);
         const hipError_t err = hipGetLastError();
         if (err != hipSuccess) return fail(FTC_ERR_HIP, "add launch failed: %s", hipGetErrorString(err));
     }
@@ -243,13 +254,13 @@ int split_scans(const ScanDesc *scans, int n, int64_t N, int64_t H, int64_t L, v
     return FTC_OK;
 }
 // padded widths of a D x F scan (0: the matrix-core kernels take no such state)
-// (129 .. 256: for the split above; multiples of 32 like the output widths, so that a tensor
+// (129 .. 512: for the split above; multiples of 32 like the output widths, so that a tensor
 // that is state rows in one scan and output columns in another needs one copy)
-int padded_rows(int64_t D) { return D <= 256 ? (int)round_up(D, 32) : 0; }
+int padded_rows(int64_t D) { return D <= 512 ? (int)round_up(D, 32) : 0; }
 // whether the matrix-core kernels take a padded D x F state
 bool padded_shape_ok(int64_t Dp, int64_t Fp) {
     int widths[kMfmaMaxSlices];
-    return Fp <= 256 && (split_widths(Dp, Fp) || (Dp <= 128 && mfma_slice_widths(Dp, Fp, widths) > 0));
+    return Fp <= 512 && (split_widths(Dp, Fp) || (Dp <= 128 && mfma_slice_widths(Dp, Fp, widths) > 0));
 }
 
 int64_t scan_workspace_bytes(int64_t N, int64_t H, int64_t L, int64_t D, int64_t F,

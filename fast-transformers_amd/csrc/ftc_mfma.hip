@@ -31,7 +31,7 @@ bool use_wg_kernel(int64_t D, int64_t F, int nscans, int64_t L, bool all_f32) {
 // then any multiple of 4 will do)
 bool tp_widths(int64_t D, int64_t F, bool forced = false) {
     const int64_t least = forced ? 4 : 16;
-    return D >= least && D <= 128 && F >= least && F <= 256 && D % 4 == 0 && F % 4 == 0;
+    return D >= least && D <= 128 && F >= least && F <= 512 && D % 4 == 0 && F % 4 == 0;
 }
 int64_t tp_fblocks(int64_t F) { return (F + 63) / 64; }
 

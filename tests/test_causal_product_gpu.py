@@ -551,6 +551,7 @@ STATE_SHAPES = {
     # the state
     "split_e160_m72": (4, 8, 600, 160, 72, 62, torch.float32),
     "split_e255_m33": (2, 4, 900, 255, 33, 63, torch.float32),
+    "split_e300_m72": (2, 4, 500, 300, 72, 64, torch.float32),
     "e32_m128": (2, 3, 700, 32, 128, 53, torch.float32),
     # register-fed kernel, column slices
     "e128_m128": (1, 3, 500, 128, 128, 54, torch.float32),
@@ -831,6 +832,7 @@ ODD_SHAPES = [
     (4, 8, 300, 200, 200, torch.float32),    # ... where the rows lie (multiples of 4)
     (10, 10, 100, 250, 17, torch.float32),   # the reference's own test sizes
     (2, 4, 600, 132, 36, torch.float32),     # a second part of four rows
+    (2, 4, 300, 511, 257, torch.float32),    # four parts, five blocks of output columns
     (1, 4, 1000, 160, 40, torch.bfloat16),   # bf16 rows beyond 128: the generic kernel
     # many short chains: the scans on the copies need no workspace of their own, and the
     # copies must still keep off the control block
@@ -851,7 +853,7 @@ def test_odd_widths_run_on_padded_copies(cp, shape):
     q, k, v, g = (nlh(t) for t in (Q, K, V, G))
     out = torch.full((N, L, H, M), float("nan"), device="cuda").permute(0, 2, 1, 3)
     cp.causal_dot_product_hip(q, k, v, out)
-    on_matrix_cores = E <= 128 or (dtype == torch.float32 and E <= 256 and M <= 256)
+    on_matrix_cores = E <= 128 or dtype == torch.float32
     assert (_native.load().ftc_last_kernel() != b"generic_scan_kernel") == on_matrix_cores
     dq, dk, dv = (torch.full((N, L, H, X), float("nan"), device="cuda", dtype=dtype).permute(0, 2, 1, 3)
                   for X in (E, E, M))

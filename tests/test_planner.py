@@ -79,9 +79,14 @@ def test_what_the_chain_parallel_kernel_leaves_to_the_others():
     assert wide[0].startswith("pad_rows_kernel: 4 operands") and "3 results" in wide[0]
     assert wide[1].startswith("scan_tp_kernel: 3 scans") and "state 128 x 128" in wide[1]
     assert lines((2, 2, 40, 10), (2, 2, 40, 3))[0].startswith("generic_scan_kernel")
-    assert lines((1, 2, 8192, 300), (1, 2, 8192, 64))[0].startswith("generic_scan_kernel")
-    # states of 129 to 256 rows: two scans over a split of the rows, the second one's rows
-    # added to the first one's
+    assert lines((1, 2, 8192, 300), (1, 2, 8192, 64), dtype=_native.FTC_BF16)[0] \
+        .startswith("generic_scan_kernel")
+    # states of 129 to 512 rows: up to four scans over a split of the rows, the later ones'
+    # rows added to the first one's
+    three = lines((1, 2, 8192, 300), (1, 2, 8192, 64))
+    assert [l.split(":")[0].split(" ")[0] for l in three] == \
+        ["scan_tp_kernel", "scan_tp_kernel", "add_rows_kernel", "scan_tp_kernel", "add_rows_kernel"]
+    assert "state 128 x 64" in three[0] and "state 128 x 64" in three[1] and "state 44 x 64" in three[3]
     two = lines((1, 2, 8192, 200), (1, 2, 8192, 64))
     assert "state 128 x 64" in two[0] and "state 72 x 64" in two[1] and two[2].startswith("add_rows_kernel: 1 result")
     two = lines((4, 8, 1000, 200), (4, 8, 1000, 200), backward=True)
@@ -156,7 +161,7 @@ def test_wide_states_on_the_chain_parallel_kernel():
 
 
 SWEEP = [(N, H, L, E, M) for (N, H) in [(1, 1), (1, 16), (2, 8), (10, 8), (64, 16)]
-         for L in [1, 64, 1000, 4096, 20000] for (E, M) in [(64, 64), (32, 128), (96, 64), (25, 70), (128, 128), (100, 36), (200, 64), (255, 129)]]
+         for L in [1, 64, 1000, 4096, 20000] for (E, M) in [(64, 64), (32, 128), (96, 64), (25, 70), (128, 128), (100, 36), (200, 64), (255, 129), (511, 300)]]
 
 
 @pytest.mark.parametrize("backward", [False, True])
