@@ -39,9 +39,9 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 matrix, published
 # carries it only while the sources are unchanged, otherwise null.
 MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {
     # workload: (bytes, kernel source hash at the time of the measurement)
-    "cfg2": (137381497, "fa1332bb6ad7d504"),
-    "cfg3": (3141841000, "fa1332bb6ad7d504"),
-    "wide": (1877425462, "fa1332bb6ad7d504"),
+    "cfg2": (137377586, "c5d7ba6bb9605e31"),
+    "cfg3": (3140482539, "c5d7ba6bb9605e31"),
+    "wide": (1877471122, "c5d7ba6bb9605e31"),
 }
 
 WORKLOADS = {
