@@ -147,6 +147,34 @@ void launch_pad_rows(void *strided, int64_t sn, int64_t sh, int64_t sl, int64_t 
                            (uint16_t *)strided, sn, sh, sl, H, L, Lp, N * H, w, wp, (uint16_t *)dense);
 }
 
+// The same between bf16 rows of the caller and fp32 dense rows (bf16 operands of a scan that
+// only the fp32 kernels take: exact on the way in, rounded to nearest even on the way out).
+template <bool PAD>
+__global__ __launch_bounds__(256) void pad_rows_bf16_kernel(uint16_t *strided, int64_t sn, int64_t sh,
+                                                            int64_t sl, int64_t H, int64_t L,
+                                                            int64_t chains, int w, int wp, float *dense) {
+    const uint32_t groups = (uint32_t)wp / 4;
+    const uint32_t j = blockIdx.x * 256u + threadIdx.x;
+    if (j >= (uint32_t)L * groups) return;
+    const uint32_t l = j / groups, c0 = (j % groups) * 4;
+    for (int64_t chain = blockIdx.y; chain < chains; chain += gridDim.y) {
+        uint16_t *row = strided + (chain / H) * sn + (chain % H) * sh + (int64_t)l * sl;
+        float *slot = dense + (chain * L + l) * wp + c0;
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            if (PAD) slot[e] = (int)(c0 + e) < w ? bf16_to_f32(row[c0 + e]) : 0.f;
+            else if ((int)(c0 + e) < w) row[c0 + e] = f32_to_bf16(slot[e]);
+        }
+    }
+}
+template <bool PAD>
+void launch_pad_rows_bf16(void *strided, int64_t sn, int64_t sh, int64_t sl, int64_t N, int64_t H,
+                          int64_t L, int w, int wp, void *dense, hipStream_t stream) {
+    const dim3 grid((unsigned)((L * (wp / 4) + 255) / 256), (unsigned)std::min<int64_t>(N * H, 65535));
+    hipLaunchKernelGGL((pad_rows_bf16_kernel<PAD>), grid, dim3(256), 0, stream, (uint16_t *)strided, sn,
+                       sh, sl, H, L, N * H, w, wp, (float *)dense);
+}
+
 // (measured down to 512 rows: E = 25, M = 33, one chain of 512 positions, forward + backward
 // 0.10 ms on the copies against 0.30 ms on the VALU kernel)
 constexpr int64_t kPadMinRows = 512;
@@ -182,8 +210,8 @@ __global__ __launch_bounds__(256) void add_rows_kernel(float *strided, int64_t s
     }
 }
 
-// workspace of the two launches of a split (the larger of the two) and of the buffers of the
-// second halves of up to kMfmaMaxScans scans
+// workspace of the launches of a split (the largest need among them) and of the buffers that
+// take the later parts' results of up to kMfmaMaxScans scans
 int64_t split_scan_workspace_bytes(int64_t N, int64_t H, int64_t L, int64_t D, int64_t F,
                                    int64_t *launch_bytes) {
     int64_t ws = FTC_WORKSPACE_CONTROL_BYTES;
@@ -200,7 +228,7 @@ int run_scans(const ScanDesc *scans, int n, int64_t N, int64_t H, int64_t L, voi
               size_t workspace_bytes, hipStream_t stream, bool may_pad);
 
 // Runs scans[0 .. n) of one shape (split_widths) as described above.  *done = false (nothing
-// launched) when the chain-parallel kernel does not take the halves or the workspace has no room.
+// launched) when the chain-parallel kernel does not take the parts or the workspace has no room.
 int split_scans(const ScanDesc *scans, int n, int64_t N, int64_t H, int64_t L, void *workspace,
                 size_t workspace_bytes, hipStream_t stream, bool *done) {
     *done = false;
@@ -264,13 +292,16 @@ bool padded_shape_ok(int64_t Dp, int64_t Fp) {
 }
 
 int64_t scan_workspace_bytes(int64_t N, int64_t H, int64_t L, int64_t D, int64_t F,
-                             bool with_pad = true);
+                             bool with_pad = true, bool bf16 = false);
 
 // workspace of the padded route of one scan: the scan's own, then dense copies of all four
 // operands (fp32 sizes: an upper bound)
-int64_t padded_scan_workspace_bytes(int64_t N, int64_t H, int64_t L, int64_t D, int64_t F) {
+// (`bf16`: rows of a state beyond 128 rows are copied whatever their widths, to convert them)
+int64_t padded_scan_workspace_bytes(int64_t N, int64_t H, int64_t L, int64_t D, int64_t F,
+                                    bool bf16 = false) {
     const int64_t Dp = padded_rows(D), Fp = round_up(F, 32), rows = N * H * L;
-    if (Dp == 0 || (Dp == D && Fp == F) || rows < kPadMinRows || !padded_shape_ok(Dp, Fp)) return 0;
+    const bool copies = Dp != D || Fp != F || (bf16 && Dp > 128);
+    if (Dp == 0 || !copies || rows < kPadMinRows || !padded_shape_ok(Dp, Fp)) return 0;
     return std::max<int64_t>(round_up(scan_workspace_bytes(N, H, L, Dp, Fp), 256),
                              FTC_WORKSPACE_CONTROL_BYTES) +
            2 * round_up(rows * Dp * 4, 256) + 2 * round_up(rows * Fp * 4, 256) +
@@ -295,6 +326,7 @@ int padded_scans(const ScanDesc *scans, int n, const bool *take, int64_t N, int6
         int dtype, width, padded;
         bool is_output;
         char *dense;
+        int dense_dtype;  // FTC_F32 for a bf16 tensor of a scan that only the fp32 kernels take
     };
     Copy copies[4 * kMfmaMaxScans];
     int ncopies = 0;
@@ -302,13 +334,13 @@ int padded_scans(const ScanDesc *scans, int n, const bool *take, int64_t N, int6
     int nwork = 0;
     int64_t ws_scan = 0;
     auto copy_of = [&](const void *ptr, int64_t sn, int64_t sh, int64_t sl, int dtype, int width,
-                       int padded, bool is_output) -> int {
+                       int padded, bool is_output, int dense_dtype) -> int {
         for (int i = 0; i < ncopies; i++)
             if (copies[i].ptr == ptr && copies[i].sn == sn && copies[i].sh == sh &&
                 copies[i].sl == sl && copies[i].width == width && copies[i].padded == padded &&
-                !copies[i].is_output && !is_output)
+                copies[i].dense_dtype == dense_dtype && !copies[i].is_output && !is_output)
                 return i;
-        copies[ncopies] = Copy{ptr, sn, sh, sl, dtype, width, padded, is_output, nullptr};
+        copies[ncopies] = Copy{ptr, sn, sh, sl, dtype, width, padded, is_output, nullptr, dense_dtype};
         return ncopies++;
     };
     // the states handed in and out, padded the same way (rows and columns)
@@ -332,27 +364,34 @@ int padded_scans(const ScanDesc *scans, int n, const bool *take, int64_t N, int6
                 states[nstates++] = StateCopy{sc.final_, sc.a.width, sc.v.width, Dp, Fp, nwork, true, nullptr};
         }
         ws_scan = std::max(ws_scan, round_up(scan_workspace_bytes(N, H, L, Dp, Fp), 256));
+        // states beyond 128 rows run on the fp32 kernels only: bf16 tensors of such a scan are
+        // converted on the way
+        const bool to_f32 = Dp > 128;
         const Operand *in[3] = {&sc.a, &sc.b, &sc.v};
         const int target[3] = {Dp, Dp, Fp};
         for (int k = 0; k < 3; k++) {
             const Operand &o = *in[k];
-            which[nwork][k] = o.width == target[k] && mfma_operand_in_place(o.ptr, o.stride_n, o.stride_h,
-                                                                           o.stride_l, o.dtype, o.width, L)
+            const int dd = to_f32 ? FTC_F32 : o.dtype;
+            which[nwork][k] = o.width == target[k] && dd == o.dtype &&
+                                      mfma_operand_in_place(o.ptr, o.stride_n, o.stride_h, o.stride_l,
+                                                            o.dtype, o.width, L)
                                   ? -1
                                   : copy_of(o.ptr, o.stride_n, o.stride_h, o.stride_l, o.dtype, o.width,
-                                            target[k], false);
+                                            target[k], false, dd);
         }
         const OperandOut &o = sc.out;
-        which[nwork][3] = o.width == Fp && mfma_operand_in_place(o.ptr, o.stride_n, o.stride_h, o.stride_l,
-                                                                 o.dtype, o.width, L)
+        const int dd = to_f32 ? FTC_F32 : o.dtype;
+        which[nwork][3] = o.width == Fp && dd == o.dtype &&
+                                  mfma_operand_in_place(o.ptr, o.stride_n, o.stride_h, o.stride_l, o.dtype,
+                                                        o.width, L)
                               ? -1
-                              : copy_of(o.ptr, o.stride_n, o.stride_h, o.stride_l, o.dtype, o.width, Fp, true);
+                              : copy_of(o.ptr, o.stride_n, o.stride_h, o.stride_l, o.dtype, o.width, Fp, true, dd);
         work[nwork++] = sc;
     }
     // the copies never lie on the control block, which every call must leave zeroed
     ws_scan = std::max<int64_t>(ws_scan, FTC_WORKSPACE_CONTROL_BYTES);
     int64_t need = ws_scan;
-    for (int i = 0; i < ncopies; i++) need += round_up(rows * copies[i].padded * esz(copies[i].dtype), 256);
+    for (int i = 0; i < ncopies; i++) need += round_up(rows * copies[i].padded * esz(copies[i].dense_dtype), 256);
     for (int i = 0; i < nstates; i++) {
         if (N * H * states[i].Dp * states[i].Fp >= 0x7fffffffLL) return FTC_OK;  // (fill kernel: 32-bit count)
         need += round_up(N * H * states[i].Dp * states[i].Fp * 4, 256);
@@ -362,7 +401,7 @@ int padded_scans(const ScanDesc *scans, int n, const bool *take, int64_t N, int6
     char *base = (char *)workspace + ws_scan;
     for (int i = 0; i < ncopies; i++) {
         copies[i].dense = base;
-        base += round_up(rows * copies[i].padded * esz(copies[i].dtype), 256);
+        base += round_up(rows * copies[i].padded * esz(copies[i].dense_dtype), 256);
     }
     for (int i = 0; i < nstates; i++) {
         StateCopy &st = states[i];
@@ -378,12 +417,12 @@ int padded_scans(const ScanDesc *scans, int n, const bool *take, int64_t N, int6
             if (which[s][k] >= 0) {
                 const Copy &c = copies[which[s][k]];
                 const int64_t w = c.padded;
-                *in[k] = Operand{c.dense, H * L * w, L * w, w, c.dtype, (int32_t)w};
+                *in[k] = Operand{c.dense, H * L * w, L * w, w, c.dense_dtype, (int32_t)w};
             }
         if (which[s][3] >= 0) {
             const Copy &c = copies[which[s][3]];
             const int64_t w = c.padded;
-            work[s].out = OperandOut{c.dense, H * L * w, L * w, w, c.dtype, (int32_t)w};
+            work[s].out = OperandOut{c.dense, H * L * w, L * w, w, c.dense_dtype, (int32_t)w};
         }
     }
     int nin = 0, nout = 0;
@@ -393,11 +432,17 @@ int padded_scans(const ScanDesc *scans, int n, const bool *take, int64_t N, int6
                   "back, workspace %lld bytes", nin, nin == 1 ? "" : "s", nout, nout == 1 ? "" : "s",
                   (long long)need);
     } else {
-        for (int i = 0; i < ncopies; i++)
-            if (!copies[i].is_output)
+        for (int i = 0; i < ncopies; i++) {
+            if (copies[i].is_output) continue;
+            if (copies[i].dense_dtype != copies[i].dtype)
+                launch_pad_rows_bf16<true>((void *)copies[i].ptr, copies[i].sn, copies[i].sh, copies[i].sl,
+                                           N, H, L, copies[i].width, copies[i].padded, copies[i].dense,
+                                           stream);
+            else
                 launch_pad_rows<true>((void *)copies[i].ptr, copies[i].sn, copies[i].sh, copies[i].sl,
                                       N, H, L, copies[i].width, copies[i].padded,
                                       esz(copies[i].dtype), copies[i].dense, stream);
+        }
         for (int i = 0; i < nstates; i++) {
             const StateCopy &st = states[i];
             if (st.is_output) continue;
@@ -411,11 +456,17 @@ int padded_scans(const ScanDesc *scans, int n, const bool *take, int64_t N, int6
     int rc = run_scans(work, nwork, N, H, L, workspace, (size_t)ws_scan, stream, false);
     if (rc) return rc;
     if (!plan_only()) {
-        for (int i = 0; i < ncopies; i++)
-            if (copies[i].is_output)
+        for (int i = 0; i < ncopies; i++) {
+            if (!copies[i].is_output) continue;
+            if (copies[i].dense_dtype != copies[i].dtype)
+                launch_pad_rows_bf16<false>((void *)copies[i].ptr, copies[i].sn, copies[i].sh,
+                                            copies[i].sl, N, H, L, copies[i].width, copies[i].padded,
+                                            copies[i].dense, stream);
+            else
                 launch_pad_rows<false>((void *)copies[i].ptr, copies[i].sn, copies[i].sh, copies[i].sl,
                                        N, H, L, copies[i].width, copies[i].padded,
                                        esz(copies[i].dtype), copies[i].dense, stream);
+        }
         for (int i = 0; i < nstates; i++) {
             const StateCopy &st = states[i];
             if (st.is_output)
@@ -437,10 +488,6 @@ bool pad_eligible(const ScanDesc &sc, int64_t rows) {
     if (Dp == 0 || rows < kPadMinRows) return false;
     if (const char *env = getenv("FTC_PAD"))  // tuning aid
         if (atoi(env) == 0) return false;
-    // (the split of states beyond 128 rows is for fp32 rows only)
-    if (Dp > 128 && !(sc.a.dtype == FTC_F32 && sc.b.dtype == FTC_F32 && sc.v.dtype == FTC_F32 &&
-                      sc.out.dtype == FTC_F32))
-        return false;
     return padded_shape_ok(Dp, round_up(sc.v.width, 32));
 }
 
@@ -530,14 +577,16 @@ int run_scans(const ScanDesc *scans, int n, int64_t N, int64_t H, int64_t L, voi
 // Upper bound over every way run_scans may slice and group scans of these widths.
 // `with_pad` = false leaves out the padded copies and the buffers of split scans: what a call
 // needs at the least (without them such a scan runs on the generic kernel).
-int64_t scan_workspace_bytes(int64_t N, int64_t H, int64_t L, int64_t D, int64_t F, bool with_pad) {
+int64_t scan_workspace_bytes(int64_t N, int64_t H, int64_t L, int64_t D, int64_t F, bool with_pad,
+                             bool bf16) {
     int64_t need = generic_scan_workspace_bytes(N, H, L, D, F);
     int widths[kMfmaMaxSlices];
     const int nslices = mfma_slice_widths(D, F, widths);
     for (int j = 0; j < nslices; j++)
         for (int k = 1; k <= kMfmaMaxScans; k++)
             need = std::max(need, mfma_scan_workspace_bytes(N, H, L, D, widths[j], k));
-    if (nslices == 0 && with_pad) need = std::max(need, padded_scan_workspace_bytes(N, H, L, D, F));
+    if (nslices == 0 && with_pad)
+        need = std::max(need, padded_scan_workspace_bytes(N, H, L, D, F, bf16));
     for (int k = 1; k <= kMfmaMaxScans; k++)
         need = std::max(need, mfma_tp_workspace_bytes(N, H, L, D, F, k));
     if (with_pad && split_widths(D, F))
@@ -595,7 +644,7 @@ int64_t ftc_causal_dot_product_workspace_bytes(int64_t N, int64_t H, int64_t L, 
     if (N * H * L == 0 || M == 0 || E == 0) return 0;
     if (E > kGenericMaxDim || M > kGenericMaxDim)
         return fail(FTC_ERR_UNSUPPORTED, "E and M must be at most %d", kGenericMaxDim);
-    return scan_workspace_bytes(N, H, L, E, M);
+    return scan_workspace_bytes(N, H, L, E, M, true, dtype == FTC_BF16);
 }
 
 int ftc_causal_dot_product(const ftc_tensor4 *queries, const ftc_tensor4 *keys,
@@ -707,9 +756,12 @@ int64_t ftc_causal_dot_backward_workspace_bytes(int64_t N, int64_t H, int64_t L,
     if (N * H * L == 0 || M == 0 || E == 0) return 0;
     if (E > kGenericMaxDim || M > kGenericMaxDim)
         return fail(FTC_ERR_UNSUPPORTED, "E and M must be at most %d", kGenericMaxDim);
-    int64_t need = std::max(scan_workspace_bytes(N, H, L, E, M), scan_workspace_bytes(N, H, L, M, E));
+    const bool bf16 = dtype == FTC_BF16;
+    int64_t need = std::max(scan_workspace_bytes(N, H, L, E, M, true, bf16),
+                            scan_workspace_bytes(N, H, L, M, E, true, bf16));
     // the padded route of the three scans together: Q, K, dQ, dK and V, G, dV as dense rows
-    if (padded_scan_workspace_bytes(N, H, L, E, M) > 0 || padded_scan_workspace_bytes(N, H, L, M, E) > 0) {
+    if (padded_scan_workspace_bytes(N, H, L, E, M, bf16) > 0 ||
+        padded_scan_workspace_bytes(N, H, L, M, E, bf16) > 0) {
         int64_t ws = 0;
         if (padded_rows(E)) ws = std::max(ws, scan_workspace_bytes(N, H, L, padded_rows(E), round_up(M, 32)));
         if (padded_rows(M)) ws = std::max(ws, scan_workspace_bytes(N, H, L, padded_rows(M), round_up(E, 32)));

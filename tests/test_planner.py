@@ -79,8 +79,11 @@ def test_what_the_chain_parallel_kernel_leaves_to_the_others():
     assert wide[0].startswith("pad_rows_kernel: 4 operands") and "3 results" in wide[0]
     assert wide[1].startswith("scan_tp_kernel: 3 scans") and "state 128 x 128" in wide[1]
     assert lines((2, 2, 40, 10), (2, 2, 40, 3))[0].startswith("generic_scan_kernel")
+    # (bf16 rows of such a scan are converted into fp32 copies on the way)
     assert lines((1, 2, 8192, 300), (1, 2, 8192, 64), dtype=_native.FTC_BF16)[0] \
-        .startswith("generic_scan_kernel")
+        .startswith("pad_rows_kernel: 3 operands")
+    assert lines((1, 2, 100, 300), (1, 2, 100, 64), dtype=_native.FTC_BF16)[0] \
+        .startswith("generic_scan_kernel")   # (too few rows for the copies)
     # states of 129 to 512 rows: up to four scans over a split of the rows, the later ones'
     # rows added to the first one's
     three = lines((1, 2, 8192, 300), (1, 2, 8192, 64))
