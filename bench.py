@@ -39,9 +39,9 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 matrix, published
 # carries it only while the sources are unchanged, otherwise null.
 MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {
     # workload: (bytes, kernel source hash at the time of the measurement)
-    "cfg2": (137377586, "c5d7ba6bb9605e31"),
-    "cfg3": (3140482539, "c5d7ba6bb9605e31"),
-    "wide": (1877471122, "c5d7ba6bb9605e31"),
+    "cfg2": (137391756, "3e8d53cbcaa977a7"),
+    "cfg3": (3137663994, "3e8d53cbcaa977a7"),
+    "wide": (1877406822, "3e8d53cbcaa977a7"),
 }
 
 WORKLOADS = {
