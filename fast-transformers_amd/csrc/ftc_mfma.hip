@@ -490,7 +490,12 @@ int mfma_scan(const ScanDesc *scans, int nscans, int64_t N, int64_t H, int64_t L
         return FTC_OK;
     }
     if (tp) {
-        launch_scan_tp(workspace, args, stream);
+        bool half_pieces = D <= 64;
+        if (const char *env = getenv("FTC_TPH")) half_pieces = half_pieces && atoi(env) != 0;  // tuning aid
+        if (half_pieces)
+            launch_scan_tph(workspace, args, stream);
+        else
+            launch_scan_tp(workspace, args, stream);
     } else if (wg) {
         launch_scan_wg_ffff(D, F, fused != nullptr, workspace, args, stream);
     } else if (dma) {

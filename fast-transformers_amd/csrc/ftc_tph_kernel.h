@@ -1,0 +1,871 @@
+// Chain-parallel form of the MFMA causal scan for gfx950 on the fp16 matrix path: all-fp32
+// rows, states of up to 64 x 64 per workgroup (output columns beyond 64 have a workgroup of
+// their own, widths that do not fill the block are clipped).
+//
+//   out[c, l, f] = sum_{j <= l} (a[c,l,:] . b[c,j,:]) * v[c,j,f]      (REV: j >= l)
+//
+// Division of labour, chunking, LDS tiles, swizzles, segments and the exchange of segment
+// sums are those of ftc_tp_kernel.h (one workgroup walks one chain; four consumer wavefronts
+// hold the state as slabs of 16 columns and share the chunk product Pt through LDS; four
+// producer wavefronts fetch rows four chunks ahead and cut them into piece tiles).  What
+// differs is the arithmetic that stands for an fp32 product:
+//
+//  * Every fp32 value x is scaled by a power of two and cut into TWO fp16 pieces, both rounded
+//    to nearest: hi = fp16(x s), lo = fp16(x s - hi).  hi + lo carries 22 significand bits of
+//    x s as long as |x s| >= 2^-3 (below that the absolute error stays under 2^-25), and
+//    |x s| < 2^16 must hold.  A product is the sum of THREE piece products (lo hi, hi lo,
+//    hi hi; lo lo is below 2^-22 of the product) on v_mfma_f32_16x16x32_f16, each exact in the
+//    fp32 accumulator: half the matrix instructions, two thirds of the LDS traffic and about
+//    a third of the vector instructions of three bf16 pieces, with results as close to
+//    float64 as those (the reference's own fp32 order is further away than either).
+//  * The scales.  Rows of a, b and v are scaled chunk by chunk by powers of two that are
+//    running ceilings: 2^(4 - e) with e the smallest exponent such that every value of that
+//    operand met so far in the walk is below 2^e in magnitude.  Scaled values therefore stay
+//    below 16, values down to 2^-7 of the largest one met so far keep 22 bits, and the error
+//    of smaller ones is below 2^-29 of that largest one -- the way the reference's running
+//    fp32 state treats small contributions.  The ceilings come about without a pass of their
+//    own: while it cuts position k of the walk, every wavefront that cuts looks at the rows of
+//    position k + 1, which it already holds in registers; a wavefront that finds a value at
+//    or above the current ceiling (rare after the first chunks) raises that position's slot
+//    in LDS with an atomic maximum, and after the workgroup barrier all eight wavefronts read
+//    the slot.  All of them thus know the same three exponents for every position.
+//  * The state is kept in the units of the scaled rows (2^(e_b + e_v - 8)); when a ceiling
+//    rises it is rescaled (exactly).  It is cut into pieces with one more power of two,
+//    2^-s, chosen so that no element exceeds 2^15: s rises when the largest element of the
+//    state before the previous chunk exceeds 2^(14 + s) (a chunk adds at most 2^13).  The
+//    chunk product needs no scale: |Pt| <= 64 * 16 * 16 = 2^14.
+//  * Ot = (S^T a^T) 2^s + v^T Pt is summed in the units of the chunk and leaves the
+//    accumulator through one v_ldexp_f32 per value.
+//
+// Results depend on where a chain is cut (the ceilings of `a` start afresh in every segment),
+// within the rounding of the pieces.
+#pragma once
+#include <type_traits>
+
+#include "ftc_tp_kernel.h"
+
+namespace ftc {
+namespace mfma {
+
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+
+__device__ __forceinline__ f32x4 mfma16h(const Frag &a, const Frag &b, f32x4 c) {
+#ifdef FTC_ABL_NOMFMA
+    asm volatile("" ::"v"(a.w[0]), "v"(b.w[0]));
+    asm volatile("" : "+v"(c));
+    return c;
+#endif
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a),
+                                                  __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+}
+
+// Two fp32 values times a power of two -> packed fp16 pieces (x0 in the low half), both
+// rounded to nearest even.  v_fma_mix{lo,hi}_f16 computes fma(x, s, c) in fp32 (exact here:
+// x s is exact, and so is the remainder of a rounding) and rounds once to fp16; the third
+// operand is the fp16 hi piece, read from the half that op_sel names and negated.
+__device__ __forceinline__ void cut_pair_f16(float x0, float x1, float s, uint32_t &hi, uint32_t &lo) {
+    asm("v_fma_mixlo_f16 %0, %1, %2, 0" : "=v"(hi) : "v"(x0), "s"(s));
+    asm("v_fma_mixhi_f16 %0, %1, %2, 0" : "+v"(hi) : "v"(x1), "s"(s));
+    asm("v_fma_mixlo_f16 %0, %1, %2, -%3 op_sel:[0,0,0] op_sel_hi:[0,0,1]"
+        : "=v"(lo) : "v"(x0), "s"(s), "v"(hi));
+    asm("v_fma_mixhi_f16 %0, %1, %2, -%3 op_sel:[0,0,1] op_sel_hi:[0,0,1]"
+        : "+v"(lo) : "v"(x1), "s"(s), "v"(hi));
+}
+// the same without a scale: one packed conversion for the hi pieces
+__device__ __forceinline__ void cut_pair_f16_unscaled(float x0, float x1, uint32_t &hi, uint32_t &lo) {
+    asm("v_cvt_pk_f16_f32 %0, %1, %2" : "=v"(hi) : "v"(x0), "v"(x1));
+    asm("v_fma_mixlo_f16 %0, %1, 1.0, -%2 op_sel:[0,0,0] op_sel_hi:[0,0,1]"
+        : "=v"(lo) : "v"(x0), "v"(hi));
+    asm("v_fma_mixhi_f16 %0, %1, 1.0, -%2 op_sel:[0,0,1] op_sel_hi:[0,0,1]"
+        : "+v"(lo) : "v"(x1), "v"(hi));
+}
+// Four consecutive fp32 values of a row -> 8 bytes of each of the two piece tiles.
+__device__ __forceinline__ void cut_quad_to_lds(const u32x4 raw, float s, lds_char *tile,
+                                                int piece_bytes, int addr) {
+    uint32_t h0, l0, h1, l1;
+    cut_pair_f16(__uint_as_float(raw.x), __uint_as_float(raw.y), s, h0, l0);
+    cut_pair_f16(__uint_as_float(raw.z), __uint_as_float(raw.w), s, h1, l1);
+    const u32x2 wh = {h0, h1}, wl = {l0, l1};
+    *(lds_vec2 *)(tile + addr) = wh;
+    *(lds_vec2 *)(tile + piece_bytes + addr) = wl;
+}
+__device__ __forceinline__ float max_abs4(const u32x4 raw, float m) {
+    m = fmaxf(fmaxf(fabsf(__uint_as_float(raw.x)), fabsf(__uint_as_float(raw.y))), m);
+    return fmaxf(fmaxf(fabsf(__uint_as_float(raw.z)), fabsf(__uint_as_float(raw.w))), m);
+}
+
+// Exponents travel as E = e + 128 with e clamped to -100 .. 120 (E = 28 .. 248), where 2^e is
+// the ceiling: every value met so far is below it.
+constexpr uint32_t kExpFloor = 28, kExpCeil = 248;
+__device__ __forceinline__ float pow2_field(int field) {  // 2^(field - 127), field clamped
+    return __uint_as_float((uint32_t)max(1, min(254, field)) << 23);
+}
+// the ceiling exponent of a non-negative float (inf and NaN: the largest)
+__device__ __forceinline__ uint32_t ceiling_of(float m) {
+    const uint32_t be = (__float_as_uint(m) >> 23) & 0xffu;  // m < 2^(be - 126)
+    return max(kExpFloor, min(kExpCeil, be + 2u));
+}
+__device__ __forceinline__ float wave_max(float m) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) m = fmaxf(m, __shfl_xor(m, off));
+    return m;
+}
+
+// The running ceilings of a, b and v as one wavefront knows them (wave-uniform).
+struct Ceilings {
+    uint32_t Ea, Eb, Ev;
+    __device__ __forceinline__ float scale_a() const { return pow2_field(259 - (int)Ea); }
+    __device__ __forceinline__ float scale_b() const { return pow2_field(259 - (int)Eb); }
+    __device__ __forceinline__ float scale_v() const { return pow2_field(259 - (int)Ev); }
+    // exponent of the state's units, and of a chunk's output units (a x state)
+    __device__ __forceinline__ int state_exp() const { return (int)(Eb + Ev) - 264; }
+    __device__ __forceinline__ int out_exp() const { return (int)(Ea + Eb + Ev) - 396; }
+};
+typedef __attribute__((address_space(3))) uint32_t lds_u32_t;
+// The slot of a position is that of its LDS buffer: words (a, b, v, unused)
+__device__ __forceinline__ void read_slot(const lds_u32_t *slots, int k, Ceilings &c) {
+    const u32x4 s = *(const lds_vec4 *)(slots + 4 * k);
+    c.Ea = max(c.Ea, (uint32_t)__builtin_amdgcn_readfirstlane(s.x));
+    c.Eb = max(c.Eb, (uint32_t)__builtin_amdgcn_readfirstlane(s.y));
+    c.Ev = max(c.Ev, (uint32_t)__builtin_amdgcn_readfirstlane(s.z));
+}
+// lane maxima of the rows of a position against the ceilings known so far: whoever finds a
+// value at or above one raises slot k, that position's
+__device__ __forceinline__ void raise_slot(lds_u32_t *slots, int k, const Ceilings &c, float ma,
+                                           float mb, float mv, int lane) {
+    const bool over = ma >= pow2_field((int)c.Ea - 1) || mb >= pow2_field((int)c.Eb - 1) ||
+                      mv >= pow2_field((int)c.Ev - 1);
+    if (__builtin_amdgcn_ballot_w64(over) != 0) {
+        const uint32_t ea = ceiling_of(wave_max(ma)), eb = ceiling_of(wave_max(mb)),
+                       ev = ceiling_of(wave_max(mv));
+        lds_u32_t *const s = slots + 4 * k;
+        if (lane == 0) {
+            if (ea > c.Ea) __hip_atomic_fetch_max(s + 0, ea, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            if (eb > c.Eb) __hip_atomic_fetch_max(s + 1, eb, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            if (ev > c.Ev) __hip_atomic_fetch_max(s + 2, ev, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        }
+    }
+}
+
+// KS: groups of 32 rows of the state (1: a state of up to 32 rows, which skips the matrix
+// instructions and fragment reads of the empty half)
+template <int KS>
+__global__ __launch_bounds__(512, 1) void scan_tph_kernel(uint32_t *__restrict__ ws_ptr, ScanArgs p) {
+    constexpr int D = 64, F = 64;              // one block of state rows and of output columns
+    constexpr int T = 256;                     // producer lanes
+    constexpr int PF = kTpAhead;               // chunks requested ahead
+    constexpr int RBA = D * 2, RBV = F * 2;    // bytes per row of an fp16 piece tile
+    constexpr int kTileA = kChunk * RBA, kTileV = kChunk * RBV;
+    constexpr int kOffB = 2 * kTileA, kOffV = 4 * kTileA;
+    constexpr int kBufBytes = 4 * kTileA + 2 * kTileV;
+    constexpr int kTileP = kChunk * 64;        // Pt pieces: 32 rows (i) of 32 j
+    constexpr int QA = D / 4, QV = F / 4;
+    constexpr int LA = kChunk * QA / T, LV = kChunk * QV / T;
+    static_assert(kChunk == 32 && T % QA == 0 && T % QV == 0 && PF == 4, "shape");
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const bool producer = wave >= 4;
+    const int w = wave & 3;
+
+    __shared__ __align__(16) char pieces_mem[3 * kBufBytes];
+    __shared__ __align__(16) char pt_mem[3 * 2 * kTileP];
+    __shared__ __align__(16) uint32_t slot_mem[16];
+    lds_char *const unit_pc = (lds_char *)pieces_mem;
+    lds_char *const pt_pc = (lds_char *)pt_mem;
+    lds_u32_t *const slots = (lds_u32_t *)slot_mem;
+
+    // ---- which chain (as in scan_tp_kernel) ----
+    const uint32_t nseg = (uint32_t)p.nseg;
+    const uint32_t chains = (uint32_t)p.waves_per_scan / nseg;
+    const uint32_t per_chain = (uint32_t)p.total_waves / chains;  // scans x segments
+    const uint32_t full = (chains / 8u) * 8u;
+    uint32_t which, chain;
+    if (blockIdx.x < full * per_chain) {
+        const uint32_t grp = blockIdx.x / (8u * per_chain), r = blockIdx.x % (8u * per_chain);
+        which = r / 8u;
+        chain = grp * 8u + r % 8u;
+    } else {
+        const uint32_t t = blockIdx.x - full * per_chain;
+        which = t / (chains - full);
+        chain = full + t % (chains - full);
+    }
+    const uint32_t virt = which / nseg;
+    const uint32_t scan_id = virt / (uint32_t)p.tp_fblocks;
+    const int fb = (int)(virt % (uint32_t)p.tp_fblocks);
+    const int Dw = p.tp_d;                      // state rows: a and b are this wide
+    const int fw = min(F, p.tp_f - F * fb);     // output columns of this block
+    const ScanOperands &op = p.scan[scan_id];
+    const bool REV = op.rev != 0;
+    const int n = (int)(chain / (uint32_t)p.H), h = (int)(chain % (uint32_t)p.H);
+    const int rows = (int)p.L;
+    const int total_chunks = (rows + kChunk - 1) / kChunk;
+    const bool exchange = p.tp_exchange != 0 && nseg > 1;
+    gu32 *const hdr = (gu32 *)ws_ptr;
+    gu32 *const flags = hdr + kHdrWords;
+    const uint32_t chain_id = virt * chains + chain;  // over all scans of the launch
+    int seg = (int)(which % nseg);
+    __shared__ uint32_t order_sh;
+    if (exchange) {
+        if (tid == 0)
+            order_sh = __hip_atomic_fetch_add(flags + kMaxWaves + chain_id, 1u, __ATOMIC_RELAXED,
+                                              __HIP_MEMORY_SCOPE_AGENT);
+        __syncthreads();
+        seg = (int)__builtin_amdgcn_readfirstlane(order_sh);
+        if ((uint32_t)seg >= nseg) {  // the control block was not zero when the launch began
+            if (tid == 0)
+                __hip_atomic_store(hdr + kHdrError, 2u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            return;
+        }
+    }
+    const int c0 = exchange ? seg * p.tp_seg_chunks : p.tp_start[seg];
+    const int nchunks = min(total_chunks, exchange ? c0 + p.tp_seg_chunks : p.tp_start[seg + 1]);
+    // the chunks walked for their state alone: so0 .. so0 + n1 - 1 (n1 a multiple of PF)
+    const int so0 = exchange ? c0 : 0;
+    const int n1 = exchange ? (seg + 1 < (int)nseg ? nchunks - c0 : 0) : c0;
+    const int nwalk = n1 + (nchunks - c0);  // (position nwalk: a chunk of zeros)
+    auto so_chunk = [&](int v) -> int { return exchange ? so0 + n1 - 1 - v : so0 + v; };
+    auto walk_chunk = [&](int v) -> int { return v < n1 ? so_chunk(v) : c0 + (v - n1); };
+    constexpr uint32_t kNoRow = 0x80000000u;  // an offset outside every descriptor
+    auto chunk_row0 = [&](int c) -> int { return REV ? rows - kChunk * (c + 1) : kChunk * c; };
+    if (tid < 16) slot_mem[tid] = 0;
+    Ceilings ce{kExpFloor, kExpFloor, kExpFloor};
+    // Position k of the walk goes through LDS buffer (B0 + k) % 3 (pieces, Pt and slot), with B0
+    // such that the first chunk of the walk proper has buffer 0: the consumers' loop over
+    // those chunks is unrolled three times and addresses LDS with immediate offsets.
+    const int B0 = (3 - n1 % 3) % 3;
+    auto next_buf = [](int b) -> int { return b == 2 ? 0 : b + 1; };
+#ifdef FTC_TIMELINE
+    // tuning aid: 32 time stamps per workgroup behind the pointer that the host passes in
+    // p.key_len (FTC_STAMP_PTR), written by lane 0 of consumer 0 (0 .. 15) and of producer 0
+    // (16 .. 31) in the fifth chunk of the walk proper
+    typedef __attribute__((address_space(1))) uint64_t gu64;
+    const bool stamp_on = p.key_len != nullptr && w == 0 && lane == 0;
+    gu64 *const stamp_base = (gu64 *)p.key_len + blockIdx.x * 32 + (producer ? 16 : 0);
+    // ... and behind those, 64 stamps per workgroup: consumer 0 after the barrier of every chunk
+    gu64 *const chunk_stamps = (gu64 *)p.key_len + gridDim.x * 32 + blockIdx.x * 64;
+#endif
+    FTC_STAMP(14);  // workgroup under way
+#ifdef FTC_TIMELINE
+    if (stamp_on && !producer) chunk_stamps[0] = __builtin_amdgcn_s_memrealtime();
+#endif
+
+    if (producer) {
+        // =========================== producers ===========================
+#ifdef FTC_ABL_PRIO
+        __builtin_amdgcn_s_setprio(3);
+#endif
+        const int ptid = w * 64 + lane;
+        const uint32_t a_slb = (uint32_t)op.a_sl * 4, b_slb = (uint32_t)op.b_sl * 4,
+                       v_slb = (uint32_t)op.v_sl * 4;
+        const char *a_seg = (const char *)op.a + ((int64_t)n * op.a_sn + (int64_t)h * op.a_sh) * 4;
+        const char *b_seg = (const char *)op.b + ((int64_t)n * op.b_sn + (int64_t)h * op.b_sh) * 4;
+        const char *v_seg = (const char *)op.v +
+                            ((int64_t)n * op.v_sn + (int64_t)h * op.v_sh + F * fb) * 4;
+        const __amdgpu_buffer_rsrc_t a_rs = __builtin_amdgcn_make_buffer_rsrc(
+            (void *)a_seg, 0, (rows - 1) * a_slb + Dw * 4, kRsrcFlags);
+        const __amdgpu_buffer_rsrc_t b_rs = __builtin_amdgcn_make_buffer_rsrc(
+            (void *)b_seg, 0, (rows - 1) * b_slb + Dw * 4, kRsrcFlags);
+        const __amdgpu_buffer_rsrc_t v_rs = __builtin_amdgcn_make_buffer_rsrc(
+            (void *)v_seg, 0, (rows - 1) * v_slb + fw * 4, kRsrcFlags);
+        // widths that do not fill the block: a lane whose four columns lie beyond the width
+        // asks outside the descriptor and cuts zeros (widths are multiples of 4)
+        const bool ab_in = 4 * (ptid % QA) < Dw;
+        const bool v_in = 4 * (ptid % QV) < fw;
+        uint32_t a_goff[LA], b_goff[LA], v_goff[LV];
+        int a_waddr[LA], b_waddr[LA], v_waddr[LV];
+#pragma unroll
+        for (int q = 0; q < LA; q++) {
+            const int u = q * T + ptid, row = u / QA, c4 = u % QA;
+            a_goff[q] = (uint32_t)row * a_slb + 16u * c4;
+            b_goff[q] = (uint32_t)row * b_slb + 16u * c4;
+            a_waddr[q] = TpSwizzle<RBA>::addr(row, 8 * c4);
+            b_waddr[q] = TpSwizzle<RBA>::addr(row, 2 * b_tile_column(4 * c4));
+        }
+#pragma unroll
+        for (int q = 0; q < LV; q++) {
+            const int u = q * T + ptid, row = u / QV, c4 = u % QV;
+            v_goff[q] = (uint32_t)row * v_slb + 16u * c4;
+            v_waddr[q] = TpSwizzle<RBV>::addr(row, 8 * c4);
+        }
+        struct Raw {
+            u32x4 a[LA], b[LA], v[LV];
+        };
+        Raw raw[PF];
+        // Every request is made every time, whether its rows exist or not (of a chunk walked
+        // for its state alone the producers need rows 0 .. 15 of b and v only; positions past
+        // the end of the walk have no rows): a request outside the descriptor costs no memory
+        // traffic and reads as zero, and with a fixed number of requests per chunk the
+        // compiler can wait for the oldest ones only.
+        static_assert(LA == 2 && LV == 2, "quad 0 of a lane: rows 0 .. 15, quad 1: rows 16 .. 31");
+        auto fetch = [&](Raw &r, int v) {  // v: position of the walk
+#ifdef FTC_ABL_NOMEM
+            v = nwalk + 100;
+#endif
+            const int row0 = v < nwalk ? chunk_row0(walk_chunk(v)) : -2 * kChunk;
+            const int row0_x = v >= n1 ? row0 : -2 * kChunk;
+#pragma unroll
+            for (int q = 0; q < LA; q++) {
+                r.a[q] = __builtin_amdgcn_raw_buffer_load_b128(
+                    a_rs, ab_in ? a_goff[q] + (uint32_t)row0_x * a_slb : kNoRow, 0, 0);
+                r.b[q] = __builtin_amdgcn_raw_buffer_load_b128(
+                    b_rs, ab_in ? b_goff[q] + (uint32_t)(q == 0 ? row0 : row0_x) * b_slb : kNoRow, 0, 0);
+            }
+#pragma unroll
+            for (int q = 0; q < LV; q++)
+                r.v[q] = __builtin_amdgcn_raw_buffer_load_b128(
+                    v_rs, v_in ? v_goff[q] + (uint32_t)(q == 0 ? row0 : row0_x) * v_slb : kNoRow, 0, 0);
+        };
+        // the largest magnitudes of the rows of position k against the ceilings (rows that
+        // were not asked for read as zeros)
+        auto look_ahead = [&](const Raw &r, int k) {
+            float ma = 0.f, mb = 0.f, mv = 0.f;
+#pragma unroll
+            for (int q = 0; q < LA; q++) ma = max_abs4(r.a[q], ma), mb = max_abs4(r.b[q], mb);
+#pragma unroll
+            for (int q = 0; q < LV; q++) mv = max_abs4(r.v[q], mv);
+            raise_slot(slots, k, ce, ma, mb, mv, lane);
+        };
+        // position k of the walk goes to its LDS buffer through register set k % PF.  The
+        // first n1 positions only feed the state: no piece of a, and the consumers cut rows
+        // 16 .. 31 of b and v themselves.
+        auto cut = [&](const Raw &r, int buf, bool own) {
+            lds_char *const pc = unit_pc + buf * kBufBytes;
+            const float sa = ce.scale_a(), sb = ce.scale_b(), sv = ce.scale_v();
+#pragma unroll
+            for (int q = 0; q < LA; q++) {
+                if (own) cut_quad_to_lds(r.a[q], sa, pc, kTileA, a_waddr[q]);
+                if (own || q == 0) cut_quad_to_lds(r.b[q], sb, pc + kOffB, kTileA, b_waddr[q]);
+            }
+#pragma unroll
+            for (int q = 0; q < LV; q++)
+                if (own || q == 0) cut_quad_to_lds(r.v[q], sv, pc + kOffV, kTileV, v_waddr[q]);
+        };
+#pragma unroll
+        for (int j = 0; j < PF; j++) fetch(raw[j], j);
+        wg_barrier();  // the slots are zero
+        look_ahead(raw[0], B0);
+        wg_barrier();  // the slot of position 0 is complete
+        // Barrier number k (k = 0: before the consumers' first position; k >= 1: in the
+        // middle of position k - 1) finds position k cut and the slot of position k + 1
+        // complete.  The last one finds a chunk of zeros.
+        int buf = B0;
+        auto step = [&](int v, int j, bool own) {
+            if (own && v == n1 + 4) FTC_STAMP(0);
+#ifndef FTC_ABL_NOLOOK
+            read_slot(slots, buf, ce);
+            look_ahead(raw[(j + 1) % PF], next_buf(buf));
+#endif
+            if (own && v == n1 + 4) FTC_STAMP(1);
+#ifndef FTC_ABL_NOCUT
+            cut(raw[j], buf, own);
+#else
+            asm volatile("" ::"v"(raw[j].a[0]), "v"(raw[j].a[1]), "v"(raw[j].b[0]), "v"(raw[j].b[1]), "v"(raw[j].v[0]), "v"(raw[j].v[1]));
+#endif
+            if (own && v == n1 + 4) FTC_STAMP(2);
+#ifndef FTC_ABL_NOFETCH
+            fetch(raw[j], v + PF);
+#endif
+            buf = buf == 2 ? 0 : buf + 1;
+            if (own && v == n1 + 4) FTC_STAMP(3);
+            wg_barrier();
+            __builtin_amdgcn_sched_barrier(0);  // one chunk at a time, in this order
+            if (own && v == n1 + 4) FTC_STAMP(4);
+        };
+        for (int v = 0; v < n1; v += PF) {
+#pragma unroll
+            for (int j = 0; j < PF; j++) step(v + j, j, false);
+        }
+        // (whole trips in the loop, the rest after it)
+        int v = n1;
+        for (; v + PF <= nwalk + 1; v += PF) {
+#pragma unroll
+            for (int j = 0; j < PF; j++) step(v + j, j, true);
+        }
+#pragma unroll
+        for (int j = 0; j < PF - 1; j++) {
+            if (v + j > nwalk) return;
+            read_slot(slots, buf, ce);
+            look_ahead(raw[(j + 1) % PF], next_buf(buf));
+            cut(raw[j], buf, true);
+            buf = buf == 2 ? 0 : buf + 1;
+            wg_barrier();
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        return;
+    }
+
+    // =========================== consumers ===========================
+    const int ln = lane & 15, g = lane >> 4;
+    const uint32_t o_slb = (uint32_t)op.o_sl * 4;
+    char *o_seg = (char *)op.out + ((int64_t)n * op.o_sn + (int64_t)h * op.o_sh + F * fb) * 4;
+    const __amdgpu_buffer_rsrc_t o_rs =
+        __builtin_amdgcn_make_buffer_rsrc((void *)o_seg, 0, (rows - 1) * o_slb + fw * 4, kRsrcFlags);
+    // Pt quadrant of this wavefront (see scan_tp_kernel)
+    const int jh = w == 0 ? 0 : w == 1 ? 1 : ((w == 2) == REV ? 1 : 0);
+    const int ih = w == 0 ? 0 : w == 1 ? 1 : 1 - jh;
+    int a_addr[2][2], b_addr[2][2];  // [local i tile][ks], [ks][u]
+#pragma unroll
+    for (int ks = 0; ks < 2; ks++) {
+#pragma unroll
+        for (int x = 0; x < 2; x++)
+            a_addr[x][ks] = TpSwizzle<RBA>::addr(16 * (x ^ ih) + ln, 2 * (32 * ks + 8 * g));
+#pragma unroll
+        for (int u = 0; u < 2; u++)
+            b_addr[ks][u] = kOffB + TpSwizzle<RBA>::addr(
+                                        16 * jh + ln, 2 * b_tile_column(32 * ks + 8 * g + 4 * u));
+    }
+    int bt_addr[4][2], vt_addr[2];
+#pragma unroll
+    for (int u2 = 0; u2 < 2; u2++) {
+        const int row = 8 * g + (ln >> 2) + 4 * u2;
+#pragma unroll
+        for (int dt = 0; dt < 4; dt++)
+            bt_addr[dt][u2] = kOffB + TpSwizzle<RBA>::addr(
+                row, 2 * b_tile_column(32 * (dt / 2) + 4 * (dt % 2) + 8 * (ln & 3)));
+        vt_addr[u2] = kOffV + TpSwizzle<RBV>::addr(row, 2 * (16 * w + 4 * (ln & 3)));
+    }
+    const int pt_waddr = TpSwizzle<64>::addr(16 * ih + ln, 2 * (16 * jh + 4 * g));
+    int pt_raddr[2];
+#pragma unroll
+    for (int x = 0; x < 2; x++) pt_raddr[x] = TpSwizzle<64>::addr(16 * (x ^ ih) + ln, 16 * g);
+    uint32_t keep[4];
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+        const int j = 16 * jh + 4 * g + r, i = 16 * ih + ln;
+        keep[r] = (REV ? (j >= i) : (j <= i)) ? 0xffffffffu : 0u;
+        asm volatile("" : "+v"(keep[r]));
+    }
+    uint32_t o_lane[2];
+#pragma unroll
+    for (int x = 0; x < 2; x++)
+        o_lane[x] = (uint32_t)(16 * (x ^ ih) + ln) * o_slb + 4u * (16 * w + 4 * g);
+    const bool o_in = 16 * w + 4 * g < fw;  // (columns beyond the width are not stored)
+
+    constexpr int NT = 2 * KS;  // state tiles of 16 rows
+    f32x4 S[4];                 // the slab, in units of 2^Ucur
+#pragma unroll
+    for (int dt = 0; dt < 4; dt++) S[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    int Ucur = 0;
+    constexpr int kPa[3] = {1, 0, 0}, kPb[3] = {0, 1, 0};  // piece products, smallest first
+    auto state_row = [&](int dt, int r) -> int { return 32 * (dt / 2) + 8 * g + 4 * (dt % 2) + r; };
+    const bool st_in = 16 * w + ln < fw;
+    auto scale_state = [&](int e) {  // S <- S 2^e
+#pragma unroll
+        for (int dt = 0; dt < NT; dt++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) S[dt][r] = __builtin_amdgcn_ldexpf(S[dt][r], e);
+    };
+    auto add_caller_state = [&]() {  // in units of 2^Ucur
+        const float *base =
+            op.s0 + (int64_t)n * op.s0_sn + (int64_t)h * op.s0_sh + F * fb + 16 * w + ln;
+#pragma unroll
+        for (int dt = 0; dt < NT; dt++) {
+            float x[4];
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                const int d = state_row(dt, r);
+                const bool in = st_in && d < Dw;
+                x[r] = *(in ? base + (int64_t)d * op.s0_sd : op.s0);
+                x[r] = in ? __builtin_amdgcn_ldexpf(x[r], -Ucur) : 0.f;
+            }
+            S[dt] += f32x4{x[0], x[1], x[2], x[3]};
+        }
+    };
+
+    Frag af[2][2][2], bfr[2][2], bt[4][2], vf[2];
+    // row-major fragment number i of a chunk (12: b for the quadrant first, then a)
+    auto rm_frag = [&](const lds_char *pc, int i) {
+        const int k = i % 2, ks = (i / 2) % 2, x = i / 4;
+        if (ks >= KS) return;
+#ifdef FTC_ABL_NOLDSR
+        if (x == 0) asm volatile("" : "=v"(bfr[ks][k].w[0]), "=v"(bfr[ks][k].w[1]), "=v"(bfr[ks][k].w[2]), "=v"(bfr[ks][k].w[3]));
+        else asm volatile("" : "=v"(af[x - 1][ks][k].w[0]), "=v"(af[x - 1][ks][k].w[1]), "=v"(af[x - 1][ks][k].w[2]), "=v"(af[x - 1][ks][k].w[3]));
+        return;
+#endif
+        if (x == 0)
+            bfr[ks][k] = lds_frag8x2(pc + k * kTileA + b_addr[ks][0], pc + k * kTileA + b_addr[ks][1]);
+        else
+            af[x - 1][ks][k] = lds_frag16(pc + k * kTileA + a_addr[x - 1][ks]);
+    };
+    // position-major fragment number i of a chunk (10: v first, then b^T tile by tile)
+    auto tr_frag_into = [&](Frag (&btx)[4][2], Frag (&vfx)[2], const lds_char *pc, int i) {
+        if (i >= 2 && (i - 2) / 4 >= KS) return;  // tiles 2, 3: rows 32 .. 63
+#ifdef FTC_ABL_NOLDSR
+        {
+            Frag &f = i < 2 ? vfx[i] : btx[(i - 2) / 2][(i - 2) % 2];
+            asm volatile("" : "=v"(f.w[0]), "=v"(f.w[1]), "=v"(f.w[2]), "=v"(f.w[3]));
+            return;
+        }
+#endif
+        if (i < 2)
+            vfx[i] = lds_frag_tr(pc + i * kTileV + vt_addr[0], pc + i * kTileV + vt_addr[1]);
+        else {
+            const int dt = (i - 2) / 2, k = (i - 2) % 2;
+            btx[dt][k] = lds_frag_tr(pc + k * kTileA + bt_addr[dt][0], pc + k * kTileA + bt_addr[dt][1]);
+        }
+    };
+    int buf = B0;  // LDS buffer of the chunk at hand
+    wg_barrier();  // the slots are zero
+    if (n1 > 0) {
+        // ---- the first n1 positions of the walk: state update only ----
+        // Rows 16 .. 31 of b and v of these chunks are fetched and cut by the consumers (lane
+        // 64 w + lane takes the quad that producer lane of the same number would take).  The
+        // loop is skewed by one chunk: while the matrix instructions of position k - 1 run,
+        // the fragments of position k arrive in the other set of registers and position
+        // k + 1 is cut.
+        const int cid = w * 64 + lane, crow = (T + cid) / QA, cc4 = (T + cid) % QA;
+        const uint32_t b_slb = (uint32_t)op.b_sl * 4, v_slb = (uint32_t)op.v_sl * 4;
+        const char *b_seg = (const char *)op.b + ((int64_t)n * op.b_sn + (int64_t)h * op.b_sh) * 4;
+        const char *v_seg = (const char *)op.v +
+                            ((int64_t)n * op.v_sn + (int64_t)h * op.v_sh + F * fb) * 4;
+        const __amdgpu_buffer_rsrc_t b_rs = __builtin_amdgcn_make_buffer_rsrc(
+            (void *)b_seg, 0, (rows - 1) * b_slb + Dw * 4, kRsrcFlags);
+        const __amdgpu_buffer_rsrc_t v_rs = __builtin_amdgcn_make_buffer_rsrc(
+            (void *)v_seg, 0, (rows - 1) * v_slb + fw * 4, kRsrcFlags);
+        const bool b_in = 4 * cc4 < Dw;
+        const bool v_in = 4 * cc4 < fw;
+        const uint32_t b_goff = (uint32_t)crow * b_slb + 16u * cc4,
+                       v_goff = (uint32_t)crow * v_slb + 16u * cc4;
+        const int b_waddr = TpSwizzle<RBA>::addr(crow, 2 * b_tile_column(4 * cc4)),
+                  v_waddr = TpSwizzle<RBV>::addr(crow, 8 * cc4);
+        struct RawC {
+            u32x4 b, v;
+        };
+        RawC rawc[PF];
+        auto cfetch = [&](RawC &r, int v) {
+#ifdef FTC_ABL_NOMEM
+            v = n1 + 100;
+#endif
+            const int row0 = v < n1 ? chunk_row0(so_chunk(v)) : -2 * kChunk;
+            r.b = __builtin_amdgcn_raw_buffer_load_b128(
+                b_rs, b_in ? b_goff + (uint32_t)row0 * b_slb : kNoRow, 0, 0);
+            r.v = __builtin_amdgcn_raw_buffer_load_b128(
+                v_rs, v_in ? v_goff + (uint32_t)row0 * v_slb : kNoRow, 0, 0);
+        };
+        auto clook = [&](const RawC &r, int k) {
+            raise_slot(slots, k, ce, 0.f, max_abs4(r.b, 0.f), max_abs4(r.v, 0.f), lane);
+        };
+        auto ccut_b = [&](const RawC &r, int bufk) {
+            cut_quad_to_lds(r.b, ce.scale_b(), unit_pc + bufk * kBufBytes + kOffB, kTileA, b_waddr);
+        };
+        auto ccut_v = [&](const RawC &r, int bufk) {
+            cut_quad_to_lds(r.v, ce.scale_v(), unit_pc + bufk * kBufBytes + kOffV, kTileV, v_waddr);
+        };
+#pragma unroll
+        for (int j = 0; j < PF; j++) cfetch(rawc[j], j);
+        clook(rawc[0], B0);
+        wg_barrier();  // the slot of position 0 is complete
+        read_slot(slots, B0, ce);
+        ccut_b(rawc[0], B0);
+        ccut_v(rawc[0], B0);
+        clook(rawc[1], next_buf(B0));
+        cfetch(rawc[0], PF);
+        wg_barrier();  // barrier 0
+        Ucur = ce.state_exp();
+        if (op.s0 && !exchange) add_caller_state();
+        int U_frag = Ucur;  // units of the fragments about to be multiplied (position k - 1)
+        int U_load = Ucur;  // units of the fragments being loaded (position k)
+        Frag bt2[4][2] = {}, vf2[2] = {};  // (the first round multiplies zeros)
+        int bufn = next_buf(B0);           // LDS buffer of the position after the one at hand
+        for (int c = 0; c < n1; c += PF) {
+#pragma unroll
+            for (int j = 0; j < PF; j++) {
+                const lds_char *pc = unit_pc + buf * kBufBytes;
+                // position c + j + 1 is cut under the matrix instructions of position
+                // c + j - 1 (position n1 is all the producers')
+                const bool cut_next = j < PF - 1 || c + PF < n1;
+                const RawC &rn = rawc[(j + 1) % PF];
+                read_slot(slots, bufn, ce);  // the ceilings of position c + j + 1
+                if (U_frag != Ucur) {               // the ceilings rose: the state shrinks
+                    scale_state(Ucur - U_frag);
+                    Ucur = U_frag;
+                }
+#pragma unroll
+                for (int i = 0; i < 12; i++) {
+                    const bool rows_exist = (i % 4) / 2 < KS;
+                    if (j % 2 == 0) {
+                        if (rows_exist) S[i % 4] = mfma16h(bt2[i % 4][kPa[i / 4]], vf2[kPb[i / 4]], S[i % 4]);
+                        if (i < 10) tr_frag_into(bt, vf, pc, i);
+                    } else {
+                        if (rows_exist) S[i % 4] = mfma16h(bt[i % 4][kPa[i / 4]], vf[kPb[i / 4]], S[i % 4]);
+                        if (i < 10) tr_frag_into(bt2, vf2, pc, i);
+                    }
+                    if (i == 6 && cut_next) ccut_b(rn, bufn);
+                    if (i == 9 && cut_next) ccut_v(rn, bufn);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+                clook(rawc[(j + 2) % PF], next_buf(bufn));
+                cfetch(rawc[(j + 1) % PF], c + j + 1 + PF);
+                U_frag = U_load;
+                U_load = ce.state_exp();
+                buf = bufn;
+                bufn = next_buf(bufn);
+                wg_barrier();
+#ifdef FTC_TIMELINE
+                if (stamp_on && c + j < 30) chunk_stamps[32 + c + j] = __builtin_amdgcn_s_memrealtime();
+#endif
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+        // the last of these positions (n1 is even: its fragments are in the second set)
+        if (U_frag != Ucur) {
+            scale_state(Ucur - U_frag);
+            Ucur = U_frag;
+        }
+#pragma unroll
+        for (int i = 0; i < 12; i++) {
+            if ((i % 4) / 2 < KS) S[i % 4] = mfma16h(bt2[i % 4][kPa[i / 4]], vf2[kPb[i / 4]], S[i % 4]);
+            rm_frag(unit_pc + buf * kBufBytes, i);  // our own first chunk is cut
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        // (the slot of position n1 was read in the last round)
+    } else {
+        wg_barrier();  // the slot of position 0 is complete
+        wg_barrier();  // barrier 0
+        read_slot(slots, 0, ce);  // (B0 = 0)
+        Ucur = ce.state_exp();
+        if (op.s0 && !exchange) add_caller_state();
+#pragma unroll
+        for (int i = 0; i < 12; i++) rm_frag(unit_pc, i);
+    }
+    if (exchange) {
+        // ---- the sum of this segment's rows goes out, the state before the segment comes in ----
+        const uint32_t total_units = (uint32_t)p.total_waves;
+        gfloat *const sums = (gfloat *)(hdr + kControlBytes / 4);
+        StateExchange<1, 1> xch(flags, sums, 4u * total_units,
+                                (uint32_t)w * total_units + chain_id * nseg + (uint32_t)seg, seg,
+                                (int)nseg, p.group, lane);
+        f32x16 Sx[1][1], X[1][1];
+#pragma unroll
+        for (int dt = 0; dt < 4; dt++)
+#pragma unroll
+            for (int r = 0; r < 4; r++)
+                Sx[0][0][4 * dt + r] = dt < NT ? __builtin_amdgcn_ldexpf(S[dt][r], Ucur) : 0.f;
+        if (n1 > 0) xch.publish_sum(Sx);
+        xch.gather(Sx, X);
+        if (xch.failed && lane == 0)
+            __hip_atomic_store(hdr + kHdrError, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        // the units of the first chunk of the second pass (its ceilings are already known)
+        Ucur = ce.state_exp();
+#pragma unroll
+        for (int dt = 0; dt < NT; dt++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) S[dt][r] = __builtin_amdgcn_ldexpf(X[0][0][4 * dt + r], -Ucur);
+        if (op.s0) add_caller_state();
+    }
+    // ---- the walk proper ----
+    // `ce` holds the ceilings of the chunk at hand, Ucur the units of S.  dU <= 0: the
+    // state's units rise by -dU with this chunk (S is rescaled once all of it has been cut).
+    int dU = Ucur - ce.state_exp();
+    int s = 0;  // S is cut as S 2^(dU - s)
+    auto lane_max_state = [&]() -> float {
+        float m = 0.f;
+#pragma unroll
+        for (int dt = 0; dt < NT; dt++)
+            m = fmaxf(fmaxf(fmaxf(fabsf(S[dt][0]), fabsf(S[dt][1])), fmaxf(fabsf(S[dt][2]), fabsf(S[dt][3]))), m);
+        return m;
+    };
+    {
+        if (dU != 0) {
+            scale_state(dU);
+            Ucur -= dU;
+            dU = 0;
+        }
+        const float m = lane_max_state();
+        while (s < 100 && __builtin_amdgcn_ballot_w64(m > pow2_field(127 + 14 + s)) != 0) s++;
+    }
+    float kappa = pow2_field(127 + dU - s);  // scale of the cut of S
+    int s_cut = s;                            // ... and the s that went into it
+    float mS = 0.f;                           // largest |S| seen while cutting
+    Frag sf[2][2];
+    auto cut_s = [&](int ks, int q) {
+#ifdef FTC_ABL_NOCUTS
+        asm volatile("" : "=v"(sf[ks][0].w[q]), "=v"(sf[ks][1].w[q]) : "v"(S[2 * ks + q / 2][2 * (q % 2)]));
+        return;
+#endif
+        const float x0 = S[2 * ks + q / 2][2 * (q % 2)], x1 = S[2 * ks + q / 2][2 * (q % 2) + 1];
+        mS = fmaxf(fmaxf(fabsf(x0), fabsf(x1)), mS);
+        cut_pair_f16(x0, x1, kappa, sf[ks][0].w[q], sf[ks][1].w[q]);
+    };
+#pragma unroll
+    for (int q = 0; q < 4; q++) cut_s(0, q);
+
+    // Ot_w of the chunk before in the units of that chunk (exponent Xo), and where its rows
+    // go (before the first chunk: nowhere)
+    f32x4 O[2];
+#pragma unroll
+    for (int x = 0; x < 2; x++) O[x] = f32x4{0.f, 0.f, 0.f, 0.f};
+    int Xo = 0;
+    uint32_t o_off = 0x80000000u;
+    auto store_rows = [&](int x) {
+#ifdef FTC_ABL_NOSTORE
+        asm volatile("" ::"v"(O[x]));
+        return;
+#endif
+        const u32x4 r = {__float_as_uint(__builtin_amdgcn_ldexpf(O[x][0], Xo)),
+                         __float_as_uint(__builtin_amdgcn_ldexpf(O[x][1], Xo)),
+                         __float_as_uint(__builtin_amdgcn_ldexpf(O[x][2], Xo)),
+                         __float_as_uint(__builtin_amdgcn_ldexpf(O[x][3], Xo))};
+        __builtin_amdgcn_raw_buffer_store_b128(r, o_rs, o_in ? o_off + o_lane[x] : kNoRow, 0, 0);
+    };
+    const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
+    // One chunk, in LDS buffer B (a compile-time number, so that every LDS access of the body
+    // has its buffer in the instruction's immediate offset).  Sums that end in one place are
+    // chained through one accumulator, with other matrix instructions in between: Ot_w =
+    // (S_w^T a^T) 2^s + v_w^T Pt needs no addition at all while s = 0, which is the rule.
+    auto chunk_body = [&](int c, auto buffer_number) {
+        constexpr int B = decltype(buffer_number)::value, BN = (B + 1) % 3;
+        const lds_char *pc = unit_pc + B * kBufBytes;
+        const lds_char *pn = unit_pc + BN * kBufBytes;
+        lds_char *const ptc = pt_pc + B * (2 * kTileP);
+        Frag pf[2][2];
+        f32x4 P = zero;
+        if (c == c0 + 4) FTC_STAMP(0);
+        __builtin_amdgcn_sched_barrier(0);
+        // phase 1: (1) the quadrant in turn with (2b) Ot_w = S_w^T a^T for rows 0 .. 31 of
+        // the state; underneath: the rows of the chunk before go out, tiles 2, 3 of S_w are
+        // cut into pieces, the position-major reads
+#pragma unroll
+        for (int i = 0; i < 6; i++) {
+            const int m = i % 3, ks = i / 3, x = i % 2, mo = i / 2;
+            if (i == 0) store_rows(0);
+            if (i == 1) store_rows(1);
+            if (ks < KS) P = mfma16h(bfr[ks][kPa[m]], af[0][ks][kPb[m]], P);
+            O[x] = mfma16h(sf[0][kPa[mo]], af[x][0][kPb[mo]], mo == 0 ? zero : O[x]);
+            if (i < 4 && KS > 1) cut_s(1, i);
+            tr_frag_into(bt, vf, pc, i);
+            if (i < 4) tr_frag_into(bt, vf, pc, 6 + i);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        if (c == c0 + 4) FTC_STAMP(1);
+        // all of S is cut: it takes the units of this chunk, and s follows its size
+        if (dU != 0) {
+            scale_state(dU);
+            mS = __builtin_amdgcn_ldexpf(mS, dU);
+            s = max(0, s + dU);
+            Ucur -= dU;
+        }
+        while (s < 100 && __builtin_amdgcn_ballot_w64(mS > pow2_field(127 + 14 + s)) != 0) s++;
+        mS = 0.f;
+        if (c == c0 + 4) FTC_STAMP(2);
+        __builtin_amdgcn_sched_barrier(0);
+        // phase 2: (2b) for rows 32 .. 63 in turn with (3) S_w += b^T v_w for tiles 0 and 1;
+        // underneath: the quadrant is masked, cut and handed to the others
+#pragma unroll
+        for (int i = 0; i < 6; i++) {
+            const int x = i % 2, m = i / 2;
+            if (KS > 1) O[x] = mfma16h(sf[1][kPa[m]], af[x][1][kPb[m]], O[x]);
+            S[i % 2] = mfma16h(bt[i % 2][kPa[m]], vf[kPb[m]], S[i % 2]);
+            if (i == 1) {
+                uint32_t h0, l0, h1, l1;
+                cut_pair_f16_unscaled(__uint_as_float(__float_as_uint(P[0]) & keep[0]),
+                                      __uint_as_float(__float_as_uint(P[1]) & keep[1]), h0, l0);
+                cut_pair_f16_unscaled(__uint_as_float(__float_as_uint(P[2]) & keep[2]),
+                                      __uint_as_float(__float_as_uint(P[3]) & keep[3]), h1, l1);
+                const u32x2 wh = {h0, h1}, wl = {l0, l1};
+                *(lds_vec2 *)(ptc + pt_waddr) = wh;
+                *(lds_vec2 *)(ptc + kTileP + pt_waddr) = wl;
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        if (c == c0 + 4) FTC_STAMP(4);
+        wg_barrier();
+        if (c == c0 + 4) FTC_STAMP(5);
+#ifdef FTC_TIMELINE
+        if (stamp_on && c - c0 < 30) chunk_stamps[c - c0 + 1] = __builtin_amdgcn_s_memrealtime();
+#endif
+        // All of Pt is in LDS, the next chunk is cut and its slot complete.
+        // phase 3: (3) for tiles 2 and 3, then (2a) Ot_w += v_w^T Pt; underneath: the next
+        // chunk's row-major fragments are requested and tiles 0, 1 of S_w cut into pieces
+#pragma unroll
+        for (int x = 0; x < 2; x++)
+#pragma unroll
+            for (int k = 0; k < 2; k++) pf[x][k] = lds_frag16(ptc + k * kTileP + pt_raddr[x]);
+        const int Xc = ce.out_exp();
+        const u32x4 slot_next = *(const lds_vec4 *)(slots + 4 * BN);
+        if (s_cut != 0) {  // (rare: the state has grown beyond 2^14 units)
+            const float r_cut = pow2_field(127 + s_cut);
+            O[0] *= r_cut;
+            O[1] *= r_cut;
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int i = 0; i < 6; i++) {
+            const int m = i / 2;
+            if (KS > 1) S[2 + i % 2] = mfma16h(bt[2 + i % 2][kPa[m]], vf[kPb[m]], S[2 + i % 2]);
+            rm_frag(pn, 2 * i);
+            rm_frag(pn, 2 * i + 1);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        // the ceilings of the next chunk
+        ce.Ea = max(ce.Ea, (uint32_t)__builtin_amdgcn_readfirstlane(slot_next.x));
+        ce.Eb = max(ce.Eb, (uint32_t)__builtin_amdgcn_readfirstlane(slot_next.y));
+        ce.Ev = max(ce.Ev, (uint32_t)__builtin_amdgcn_readfirstlane(slot_next.z));
+        dU = Ucur - ce.state_exp();
+        kappa = pow2_field(127 + dU - s);
+        s_cut = s;
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int i = 0; i < 6; i++) {
+            const int x = i % 2, m = i / 2;
+            O[x] = mfma16h(vf[kPa[m]], pf[x][kPb[m]], O[x]);
+            if (i < 4) cut_s(0, i);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        o_off = (uint32_t)chunk_row0(c) * o_slb;
+        Xo = Xc;
+        if (c == c0 + 4) FTC_STAMP(6);
+    };
+    {
+        int c = c0;
+#ifndef FTC_ABL_NOCONS
+        for (; c + 3 <= nchunks; c += 3) {
+            chunk_body(c, std::integral_constant<int, 0>());
+            chunk_body(c + 1, std::integral_constant<int, 1>());
+            chunk_body(c + 2, std::integral_constant<int, 2>());
+        }
+        if (c < nchunks) chunk_body(c++, std::integral_constant<int, 0>());
+        if (c < nchunks) chunk_body(c++, std::integral_constant<int, 1>());
+#else
+        for (; c < nchunks; c++) wg_barrier();
+#endif
+    }
+    store_rows(0);
+    store_rows(1);
+    FTC_STAMP(15);  // last rows on their way
+    if (op.s_out && seg == (int)nseg - 1) {
+        float *base =
+            op.s_out + (int64_t)n * op.so_sn + (int64_t)h * op.so_sh + F * fb + 16 * w + ln;
+#pragma unroll
+        for (int dt = 0; dt < NT; dt++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                const int d = state_row(dt, r);
+                if (st_in && d < Dw) base[(int64_t)d * op.so_sd] = __builtin_amdgcn_ldexpf(S[dt][r], Ucur);
+            }
+    }
+    // the last consumer of the launch leaves the control block zeroed
+    if (exchange) {
+        const uint32_t total_units = (uint32_t)p.total_waves;
+        uint32_t done = 0;
+        if (lane == 0)
+            done = __hip_atomic_fetch_add(hdr + kHdrDone, 1u, __ATOMIC_RELAXED,
+                                          __HIP_MEMORY_SCOPE_AGENT);
+        done = __builtin_amdgcn_readfirstlane(done);
+        if (done == 4u * total_units - 1) {
+            for (uint32_t i = lane; i < 4u * total_units; i += kWave)
+                __hip_atomic_store(flags + i, kFlagEmpty, __ATOMIC_RELAXED,
+                                   __HIP_MEMORY_SCOPE_AGENT);
+            for (uint32_t i = lane; i < total_units / nseg; i += kWave)
+                __hip_atomic_store(flags + kMaxWaves + i, 0u, __ATOMIC_RELAXED,
+                                   __HIP_MEMORY_SCOPE_AGENT);
+            if (lane == 0)
+                __hip_atomic_store(hdr + kHdrDone, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+    }
+}
+
+}  // namespace mfma
+}  // namespace ftc
