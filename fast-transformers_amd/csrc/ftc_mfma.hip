@@ -473,7 +473,13 @@ int mfma_scan(const ScanDesc *scans, int nscans, int64_t N, int64_t H, int64_t L
     // fp32 states of up to 64 rows: the kernel that feeds its fragments from LDS tiles
     bool dma = D <= 64 && combo == kFFFF;
     if (const char *env = getenv("FTC_DMA")) dma = dma && atoi(env) != 0;  // tuning aid
-    note_kernel(tp ? (tpx_seg_chunks > 0 ? "scan_tp_kernel (exchange)" : "scan_tp_kernel") : wg ? (fused ? "scan_wg_kernel<NORM>" : "scan_wg_kernel")
+    // chain-parallel scans of states of up to 64 rows run on the fp16 matrix path
+    // (ftc_tph_kernel.h: two scaled fp16 pieces per value), wider ones on three bf16 pieces
+    bool half_pieces = tp && D <= 64;
+    if (const char *env = getenv("FTC_TPH")) half_pieces = half_pieces && atoi(env) != 0;  // tuning aid
+    note_kernel(tp ? (half_pieces ? (tpx_seg_chunks > 0 ? "scan_tph_kernel (exchange)" : "scan_tph_kernel")
+                                  : (tpx_seg_chunks > 0 ? "scan_tp_kernel (exchange)" : "scan_tp_kernel"))
+                : wg ? (fused ? "scan_wg_kernel<NORM>" : "scan_wg_kernel")
                 : dma ? "scan_dma_kernel" : "scan_mfma_kernel");
     if (plan_only()) {
         char cuts[160] = "";
@@ -490,8 +496,6 @@ int mfma_scan(const ScanDesc *scans, int nscans, int64_t N, int64_t H, int64_t L
         return FTC_OK;
     }
     if (tp) {
-        bool half_pieces = D <= 64;
-        if (const char *env = getenv("FTC_TPH")) half_pieces = half_pieces && atoi(env) != 0;  // tuning aid
         if (half_pieces)
             launch_scan_tph(workspace, args, stream);
         else

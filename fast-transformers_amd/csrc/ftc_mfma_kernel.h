@@ -450,7 +450,10 @@ constexpr int kMaxScans = kMfmaMaxScans;
 
 constexpr int kMaxTpSegments = 16;
 // chunks that the chain-parallel kernel requests ahead (measured on cfg2: 6 and 8 are slower)
-constexpr int kTpAhead = 4;
+#ifndef FTC_TP_AHEAD
+#define FTC_TP_AHEAD 4
+#endif
+constexpr int kTpAhead = FTC_TP_AHEAD;
 
 struct ScanArgs {
     ScanOperands scan[kMaxScans];

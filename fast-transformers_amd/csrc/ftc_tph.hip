@@ -6,7 +6,7 @@ namespace mfma {
 
 void launch_scan_tph(void *ws, const ScanArgs &args, hipStream_t stream) {
     // (grid as for launch_scan_tp)
-    const dim3 grid((unsigned)args.total_waves), block(512);
+    const dim3 grid((unsigned)args.total_waves), block(768);
     if (args.tp_d <= 32)
         hipLaunchKernelGGL((scan_tph_kernel<1>), grid, block, 0, stream, (uint32_t *)ws, args);
     else

@@ -50,41 +50,49 @@ namespace mfma {
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 
 __device__ __forceinline__ f32x4 mfma16h(const Frag &a, const Frag &b, f32x4 c) {
-#ifdef FTC_ABL_NOMFMA
-    asm volatile("" ::"v"(a.w[0]), "v"(b.w[0]));
-    asm volatile("" : "+v"(c));
-    return c;
-#endif
     return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a),
                                                   __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
 }
 
-// Two fp32 values times a power of two -> packed fp16 pieces (x0 in the low half), both
+// Four fp32 values times a power of two -> packed fp16 pieces (x0, x2 in the low halves), all
 // rounded to nearest even.  v_fma_mix{lo,hi}_f16 computes fma(x, s, c) in fp32 (exact here:
 // x s is exact, and so is the remainder of a rounding) and rounds once to fp16; the third
-// operand is the fp16 hi piece, read from the half that op_sel names and negated.
-__device__ __forceinline__ void cut_pair_f16(float x0, float x1, float s, uint32_t &hi, uint32_t &lo) {
-    asm("v_fma_mixlo_f16 %0, %1, %2, 0" : "=v"(hi) : "v"(x0), "s"(s));
-    asm("v_fma_mixhi_f16 %0, %1, %2, 0" : "+v"(hi) : "v"(x1), "s"(s));
-    asm("v_fma_mixlo_f16 %0, %1, %2, -%3 op_sel:[0,0,0] op_sel_hi:[0,0,1]"
-        : "=v"(lo) : "v"(x0), "s"(s), "v"(hi));
-    asm("v_fma_mixhi_f16 %0, %1, %2, -%3 op_sel:[0,0,1] op_sel_hi:[0,0,1]"
-        : "+v"(lo) : "v"(x1), "s"(s), "v"(hi));
+// operand is the fp16 hi piece, read from the half that op_sel names and negated.  The two
+// pairs are cut in turn, so that no instruction reads (or completes) a half-written register
+// right after the instruction that wrote it: that costs a wait state each time.
+__device__ __forceinline__ void cut_quad_f16(float x0, float x1, float x2, float x3, float s,
+                                             uint32_t &h01, uint32_t &h23, uint32_t &l01,
+                                             uint32_t &l23) {
+    asm("v_fma_mixlo_f16 %0, %4, %8, 0\n\t"
+        "v_fma_mixlo_f16 %1, %6, %8, 0\n\t"
+        "v_fma_mixhi_f16 %0, %5, %8, 0\n\t"
+        "v_fma_mixhi_f16 %1, %7, %8, 0\n\t"
+        "v_fma_mixlo_f16 %2, %4, %8, -%0 op_sel:[0,0,0] op_sel_hi:[0,0,1]\n\t"
+        "v_fma_mixlo_f16 %3, %6, %8, -%1 op_sel:[0,0,0] op_sel_hi:[0,0,1]\n\t"
+        "v_fma_mixhi_f16 %2, %5, %8, -%0 op_sel:[0,0,1] op_sel_hi:[0,0,1]\n\t"
+        "v_fma_mixhi_f16 %3, %7, %8, -%1 op_sel:[0,0,1] op_sel_hi:[0,0,1]"
+        : "=&v"(h01), "=&v"(h23), "=&v"(l01), "=&v"(l23)
+        : "v"(x0), "v"(x1), "v"(x2), "v"(x3), "v"(s));
 }
-// the same without a scale: one packed conversion for the hi pieces
-__device__ __forceinline__ void cut_pair_f16_unscaled(float x0, float x1, uint32_t &hi, uint32_t &lo) {
-    asm("v_cvt_pk_f16_f32 %0, %1, %2" : "=v"(hi) : "v"(x0), "v"(x1));
-    asm("v_fma_mixlo_f16 %0, %1, 1.0, -%2 op_sel:[0,0,0] op_sel_hi:[0,0,1]"
-        : "=v"(lo) : "v"(x0), "v"(hi));
-    asm("v_fma_mixhi_f16 %0, %1, 1.0, -%2 op_sel:[0,0,1] op_sel_hi:[0,0,1]"
-        : "+v"(lo) : "v"(x1), "v"(hi));
+// the same without a scale: one packed conversion per pair for the hi pieces
+__device__ __forceinline__ void cut_quad_f16_unscaled(float x0, float x1, float x2, float x3,
+                                                      uint32_t &h01, uint32_t &h23, uint32_t &l01,
+                                                      uint32_t &l23) {
+    asm("v_cvt_pk_f16_f32 %0, %4, %5\n\t"
+        "v_cvt_pk_f16_f32 %1, %6, %7\n\t"
+        "v_fma_mixlo_f16 %2, %4, 1.0, -%0 op_sel:[0,0,0] op_sel_hi:[0,0,1]\n\t"
+        "v_fma_mixlo_f16 %3, %6, 1.0, -%1 op_sel:[0,0,0] op_sel_hi:[0,0,1]\n\t"
+        "v_fma_mixhi_f16 %2, %5, 1.0, -%0 op_sel:[0,0,1] op_sel_hi:[0,0,1]\n\t"
+        "v_fma_mixhi_f16 %3, %7, 1.0, -%1 op_sel:[0,0,1] op_sel_hi:[0,0,1]"
+        : "=&v"(h01), "=&v"(h23), "=&v"(l01), "=&v"(l23)
+        : "v"(x0), "v"(x1), "v"(x2), "v"(x3));
 }
 // Four consecutive fp32 values of a row -> 8 bytes of each of the two piece tiles.
 __device__ __forceinline__ void cut_quad_to_lds(const u32x4 raw, float s, lds_char *tile,
                                                 int piece_bytes, int addr) {
     uint32_t h0, l0, h1, l1;
-    cut_pair_f16(__uint_as_float(raw.x), __uint_as_float(raw.y), s, h0, l0);
-    cut_pair_f16(__uint_as_float(raw.z), __uint_as_float(raw.w), s, h1, l1);
+    cut_quad_f16(__uint_as_float(raw.x), __uint_as_float(raw.y), __uint_as_float(raw.z),
+                 __uint_as_float(raw.w), s, h0, h1, l0, l1);
     const u32x2 wh = {h0, h1}, wl = {l0, l1};
     *(lds_vec2 *)(tile + addr) = wh;
     *(lds_vec2 *)(tile + piece_bytes + addr) = wl;
@@ -150,9 +158,9 @@ __device__ __forceinline__ void raise_slot(lds_u32_t *slots, int k, const Ceilin
 // KS: groups of 32 rows of the state (1: a state of up to 32 rows, which skips the matrix
 // instructions and fragment reads of the empty half)
 template <int KS>
-__global__ __launch_bounds__(512, 1) void scan_tph_kernel(uint32_t *__restrict__ ws_ptr, ScanArgs p) {
+__global__ __launch_bounds__(768, 3) void scan_tph_kernel(uint32_t *__restrict__ ws_ptr, ScanArgs p) {
     constexpr int D = 64, F = 64;              // one block of state rows and of output columns
-    constexpr int T = 256;                     // producer lanes
+    constexpr int T = 512;                     // producer lanes (eight wavefronts)
     constexpr int PF = kTpAhead;               // chunks requested ahead
     constexpr int RBA = D * 2, RBV = F * 2;    // bytes per row of an fp16 piece tile
     constexpr int kTileA = kChunk * RBA, kTileV = kChunk * RBV;
@@ -161,13 +169,13 @@ __global__ __launch_bounds__(512, 1) void scan_tph_kernel(uint32_t *__restrict__
     constexpr int kTileP = kChunk * 64;        // Pt pieces: 32 rows (i) of 32 j
     constexpr int QA = D / 4, QV = F / 4;
     constexpr int LA = kChunk * QA / T, LV = kChunk * QV / T;
-    static_assert(kChunk == 32 && T % QA == 0 && T % QV == 0 && PF == 4, "shape");
+    static_assert(kChunk == 32 && T % QA == 0 && T % QV == 0, "shape");
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const bool producer = wave >= 4;
-    const int w = wave & 3;
+    const int w = wave & 3;  // (consumers)
 
     __shared__ __align__(16) char pieces_mem[3 * kBufBytes];
     __shared__ __align__(16) char pt_mem[3 * 2 * kTileP];
@@ -249,14 +257,12 @@ __global__ __launch_bounds__(512, 1) void scan_tph_kernel(uint32_t *__restrict__
     FTC_STAMP(14);  // workgroup under way
 #ifdef FTC_TIMELINE
     if (stamp_on && !producer) chunk_stamps[0] = __builtin_amdgcn_s_memrealtime();
+    if (stamp_on && !producer) stamp_base[12] = __builtin_amdgcn_s_memtime();
 #endif
 
     if (producer) {
         // =========================== producers ===========================
-#ifdef FTC_ABL_PRIO
-        __builtin_amdgcn_s_setprio(3);
-#endif
-        const int ptid = w * 64 + lane;
+        const int ptid = (wave - 4) * 64 + lane;
         const uint32_t a_slb = (uint32_t)op.a_sl * 4, b_slb = (uint32_t)op.b_sl * 4,
                        v_slb = (uint32_t)op.v_sl * 4;
         const char *a_seg = (const char *)op.a + ((int64_t)n * op.a_sn + (int64_t)h * op.a_sh) * 4;
@@ -269,78 +275,51 @@ __global__ __launch_bounds__(512, 1) void scan_tph_kernel(uint32_t *__restrict__
             (void *)b_seg, 0, (rows - 1) * b_slb + Dw * 4, kRsrcFlags);
         const __amdgpu_buffer_rsrc_t v_rs = __builtin_amdgcn_make_buffer_rsrc(
             (void *)v_seg, 0, (rows - 1) * v_slb + fw * 4, kRsrcFlags);
-        // widths that do not fill the block: a lane whose four columns lie beyond the width
-        // asks outside the descriptor and cuts zeros (widths are multiples of 4)
-        const bool ab_in = 4 * (ptid % QA) < Dw;
-        const bool v_in = 4 * (ptid % QV) < fw;
-        uint32_t a_goff[LA], b_goff[LA], v_goff[LV];
-        int a_waddr[LA], b_waddr[LA], v_waddr[LV];
-#pragma unroll
-        for (int q = 0; q < LA; q++) {
-            const int u = q * T + ptid, row = u / QA, c4 = u % QA;
-            a_goff[q] = (uint32_t)row * a_slb + 16u * c4;
-            b_goff[q] = (uint32_t)row * b_slb + 16u * c4;
-            a_waddr[q] = TpSwizzle<RBA>::addr(row, 8 * c4);
-            b_waddr[q] = TpSwizzle<RBA>::addr(row, 2 * b_tile_column(4 * c4));
-        }
-#pragma unroll
-        for (int q = 0; q < LV; q++) {
-            const int u = q * T + ptid, row = u / QV, c4 = u % QV;
-            v_goff[q] = (uint32_t)row * v_slb + 16u * c4;
-            v_waddr[q] = TpSwizzle<RBV>::addr(row, 8 * c4);
-        }
+        // One quad (four columns of one row) of every operand per lane and position.  Widths
+        // that do not fill the block: a lane whose four columns lie beyond the width asks
+        // outside the descriptor and cuts zeros (widths are multiples of 4).
+        static_assert(LA == 1 && LV == 1 && QA == QV, "one quad per lane");
+        const int prow = ptid / QA, pc4 = ptid % QA;
+        const bool ab_in = 4 * pc4 < Dw;
+        const bool v_in = 4 * pc4 < fw;
+        const uint32_t a_goff = (uint32_t)prow * a_slb + 16u * pc4,
+                       b_goff = (uint32_t)prow * b_slb + 16u * pc4,
+                       v_goff = (uint32_t)prow * v_slb + 16u * pc4;
+        const int a_waddr = TpSwizzle<RBA>::addr(prow, 8 * pc4),
+                  b_waddr = TpSwizzle<RBA>::addr(prow, 2 * b_tile_column(4 * pc4)),
+                  v_waddr = TpSwizzle<RBV>::addr(prow, 8 * pc4);
         struct Raw {
-            u32x4 a[LA], b[LA], v[LV];
+            u32x4 a, b, v;
         };
         Raw raw[PF];
-        // Every request is made every time, whether its rows exist or not (of a chunk walked
-        // for its state alone the producers need rows 0 .. 15 of b and v only; positions past
-        // the end of the walk have no rows): a request outside the descriptor costs no memory
-        // traffic and reads as zero, and with a fixed number of requests per chunk the
-        // compiler can wait for the oldest ones only.
-        static_assert(LA == 2 && LV == 2, "quad 0 of a lane: rows 0 .. 15, quad 1: rows 16 .. 31");
+        // Every request is made every time, whether its rows exist or not (a chunk walked for
+        // its state alone needs no rows of a; positions past the end of the walk have no
+        // rows): a request outside the descriptor costs no memory traffic and reads as zero,
+        // and with a fixed number of requests per chunk the compiler can wait for the oldest
+        // ones only.
         auto fetch = [&](Raw &r, int v) {  // v: position of the walk
-#ifdef FTC_ABL_NOMEM
-            v = nwalk + 100;
-#endif
             const int row0 = v < nwalk ? chunk_row0(walk_chunk(v)) : -2 * kChunk;
             const int row0_x = v >= n1 ? row0 : -2 * kChunk;
-#pragma unroll
-            for (int q = 0; q < LA; q++) {
-                r.a[q] = __builtin_amdgcn_raw_buffer_load_b128(
-                    a_rs, ab_in ? a_goff[q] + (uint32_t)row0_x * a_slb : kNoRow, 0, 0);
-                r.b[q] = __builtin_amdgcn_raw_buffer_load_b128(
-                    b_rs, ab_in ? b_goff[q] + (uint32_t)(q == 0 ? row0 : row0_x) * b_slb : kNoRow, 0, 0);
-            }
-#pragma unroll
-            for (int q = 0; q < LV; q++)
-                r.v[q] = __builtin_amdgcn_raw_buffer_load_b128(
-                    v_rs, v_in ? v_goff[q] + (uint32_t)(q == 0 ? row0 : row0_x) * v_slb : kNoRow, 0, 0);
+            r.a = __builtin_amdgcn_raw_buffer_load_b128(
+                a_rs, ab_in ? a_goff + (uint32_t)row0_x * a_slb : kNoRow, 0, 0);
+            r.b = __builtin_amdgcn_raw_buffer_load_b128(
+                b_rs, ab_in ? b_goff + (uint32_t)row0 * b_slb : kNoRow, 0, 0);
+            r.v = __builtin_amdgcn_raw_buffer_load_b128(
+                v_rs, v_in ? v_goff + (uint32_t)row0 * v_slb : kNoRow, 0, 0);
         };
-        // the largest magnitudes of the rows of position k against the ceilings (rows that
-        // were not asked for read as zeros)
+        // the largest magnitudes of the rows of a position against the ceilings (rows that
+        // were not asked for read as zeros); k: that position's slot
         auto look_ahead = [&](const Raw &r, int k) {
-            float ma = 0.f, mb = 0.f, mv = 0.f;
-#pragma unroll
-            for (int q = 0; q < LA; q++) ma = max_abs4(r.a[q], ma), mb = max_abs4(r.b[q], mb);
-#pragma unroll
-            for (int q = 0; q < LV; q++) mv = max_abs4(r.v[q], mv);
-            raise_slot(slots, k, ce, ma, mb, mv, lane);
+            raise_slot(slots, k, ce, max_abs4(r.a, 0.f), max_abs4(r.b, 0.f), max_abs4(r.v, 0.f), lane);
         };
-        // position k of the walk goes to its LDS buffer through register set k % PF.  The
-        // first n1 positions only feed the state: no piece of a, and the consumers cut rows
-        // 16 .. 31 of b and v themselves.
+        // A position of the walk goes to its LDS buffer through register set (position % PF).
+        // The first n1 positions only feed the state: no piece of a.
         auto cut = [&](const Raw &r, int buf, bool own) {
             lds_char *const pc = unit_pc + buf * kBufBytes;
-            const float sa = ce.scale_a(), sb = ce.scale_b(), sv = ce.scale_v();
-#pragma unroll
-            for (int q = 0; q < LA; q++) {
-                if (own) cut_quad_to_lds(r.a[q], sa, pc, kTileA, a_waddr[q]);
-                if (own || q == 0) cut_quad_to_lds(r.b[q], sb, pc + kOffB, kTileA, b_waddr[q]);
-            }
-#pragma unroll
-            for (int q = 0; q < LV; q++)
-                if (own || q == 0) cut_quad_to_lds(r.v[q], sv, pc + kOffV, kTileV, v_waddr[q]);
+            if (own) cut_quad_to_lds(r.a, ce.scale_a(), pc, kTileA, a_waddr);
+            cut_quad_to_lds(r.b, ce.scale_b(), pc + kOffB, kTileA, b_waddr);
+            cut_quad_to_lds(r.v, ce.scale_v(), pc + kOffV, kTileV, v_waddr);
+            if (!own) asm volatile("" ::"v"(r.a));
         };
 #pragma unroll
         for (int j = 0; j < PF; j++) fetch(raw[j], j);
@@ -353,20 +332,12 @@ __global__ __launch_bounds__(512, 1) void scan_tph_kernel(uint32_t *__restrict__
         int buf = B0;
         auto step = [&](int v, int j, bool own) {
             if (own && v == n1 + 4) FTC_STAMP(0);
-#ifndef FTC_ABL_NOLOOK
             read_slot(slots, buf, ce);
             look_ahead(raw[(j + 1) % PF], next_buf(buf));
-#endif
             if (own && v == n1 + 4) FTC_STAMP(1);
-#ifndef FTC_ABL_NOCUT
             cut(raw[j], buf, own);
-#else
-            asm volatile("" ::"v"(raw[j].a[0]), "v"(raw[j].a[1]), "v"(raw[j].b[0]), "v"(raw[j].b[1]), "v"(raw[j].v[0]), "v"(raw[j].v[1]));
-#endif
             if (own && v == n1 + 4) FTC_STAMP(2);
-#ifndef FTC_ABL_NOFETCH
             fetch(raw[j], v + PF);
-#endif
             buf = buf == 2 ? 0 : buf + 1;
             if (own && v == n1 + 4) FTC_STAMP(3);
             wg_barrier();
@@ -479,11 +450,6 @@ __global__ __launch_bounds__(512, 1) void scan_tph_kernel(uint32_t *__restrict__
     auto rm_frag = [&](const lds_char *pc, int i) {
         const int k = i % 2, ks = (i / 2) % 2, x = i / 4;
         if (ks >= KS) return;
-#ifdef FTC_ABL_NOLDSR
-        if (x == 0) asm volatile("" : "=v"(bfr[ks][k].w[0]), "=v"(bfr[ks][k].w[1]), "=v"(bfr[ks][k].w[2]), "=v"(bfr[ks][k].w[3]));
-        else asm volatile("" : "=v"(af[x - 1][ks][k].w[0]), "=v"(af[x - 1][ks][k].w[1]), "=v"(af[x - 1][ks][k].w[2]), "=v"(af[x - 1][ks][k].w[3]));
-        return;
-#endif
         if (x == 0)
             bfr[ks][k] = lds_frag8x2(pc + k * kTileA + b_addr[ks][0], pc + k * kTileA + b_addr[ks][1]);
         else
@@ -492,13 +458,6 @@ __global__ __launch_bounds__(512, 1) void scan_tph_kernel(uint32_t *__restrict__
     // position-major fragment number i of a chunk (10: v first, then b^T tile by tile)
     auto tr_frag_into = [&](Frag (&btx)[4][2], Frag (&vfx)[2], const lds_char *pc, int i) {
         if (i >= 2 && (i - 2) / 4 >= KS) return;  // tiles 2, 3: rows 32 .. 63
-#ifdef FTC_ABL_NOLDSR
-        {
-            Frag &f = i < 2 ? vfx[i] : btx[(i - 2) / 2][(i - 2) % 2];
-            asm volatile("" : "=v"(f.w[0]), "=v"(f.w[1]), "=v"(f.w[2]), "=v"(f.w[3]));
-            return;
-        }
-#endif
         if (i < 2)
             vfx[i] = lds_frag_tr(pc + i * kTileV + vt_addr[0], pc + i * kTileV + vt_addr[1]);
         else {
@@ -508,79 +467,25 @@ __global__ __launch_bounds__(512, 1) void scan_tph_kernel(uint32_t *__restrict__
     };
     int buf = B0;  // LDS buffer of the chunk at hand
     wg_barrier();  // the slots are zero
+    wg_barrier();  // the slot of position 0 is complete
+    wg_barrier();  // barrier 0: position 0 is cut
+    read_slot(slots, B0, ce);
+    Ucur = ce.state_exp();
+    if (op.s0 && !exchange) add_caller_state();
     if (n1 > 0) {
         // ---- the first n1 positions of the walk: state update only ----
-        // Rows 16 .. 31 of b and v of these chunks are fetched and cut by the consumers (lane
-        // 64 w + lane takes the quad that producer lane of the same number would take).  The
-        // loop is skewed by one chunk: while the matrix instructions of position k - 1 run,
-        // the fragments of position k arrive in the other set of registers and position
-        // k + 1 is cut.
-        const int cid = w * 64 + lane, crow = (T + cid) / QA, cc4 = (T + cid) % QA;
-        const uint32_t b_slb = (uint32_t)op.b_sl * 4, v_slb = (uint32_t)op.v_sl * 4;
-        const char *b_seg = (const char *)op.b + ((int64_t)n * op.b_sn + (int64_t)h * op.b_sh) * 4;
-        const char *v_seg = (const char *)op.v +
-                            ((int64_t)n * op.v_sn + (int64_t)h * op.v_sh + F * fb) * 4;
-        const __amdgpu_buffer_rsrc_t b_rs = __builtin_amdgcn_make_buffer_rsrc(
-            (void *)b_seg, 0, (rows - 1) * b_slb + Dw * 4, kRsrcFlags);
-        const __amdgpu_buffer_rsrc_t v_rs = __builtin_amdgcn_make_buffer_rsrc(
-            (void *)v_seg, 0, (rows - 1) * v_slb + fw * 4, kRsrcFlags);
-        const bool b_in = 4 * cc4 < Dw;
-        const bool v_in = 4 * cc4 < fw;
-        const uint32_t b_goff = (uint32_t)crow * b_slb + 16u * cc4,
-                       v_goff = (uint32_t)crow * v_slb + 16u * cc4;
-        const int b_waddr = TpSwizzle<RBA>::addr(crow, 2 * b_tile_column(4 * cc4)),
-                  v_waddr = TpSwizzle<RBV>::addr(crow, 8 * cc4);
-        struct RawC {
-            u32x4 b, v;
-        };
-        RawC rawc[PF];
-        auto cfetch = [&](RawC &r, int v) {
-#ifdef FTC_ABL_NOMEM
-            v = n1 + 100;
-#endif
-            const int row0 = v < n1 ? chunk_row0(so_chunk(v)) : -2 * kChunk;
-            r.b = __builtin_amdgcn_raw_buffer_load_b128(
-                b_rs, b_in ? b_goff + (uint32_t)row0 * b_slb : kNoRow, 0, 0);
-            r.v = __builtin_amdgcn_raw_buffer_load_b128(
-                v_rs, v_in ? v_goff + (uint32_t)row0 * v_slb : kNoRow, 0, 0);
-        };
-        auto clook = [&](const RawC &r, int k) {
-            raise_slot(slots, k, ce, 0.f, max_abs4(r.b, 0.f), max_abs4(r.v, 0.f), lane);
-        };
-        auto ccut_b = [&](const RawC &r, int bufk) {
-            cut_quad_to_lds(r.b, ce.scale_b(), unit_pc + bufk * kBufBytes + kOffB, kTileA, b_waddr);
-        };
-        auto ccut_v = [&](const RawC &r, int bufk) {
-            cut_quad_to_lds(r.v, ce.scale_v(), unit_pc + bufk * kBufBytes + kOffV, kTileV, v_waddr);
-        };
-#pragma unroll
-        for (int j = 0; j < PF; j++) cfetch(rawc[j], j);
-        clook(rawc[0], B0);
-        wg_barrier();  // the slot of position 0 is complete
-        read_slot(slots, B0, ce);
-        ccut_b(rawc[0], B0);
-        ccut_v(rawc[0], B0);
-        clook(rawc[1], next_buf(B0));
-        cfetch(rawc[0], PF);
-        wg_barrier();  // barrier 0
-        Ucur = ce.state_exp();
-        if (op.s0 && !exchange) add_caller_state();
-        int U_frag = Ucur;  // units of the fragments about to be multiplied (position k - 1)
-        int U_load = Ucur;  // units of the fragments being loaded (position k)
+        // The loop is skewed by one position: while the matrix instructions of position k - 1
+        // run, the fragments of position k arrive in the other set of registers.
+        int U_prev = Ucur;                 // units of the fragments about to be multiplied
         Frag bt2[4][2] = {}, vf2[2] = {};  // (the first round multiplies zeros)
-        int bufn = next_buf(B0);           // LDS buffer of the position after the one at hand
         for (int c = 0; c < n1; c += PF) {
 #pragma unroll
             for (int j = 0; j < PF; j++) {
                 const lds_char *pc = unit_pc + buf * kBufBytes;
-                // position c + j + 1 is cut under the matrix instructions of position
-                // c + j - 1 (position n1 is all the producers')
-                const bool cut_next = j < PF - 1 || c + PF < n1;
-                const RawC &rn = rawc[(j + 1) % PF];
-                read_slot(slots, bufn, ce);  // the ceilings of position c + j + 1
-                if (U_frag != Ucur) {               // the ceilings rose: the state shrinks
-                    scale_state(Ucur - U_frag);
-                    Ucur = U_frag;
+                read_slot(slots, buf, ce);  // the ceilings of position c + j
+                if (U_prev != Ucur) {       // the ceilings rose: the state shrinks
+                    scale_state(Ucur - U_prev);
+                    Ucur = U_prev;
                 }
 #pragma unroll
                 for (int i = 0; i < 12; i++) {
@@ -592,16 +497,10 @@ __global__ __launch_bounds__(512, 1) void scan_tph_kernel(uint32_t *__restrict__
                         if (rows_exist) S[i % 4] = mfma16h(bt[i % 4][kPa[i / 4]], vf[kPb[i / 4]], S[i % 4]);
                         if (i < 10) tr_frag_into(bt2, vf2, pc, i);
                     }
-                    if (i == 6 && cut_next) ccut_b(rn, bufn);
-                    if (i == 9 && cut_next) ccut_v(rn, bufn);
                     __builtin_amdgcn_sched_barrier(0);
                 }
-                clook(rawc[(j + 2) % PF], next_buf(bufn));
-                cfetch(rawc[(j + 1) % PF], c + j + 1 + PF);
-                U_frag = U_load;
-                U_load = ce.state_exp();
-                buf = bufn;
-                bufn = next_buf(bufn);
+                U_prev = ce.state_exp();
+                buf = next_buf(buf);
                 wg_barrier();
 #ifdef FTC_TIMELINE
                 if (stamp_on && c + j < 30) chunk_stamps[32 + c + j] = __builtin_amdgcn_s_memrealtime();
@@ -610,9 +509,9 @@ __global__ __launch_bounds__(512, 1) void scan_tph_kernel(uint32_t *__restrict__
             }
         }
         // the last of these positions (n1 is even: its fragments are in the second set)
-        if (U_frag != Ucur) {
-            scale_state(Ucur - U_frag);
-            Ucur = U_frag;
+        if (U_prev != Ucur) {
+            scale_state(Ucur - U_prev);
+            Ucur = U_prev;
         }
 #pragma unroll
         for (int i = 0; i < 12; i++) {
@@ -620,13 +519,8 @@ __global__ __launch_bounds__(512, 1) void scan_tph_kernel(uint32_t *__restrict__
             rm_frag(unit_pc + buf * kBufBytes, i);  // our own first chunk is cut
             __builtin_amdgcn_sched_barrier(0);
         }
-        // (the slot of position n1 was read in the last round)
+        read_slot(slots, buf, ce);  // the ceilings of our own first chunk
     } else {
-        wg_barrier();  // the slot of position 0 is complete
-        wg_barrier();  // barrier 0
-        read_slot(slots, 0, ce);  // (B0 = 0)
-        Ucur = ce.state_exp();
-        if (op.s0 && !exchange) add_caller_state();
 #pragma unroll
         for (int i = 0; i < 12; i++) rm_frag(unit_pc, i);
     }
@@ -680,17 +574,15 @@ __global__ __launch_bounds__(512, 1) void scan_tph_kernel(uint32_t *__restrict__
     int s_cut = s;                            // ... and the s that went into it
     float mS = 0.f;                           // largest |S| seen while cutting
     Frag sf[2][2];
-    auto cut_s = [&](int ks, int q) {
-#ifdef FTC_ABL_NOCUTS
-        asm volatile("" : "=v"(sf[ks][0].w[q]), "=v"(sf[ks][1].w[q]) : "v"(S[2 * ks + q / 2][2 * (q % 2)]));
-        return;
-#endif
-        const float x0 = S[2 * ks + q / 2][2 * (q % 2)], x1 = S[2 * ks + q / 2][2 * (q % 2) + 1];
-        mS = fmaxf(fmaxf(fabsf(x0), fabsf(x1)), mS);
-        cut_pair_f16(x0, x1, kappa, sf[ks][0].w[q], sf[ks][1].w[q]);
+    // tile 2 ks + u of S_w -> words 2 u, 2 u + 1 of the fragments of k-step ks
+    auto cut_s = [&](int ks, int u) {
+        const f32x4 x = S[2 * ks + u];
+        mS = fmaxf(fmaxf(fmaxf(fabsf(x[0]), fabsf(x[1])), fmaxf(fabsf(x[2]), fabsf(x[3]))), mS);
+        cut_quad_f16(x[0], x[1], x[2], x[3], kappa, sf[ks][0].w[2 * u], sf[ks][0].w[2 * u + 1],
+                     sf[ks][1].w[2 * u], sf[ks][1].w[2 * u + 1]);
     };
-#pragma unroll
-    for (int q = 0; q < 4; q++) cut_s(0, q);
+    cut_s(0, 0);
+    cut_s(0, 1);
 
     // Ot_w of the chunk before in the units of that chunk (exponent Xo), and where its rows
     // go (before the first chunk: nowhere)
@@ -700,10 +592,6 @@ __global__ __launch_bounds__(512, 1) void scan_tph_kernel(uint32_t *__restrict__
     int Xo = 0;
     uint32_t o_off = 0x80000000u;
     auto store_rows = [&](int x) {
-#ifdef FTC_ABL_NOSTORE
-        asm volatile("" ::"v"(O[x]));
-        return;
-#endif
         const u32x4 r = {__float_as_uint(__builtin_amdgcn_ldexpf(O[x][0], Xo)),
                          __float_as_uint(__builtin_amdgcn_ldexpf(O[x][1], Xo)),
                          __float_as_uint(__builtin_amdgcn_ldexpf(O[x][2], Xo)),
@@ -734,7 +622,7 @@ __global__ __launch_bounds__(512, 1) void scan_tph_kernel(uint32_t *__restrict__
             if (i == 1) store_rows(1);
             if (ks < KS) P = mfma16h(bfr[ks][kPa[m]], af[0][ks][kPb[m]], P);
             O[x] = mfma16h(sf[0][kPa[mo]], af[x][0][kPb[mo]], mo == 0 ? zero : O[x]);
-            if (i < 4 && KS > 1) cut_s(1, i);
+            if ((i == 1 || i == 3) && KS > 1) cut_s(1, i / 2);
             tr_frag_into(bt, vf, pc, i);
             if (i < 4) tr_frag_into(bt, vf, pc, 6 + i);
             __builtin_amdgcn_sched_barrier(0);
@@ -760,10 +648,10 @@ __global__ __launch_bounds__(512, 1) void scan_tph_kernel(uint32_t *__restrict__
             S[i % 2] = mfma16h(bt[i % 2][kPa[m]], vf[kPb[m]], S[i % 2]);
             if (i == 1) {
                 uint32_t h0, l0, h1, l1;
-                cut_pair_f16_unscaled(__uint_as_float(__float_as_uint(P[0]) & keep[0]),
-                                      __uint_as_float(__float_as_uint(P[1]) & keep[1]), h0, l0);
-                cut_pair_f16_unscaled(__uint_as_float(__float_as_uint(P[2]) & keep[2]),
-                                      __uint_as_float(__float_as_uint(P[3]) & keep[3]), h1, l1);
+                cut_quad_f16_unscaled(__uint_as_float(__float_as_uint(P[0]) & keep[0]),
+                                      __uint_as_float(__float_as_uint(P[1]) & keep[1]),
+                                      __uint_as_float(__float_as_uint(P[2]) & keep[2]),
+                                      __uint_as_float(__float_as_uint(P[3]) & keep[3]), h0, h1, l0, l1);
                 const u32x2 wh = {h0, h1}, wl = {l0, l1};
                 *(lds_vec2 *)(ptc + pt_waddr) = wh;
                 *(lds_vec2 *)(ptc + kTileP + pt_waddr) = wl;
@@ -811,7 +699,7 @@ __global__ __launch_bounds__(512, 1) void scan_tph_kernel(uint32_t *__restrict__
         for (int i = 0; i < 6; i++) {
             const int x = i % 2, m = i / 2;
             O[x] = mfma16h(vf[kPa[m]], pf[x][kPb[m]], O[x]);
-            if (i < 4) cut_s(0, i);
+            if (i == 1 || i == 3) cut_s(0, i / 2);
             __builtin_amdgcn_sched_barrier(0);
         }
         o_off = (uint32_t)chunk_row0(c) * o_slb;
@@ -820,7 +708,6 @@ __global__ __launch_bounds__(512, 1) void scan_tph_kernel(uint32_t *__restrict__
     };
     {
         int c = c0;
-#ifndef FTC_ABL_NOCONS
         for (; c + 3 <= nchunks; c += 3) {
             chunk_body(c, std::integral_constant<int, 0>());
             chunk_body(c + 1, std::integral_constant<int, 1>());
@@ -828,13 +715,13 @@ __global__ __launch_bounds__(512, 1) void scan_tph_kernel(uint32_t *__restrict__
         }
         if (c < nchunks) chunk_body(c++, std::integral_constant<int, 0>());
         if (c < nchunks) chunk_body(c++, std::integral_constant<int, 1>());
-#else
-        for (; c < nchunks; c++) wg_barrier();
-#endif
     }
     store_rows(0);
     store_rows(1);
     FTC_STAMP(15);  // last rows on their way
+#ifdef FTC_TIMELINE
+    if (stamp_on) stamp_base[13] = __builtin_amdgcn_s_memtime();
+#endif
     if (op.s_out && seg == (int)nseg - 1) {
         float *base =
             op.s_out + (int64_t)n * op.so_sn + (int64_t)h * op.so_sh + F * fb + 16 * w + ln;

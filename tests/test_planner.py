@@ -25,17 +25,17 @@ def field(line, pattern):
 
 def test_headline_shape():
     fwd = lines((10, 8, 1000, 64), (10, 8, 1000, 64))
-    assert len(fwd) == 1 and fwd[0].startswith("scan_tp_kernel:")
+    assert len(fwd) == 1 and fwd[0].startswith("scan_tph_kernel:")
     assert "3 segments" in fwd[0] and "cuts at chunks 0,12,24,32" in fwd[0]
     assert "240 workgroups" in fwd[0] and "workspace 0 bytes" in fwd[0]
     bwd = lines((10, 8, 1000, 64), (10, 8, 1000, 64), backward=True)
-    assert len(bwd) == 1 and bwd[0].startswith("scan_tp_kernel: 3 scans")
+    assert len(bwd) == 1 and bwd[0].startswith("scan_tph_kernel: 3 scans")
     assert "1 segment " in bwd[0] and "240 workgroups" in bwd[0]
 
 
 def test_long_chains_exchange_their_segment_sums():
     fwd = lines((1, 16, 65536, 64), (1, 16, 65536, 64))
-    assert fwd[0].startswith("scan_tp_kernel (exchange):")
+    assert fwd[0].startswith("scan_tph_kernel (exchange):")
     assert "16 segments of 4096 rows" in fwd[0] and "256 workgroups" in fwd[0]
     need = int(field(fwd[0], r"workspace (\d+) bytes"))
     lib = _native.load()
@@ -45,7 +45,7 @@ def test_long_chains_exchange_their_segment_sums():
     assert bwd[0].startswith("scan_dma_kernel: 3 scans")
     # config 4's operator shape
     op = lines((10, 8, 4096, 64), (10, 8, 4096, 64))
-    assert op[0].startswith("scan_tp_kernel (exchange):") and "3 segments of 1408 rows" in op[0]
+    assert op[0].startswith("scan_tph_kernel (exchange):") and "3 segments of 1408 rows" in op[0]
 
 
 def test_what_the_chain_parallel_kernel_leaves_to_the_others():
@@ -60,7 +60,7 @@ def test_what_the_chain_parallel_kernel_leaves_to_the_others():
     assert lines((10, 8, 1000, 32), (10, 8, 1000, 32))[0].startswith("scan_dma_kernel")
     # (32 rows or columns: the chain-parallel kernel on whole chains unless both are 32,
     # the kernels that split L where it would need an exchange)
-    assert lines((10, 8, 1000, 32), (10, 8, 1000, 128))[0].startswith("scan_tp_kernel:")
+    assert lines((10, 8, 1000, 32), (10, 8, 1000, 128))[0].startswith("scan_tph_kernel:")
     assert lines((4, 16, 16384, 32), (4, 16, 16384, 128))[0].startswith("scan_dma_kernel")
     assert lines((1, 3, 500, 128), (1, 3, 500, 128))[0].startswith("scan_mfma_kernel")  # few chains
     assert lines((4, 8, 1000, 64), (4, 8, 1000, 64), dtype=_native.FTC_BF16)[0] \
@@ -71,10 +71,10 @@ def test_what_the_chain_parallel_kernel_leaves_to_the_others():
     # backward the two copies serve all three scans, and dQ and dK are copied back)
     odd = lines((8, 16, 4096, 25), (8, 16, 4096, 64))
     assert odd[0].startswith("pad_rows_kernel: 2 operands") and "0 results" in odd[0]
-    assert odd[1].startswith("scan_tp_kernel") and "state 32 x 64" in odd[1]
+    assert odd[1].startswith("scan_tph_kernel") and "state 32 x 64" in odd[1]
     odd = lines((8, 16, 4096, 25), (8, 16, 4096, 64), backward=True)
     assert odd[0].startswith("pad_rows_kernel: 2 operands") and "2 results" in odd[0]
-    assert odd[1].startswith("scan_tp_kernel: 2 scans") and "state 64 x 32" in odd[1]
+    assert odd[1].startswith("scan_tph_kernel: 2 scans") and "state 64 x 32" in odd[1]
     wide = lines((8, 16, 4096, 99), (8, 16, 4096, 101), backward=True)
     assert wide[0].startswith("pad_rows_kernel: 4 operands") and "3 results" in wide[0]
     assert wide[1].startswith("scan_tp_kernel: 3 scans") and "state 128 x 128" in wide[1]
@@ -88,7 +88,7 @@ def test_what_the_chain_parallel_kernel_leaves_to_the_others():
     # rows added to the first one's
     three = lines((1, 2, 8192, 300), (1, 2, 8192, 64))
     assert [l.split(":")[0].split(" ")[0] for l in three] == \
-        ["scan_tp_kernel", "scan_tp_kernel", "add_rows_kernel", "scan_tp_kernel", "add_rows_kernel"]
+        ["scan_tp_kernel", "scan_tp_kernel", "add_rows_kernel", "scan_tph_kernel", "add_rows_kernel"]
     assert "state 128 x 64" in three[0] and "state 128 x 64" in three[1] and "state 44 x 64" in three[3]
     two = lines((1, 2, 8192, 200), (1, 2, 8192, 64))
     assert "state 128 x 64" in two[0] and "state 72 x 64" in two[1] and two[2].startswith("add_rows_kernel: 1 result")
@@ -111,7 +111,7 @@ def test_cut_chains(chains, L):
     no longer than with equal segments (of whole groups of four chunks)."""
     N, H = chains
     line = lines((N, H, L, 64), (N, H, L, 64))[0]
-    if not line.startswith("scan_tp_kernel:"):
+    if not line.startswith("scan_tph_kernel:"):
         return
     cuts = [int(x) for x in field(line, r"cuts at chunks ([\d,]*\d)").split(",")]
     nseg = int(field(line, r"(\d+) segments? of"))
