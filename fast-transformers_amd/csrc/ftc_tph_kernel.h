@@ -18,17 +18,21 @@
 //    fp32 accumulator: half the matrix instructions, two thirds of the LDS traffic and about
 //    a third of the vector instructions of three bf16 pieces, with results as close to
 //    float64 as those (the reference's own fp32 order is further away than either).
-//  * The scales.  Rows of a, b and v are scaled chunk by chunk by powers of two that are
-//    running ceilings: 2^(4 - e) with e the smallest exponent such that every value of that
-//    operand met so far in the walk is below 2^e in magnitude.  Scaled values therefore stay
-//    below 16, values down to 2^-7 of the largest one met so far keep 22 bits, and the error
-//    of smaller ones is below 2^-29 of that largest one -- the way the reference's running
-//    fp32 state treats small contributions.  The ceilings come about without a pass of their
-//    own: while it cuts position k of the walk, every wavefront that cuts looks at the rows of
-//    position k + 1, which it already holds in registers; a wavefront that finds a value at
-//    or above the current ceiling (rare after the first chunks) raises that position's slot
-//    in LDS with an atomic maximum, and after the workgroup barrier all eight wavefronts read
-//    the slot.  All of them thus know the same three exponents for every position.
+//  * The scales.  Rows are scaled chunk by chunk by powers of two, 2^(4 - e) with 2^e a
+//    ceiling above every magnitude concerned: for b and v, whose products add up in the
+//    state, every value of that operand met so far in the walk (a ceiling that only rises);
+//    for a, the values of the chunk alone.  Scaled values therefore stay below 16, values
+//    down to 2^-7 of the ceiling keep 22 bits, and the error of smaller ones is below 2^-29 of
+//    the ceiling -- for b and v the way the reference's running fp32 state treats small
+//    contributions, for a within the 32 rows of a chunk.  The ceilings come about without a
+//    pass of their own: while they cut position k of the walk, the producers look at the rows
+//    of position k + 1, which they already hold in registers, and enter what they find in
+//    that position's slot in LDS with atomic maxima (for b and v only when a value reaches the
+//    running ceiling: rare after the first chunks; for a one word per wavefront and
+//    position); after the
+//    workgroup barrier all twelve wavefronts read the slot.  All of them thus know the same
+//    three exponents for every position, and they depend on the rows alone: however a chain
+//    is cut into segments, the results are the same bit for bit.
 //  * The state is kept in the units of the scaled rows (2^(e_b + e_v - 8)); when a ceiling
 //    rises it is rescaled (exactly).  It is cut into pieces with one more power of two,
 //    2^-s, chosen so that no element exceeds 2^15: s rises when the largest element of the
@@ -36,9 +40,6 @@
 //    chunk product needs no scale: |Pt| <= 64 * 16 * 16 = 2^14.
 //  * Ot = (S^T a^T) 2^s + v^T Pt is summed in the units of the chunk and leaves the
 //    accumulator through one v_ldexp_f32 per value.
-//
-// Results depend on where a chain is cut (the ceilings of `a` start afresh in every segment),
-// within the rounding of the pieces.
 #pragma once
 #include <type_traits>
 
@@ -113,10 +114,24 @@ __device__ __forceinline__ uint32_t ceiling_of(float m) {
     const uint32_t be = (__float_as_uint(m) >> 23) & 0xffu;  // m < 2^(be - 126)
     return max(kExpFloor, min(kExpCeil, be + 2u));
 }
+// The largest of a non-negative float over the wavefront (wave-uniform): four steps inside
+// the rows of 16 lanes on the data-parallel path, then one lane of every row.
+template <int CTRL>
+__device__ __forceinline__ float max_with_dpp(float x) {
+    return fmaxf(x, __uint_as_float((uint32_t)__builtin_amdgcn_update_dpp(
+                        0, (int)__float_as_uint(x), CTRL, 0xf, 0xf, true)));
+}
 __device__ __forceinline__ float wave_max(float m) {
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) m = fmaxf(m, __shfl_xor(m, off));
-    return m;
+    m = max_with_dpp<0xb1>(m);   // quad_perm [1, 0, 3, 2]
+    m = max_with_dpp<0x4e>(m);   // quad_perm [2, 3, 0, 1]
+    m = max_with_dpp<0x141>(m);  // row_half_mirror
+    m = max_with_dpp<0x140>(m);  // row_mirror
+    const uint32_t b = __float_as_uint(m);
+    const uint32_t r = max(max((uint32_t)__builtin_amdgcn_readlane((int)b, 0),
+                               (uint32_t)__builtin_amdgcn_readlane((int)b, 16)),
+                           max((uint32_t)__builtin_amdgcn_readlane((int)b, 32),
+                               (uint32_t)__builtin_amdgcn_readlane((int)b, 48)));
+    return __uint_as_float(r);  // (non-negative floats order like their bit patterns)
 }
 
 // The running ceilings of a, b and v as one wavefront knows them (wave-uniform).
@@ -130,25 +145,31 @@ struct Ceilings {
     __device__ __forceinline__ int out_exp() const { return (int)(Ea + Eb + Ev) - 396; }
 };
 typedef __attribute__((address_space(3))) uint32_t lds_u32_t;
-// The slot of a position is that of its LDS buffer: words (a, b, v, unused)
+// The slot of a position is that of its LDS buffer: words (a, b, v, unused).  The words of b
+// and v hold ceilings that only ever rise (a stale one is harmless: it is below the running
+// ceiling that every wavefront carries).  The word of a holds the ceiling of the rows of that
+// one position, tagged with the position's number in the upper 24 bits, so that what the
+// slot held three positions ago is always smaller and needs no clearing.
 __device__ __forceinline__ void read_slot(const lds_u32_t *slots, int k, Ceilings &c) {
     const u32x4 s = *(const lds_vec4 *)(slots + 4 * k);
-    c.Ea = max(c.Ea, (uint32_t)__builtin_amdgcn_readfirstlane(s.x));
+    c.Ea = max(kExpFloor, (uint32_t)__builtin_amdgcn_readfirstlane(s.x) & 0xffu);
     c.Eb = max(c.Eb, (uint32_t)__builtin_amdgcn_readfirstlane(s.y));
     c.Ev = max(c.Ev, (uint32_t)__builtin_amdgcn_readfirstlane(s.z));
 }
-// lane maxima of the rows of a position against the ceilings known so far: whoever finds a
-// value at or above one raises slot k, that position's
-__device__ __forceinline__ void raise_slot(lds_u32_t *slots, int k, const Ceilings &c, float ma,
-                                           float mb, float mv, int lane) {
-    const bool over = ma >= pow2_field((int)c.Ea - 1) || mb >= pow2_field((int)c.Eb - 1) ||
-                      mv >= pow2_field((int)c.Ev - 1);
+// Lane maxima of the rows of position `pos` (slot k) against the ceilings of the position
+// before it.  a: every wavefront that holds rows enters the ceiling of its own rows.  b, v:
+// whoever finds a value at or above the running ceiling raises the slot.
+__device__ __forceinline__ void raise_slot(lds_u32_t *slots, int k, int pos, const Ceilings &c,
+                                           float ma, float mb, float mv, int lane) {
+    lds_u32_t *const s = slots + 4 * k;
+    const uint32_t ea = ceiling_of(wave_max(ma));
+    if (lane == 0)
+        __hip_atomic_fetch_max(s + 0, ((uint32_t)(pos + 1) << 8) | ea, __ATOMIC_RELAXED,
+                               __HIP_MEMORY_SCOPE_WORKGROUP);
+    const bool over = mb >= pow2_field((int)c.Eb - 1) || mv >= pow2_field((int)c.Ev - 1);
     if (__builtin_amdgcn_ballot_w64(over) != 0) {
-        const uint32_t ea = ceiling_of(wave_max(ma)), eb = ceiling_of(wave_max(mb)),
-                       ev = ceiling_of(wave_max(mv));
-        lds_u32_t *const s = slots + 4 * k;
+        const uint32_t eb = ceiling_of(wave_max(mb)), ev = ceiling_of(wave_max(mv));
         if (lane == 0) {
-            if (ea > c.Ea) __hip_atomic_fetch_max(s + 0, ea, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
             if (eb > c.Eb) __hip_atomic_fetch_max(s + 1, eb, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
             if (ev > c.Ev) __hip_atomic_fetch_max(s + 2, ev, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
         }
@@ -309,8 +330,8 @@ __global__ __launch_bounds__(768, 3) void scan_tph_kernel(uint32_t *__restrict__
         };
         // the largest magnitudes of the rows of a position against the ceilings (rows that
         // were not asked for read as zeros); k: that position's slot
-        auto look_ahead = [&](const Raw &r, int k) {
-            raise_slot(slots, k, ce, max_abs4(r.a, 0.f), max_abs4(r.b, 0.f), max_abs4(r.v, 0.f), lane);
+        auto look_ahead = [&](const Raw &r, int k, int pos) {
+            raise_slot(slots, k, pos, ce, max_abs4(r.a, 0.f), max_abs4(r.b, 0.f), max_abs4(r.v, 0.f), lane);
         };
         // A position of the walk goes to its LDS buffer through register set (position % PF).
         // The first n1 positions only feed the state: no piece of a.
@@ -324,7 +345,7 @@ __global__ __launch_bounds__(768, 3) void scan_tph_kernel(uint32_t *__restrict__
 #pragma unroll
         for (int j = 0; j < PF; j++) fetch(raw[j], j);
         wg_barrier();  // the slots are zero
-        look_ahead(raw[0], B0);
+        look_ahead(raw[0], B0, 0);
         wg_barrier();  // the slot of position 0 is complete
         // Barrier number k (k = 0: before the consumers' first position; k >= 1: in the
         // middle of position k - 1) finds position k cut and the slot of position k + 1
@@ -333,7 +354,7 @@ __global__ __launch_bounds__(768, 3) void scan_tph_kernel(uint32_t *__restrict__
         auto step = [&](int v, int j, bool own) {
             if (own && v == n1 + 4) FTC_STAMP(0);
             read_slot(slots, buf, ce);
-            look_ahead(raw[(j + 1) % PF], next_buf(buf));
+            look_ahead(raw[(j + 1) % PF], next_buf(buf), v + 1);
             if (own && v == n1 + 4) FTC_STAMP(1);
             cut(raw[j], buf, own);
             if (own && v == n1 + 4) FTC_STAMP(2);
@@ -358,7 +379,7 @@ __global__ __launch_bounds__(768, 3) void scan_tph_kernel(uint32_t *__restrict__
         for (int j = 0; j < PF - 1; j++) {
             if (v + j > nwalk) return;
             read_slot(slots, buf, ce);
-            look_ahead(raw[(j + 1) % PF], next_buf(buf));
+            look_ahead(raw[(j + 1) % PF], next_buf(buf), v + j + 1);
             cut(raw[j], buf, true);
             buf = buf == 2 ? 0 : buf + 1;
             wg_barrier();
@@ -688,7 +709,7 @@ __global__ __launch_bounds__(768, 3) void scan_tph_kernel(uint32_t *__restrict__
             __builtin_amdgcn_sched_barrier(0);
         }
         // the ceilings of the next chunk
-        ce.Ea = max(ce.Ea, (uint32_t)__builtin_amdgcn_readfirstlane(slot_next.x));
+        ce.Ea = max(kExpFloor, (uint32_t)__builtin_amdgcn_readfirstlane(slot_next.x) & 0xffu);
         ce.Eb = max(ce.Eb, (uint32_t)__builtin_amdgcn_readfirstlane(slot_next.y));
         ce.Ev = max(ce.Ev, (uint32_t)__builtin_amdgcn_readfirstlane(slot_next.z));
         dU = Ucur - ce.state_exp();
