@@ -9,12 +9,16 @@ HBM.  The default workload is the configuration the metric is quoted on:
 N=10, H=8, L=1000, E=M=64, fp32.  Steps rotate over several input sets (> 512 MB in total) so
 that the 256 MB Infinity Cache cannot serve a step from the previous one.
 
-Prints ONE JSON line.  ``value`` is N*L / t(fwd+bwd) in Mtokens/s.  ``roofline`` covers the
-backward launch sequence (the dominant part of a step) against HBM: algorithmic bytes are
-4*(4E+3M) per (n,h,l) position for fp32 (read Q,K,V,G, write dQ,dK,dV), timed with events on
-the stream the kernels are launched on.  ``cpu_baseline`` times the reference's own CPU
-extension (or, when it is not built, its C restatement) on this box's host cores over a
-bounded number of calls of the same workload.
+Prints ONE JSON line.  ``value`` is N*L / t(fwd+bwd) in Mtokens/s.  ``roofline`` is the mean
+over the two launches of a step (forward: one scan, backward: three scans side by side):
+algorithmic bytes per launch = 4*((2E+2M) + (4E+3M))/2 per (n,h,l) position for fp32 (forward
+reads Q,K,V and writes the product; backward reads Q,K,V,G and writes dQ,dK,dV), algorithmic
+flops 14*E*M/2, over the mean of the two launch durations, timed with events on the stream
+the kernels are launched on; both the HBM and the matrix-core fraction are given and the one
+with the larger minimum time is named as the bound.  With the default workload the line also
+carries a few timed steps of cfg3 and cfg5 (``config.secondary``).  ``cpu_baseline`` times
+the reference's own CPU extension (or, when it is not built, its C restatement) on this box's
+host cores over a bounded number of calls of the same workload.
 """
 import argparse
 import json
@@ -84,56 +88,19 @@ def alg_bytes_per_position(E, M, dtype):
     return 2 * (2 * E + M) + 4 * M, 2 * (2 * E + M) + 4 * M + 2 * (2 * E + M)
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=None, help="timed steps (default: 1000; 50 for cfg4)")
-    ap.add_argument("--warmup", type=int, default=None,
-                    help="untimed steps first (default: 200, past the clock ramp; 5 for cfg4)")
-    ap.add_argument("--workload", default="cfg2", choices=sorted(WORKLOADS) + ["cfg4"])
-    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--sets", type=int, default=0, help="input sets to rotate over (0 = auto)")
-    ap.add_argument("--ramp-ms", type=float, default=300.0,
-                    help="set-up: untimed steps for this many milliseconds before the warm-up "
-                         "steps, so that the GPU clocks have ramped (0 to skip)")
-    ap.add_argument("--print-kernel-hash", action="store_true",
-                    help="print the kernel source hash that stamps measured traffic and exit")
-    ap.add_argument("--calibrate-copy", action="store_true",
-                    help="also run one 256 MiB device copy (a known-size kernel for scaling "
-                         "the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)")
-    args = ap.parse_args()
-    if args.steps is None:
-        args.steps = 50 if args.workload == "cfg4" else 1000
-    if args.warmup is None:
-        args.warmup = 5 if args.workload == "cfg4" else 200
-    if args.print_kernel_hash:
-        print(kernel_source_hash())
-        return
-    if args.gpus != 1:
-        print("bench.py: this build runs on ONE GPU (the path shards over N*H with no "
-              "communication; no multi-GPU figure is produced). Use --gpus 1.", file=sys.stderr)
-        sys.exit(2)
-
+def measure(workload, steps, warmup, ramp_ms, sets_arg=0, calibrate_copy=False, wrapper_leg=True):
+    """Times `steps` forward + backward steps of one workload through the C ABI and returns the
+    JSON line's dictionary (without the CPU baseline)."""
     import torch
     from fast_transformers_amd import _native
     from fast_transformers_amd.causal_product import causal_dot_product_hip, \
         causal_dot_backward_hip
-
-    if args.workload == "cfg4":
-        return encoder_workload(args)
-
-    if not torch.cuda.is_available():
-        print("bench.py: no GPU visible", file=sys.stderr)
-        sys.exit(1)
-    _native.load()
-    torch.cuda.set_device(0)
     dev = torch.device("cuda:0")
-
-    N, H, L, E, M, dtype, seed = WORKLOADS[args.workload]
+    N, H, L, E, M, dtype, seed = WORKLOADS[workload]
     tdtype = torch.float32 if dtype == "f32" else torch.bfloat16
     esz = 4 if dtype == "f32" else 2
     set_bytes = N * H * L * ((2 * E + M) * esz * 2 + 2 * M * 4)
-    nsets = args.sets or max(1, min(8, -(-(768 << 20) // set_bytes)))
+    nsets = sets_arg or max(1, min(8, -(-(768 << 20) // set_bytes)))
 
     gen = torch.Generator(device="cpu").manual_seed(seed)
     sets = []
@@ -186,7 +153,7 @@ def main():
         fwd(i)
         bwd(i)
 
-    if args.calibrate_copy:
+    if calibrate_copy:
         src = torch.empty(64 << 20, dtype=torch.float32, device=dev).normal_()
         dst = torch.empty_like(src)
         dst.copy_(src)          # reads 256 MiB, writes 256 MiB
@@ -202,24 +169,24 @@ def main():
     # set-up: a fresh GPU takes a few hundred milliseconds of load to reach its clocks
     t_ramp = time.perf_counter()
     i = 0
-    while (time.perf_counter() - t_ramp) * 1e3 < args.ramp_ms:
+    while (time.perf_counter() - t_ramp) * 1e3 < ramp_ms:
         for _ in range(20):
             step(i)
             i += 1
         torch.cuda.synchronize()
-    for i in range(args.warmup):
+    for i in range(warmup):
         step(i)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for i in range(args.steps):
+    for i in range(steps):
         step(i)
     torch.cuda.synchronize()
     t1 = time.perf_counter()
-    ms_per_step = (t1 - t0) * 1e3 / args.steps
+    ms_per_step = (t1 - t0) * 1e3 / steps
 
     # per-direction device time with events on the launch stream
-    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(args.steps)]
-    for i in range(args.steps):
+    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(steps)]
+    for i in range(steps):
         ev[i][0].record()
         fwd(i)
         ev[i][1].record()
@@ -229,13 +196,15 @@ def main():
     assert int(ws[8:12].view(torch.int32).item()) == 0, "a wavefront gave up waiting"
 
     # cost of going through the Python wrapper instead (same work, wall clock)
-    t2 = time.perf_counter()
-    for i in range(args.steps):
-        (q, k, v, g), (o, dq, dk, dv) = sets[i % nsets]
-        causal_dot_product_hip(q, k, v, o)
-        causal_dot_backward_hip(q, k, v, g, dq, dk, dv)
-    torch.cuda.synchronize()
-    wrapper_ms = (time.perf_counter() - t2) * 1e3 / args.steps
+    wrapper_ms = float("nan")
+    if wrapper_leg:
+        t2 = time.perf_counter()
+        for i in range(steps):
+            (q, k, v, g), (o, dq, dk, dv) = sets[i % nsets]
+            causal_dot_product_hip(q, k, v, o)
+            causal_dot_backward_hip(q, k, v, g, dq, dk, dv)
+        torch.cuda.synchronize()
+        wrapper_ms = (time.perf_counter() - t2) * 1e3 / steps
     fwd_ms = sorted(e[0].elapsed_time(e[1]) for e in ev)
     bwd_ms = sorted(e[1].elapsed_time(e[2]) for e in ev)
     fwd_avg, bwd_avg = sum(fwd_ms) / len(fwd_ms), sum(bwd_ms) / len(bwd_ms)
@@ -272,8 +241,8 @@ def main():
         "value": round(value, 3),
         "unit": "Mtokens/s",
         "n_gpus": 1,
-        "steps": args.steps,
-        "warmup": args.warmup,
+        "steps": steps,
+        "warmup": warmup,
         "ms_per_step": round(ms_per_step, 5),
         "higher_is_better": True,
         "scaling": "weak",
@@ -281,7 +250,7 @@ def main():
         "dtype": "f32" if dtype == "f32" else "bf16 in / f32 accumulate",
         "data": "synthetic",
         "config": {"workload": "%s: causal_dot_product fwd+bwd N=%d H=%d L=%d E=%d M=%d %s"
-                               % (args.workload, N, H, L, E, M, dtype),
+                               % (workload, N, H, L, E, M, dtype),
                    "input_sets_rotated": nsets,
                    "token_heads_per_s": round(TH / (ms_per_step * 1e-3), 1),
                    "python_wrapper_ms_per_step": round(wrapper_ms, 5),
@@ -302,10 +271,78 @@ def main():
                      "launch_ms_avg": round(launch_ms, 5),
                      "alg_bytes_per_launch": int(launch_bytes),
                      "alg_flops_per_launch": int(launch_flops),
-                     "traffic": measured_traffic(args.workload),
+                     "traffic": measured_traffic(workload),
                      "kernel_source_hash": kernel_source_hash()},
     }
 
+    return result, (N, H, L, E, M, seed)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=None, help="timed steps (default: 1000; 50 for cfg4)")
+    ap.add_argument("--warmup", type=int, default=None,
+                    help="untimed steps first (default: 200, past the clock ramp; 5 for cfg4)")
+    ap.add_argument("--workload", default="cfg2", choices=sorted(WORKLOADS) + ["cfg4"])
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-secondary", action="store_true",
+                    help="cfg2 only: skip the few timed steps of cfg3 and cfg5 that the line "
+                         "carries as config.secondary")
+    ap.add_argument("--sets", type=int, default=0, help="input sets to rotate over (0 = auto)")
+    ap.add_argument("--ramp-ms", type=float, default=300.0,
+                    help="set-up: untimed steps for this many milliseconds before the warm-up "
+                         "steps, so that the GPU clocks have ramped (0 to skip)")
+    ap.add_argument("--print-kernel-hash", action="store_true",
+                    help="print the kernel source hash that stamps measured traffic and exit")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run one 256 MiB device copy (a known-size kernel for scaling "
+                         "the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)")
+    args = ap.parse_args()
+    if args.steps is None:
+        args.steps = 50 if args.workload == "cfg4" else 1000
+    if args.warmup is None:
+        args.warmup = 5 if args.workload == "cfg4" else 200
+    if args.print_kernel_hash:
+        print(kernel_source_hash())
+        return
+    if args.gpus != 1:
+        print("bench.py: this build runs on ONE GPU (the path shards over N*H with no "
+              "communication; no multi-GPU figure is produced). Use --gpus 1.", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from fast_transformers_amd import _native
+    from fast_transformers_amd.causal_product import causal_dot_product_hip, \
+        causal_dot_backward_hip
+
+    if args.workload == "cfg4":
+        return encoder_workload(args)
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    _native.load()
+    torch.cuda.set_device(0)
+    dev = torch.device("cuda:0")
+
+    result, (N, H, L, E, M, seed) = measure(args.workload, args.steps, args.warmup, args.ramp_ms,
+                                            args.sets, args.calibrate_copy)
+    # The other two single-kernel configurations, a few steps each, in the same line: the
+    # long-sequence shape (cfg3) and the bf16 / asymmetric one (cfg5).
+    if args.workload == "cfg2" and not args.no_secondary:
+        torch.cuda.empty_cache()
+        secondary = {}
+        for name in ("cfg3", "cfg5"):
+            r, _ = measure(name, 10, 3, 0.0, wrapper_leg=False)
+            secondary[name] = {
+                "workload": r["config"]["workload"], "ms_per_step": r["ms_per_step"],
+                "Mtokens_per_s": r["value"], "fwd_ms_avg": r["config"]["fwd_ms_avg"],
+                "bwd_ms_avg": r["config"]["bwd_ms_avg"], "bound": r["roofline"]["bound"],
+                "hbm_frac": r["roofline"]["hbm"]["frac"], "mfma_frac": r["roofline"]["mfma"]["frac"],
+                "kernels": r["roofline"]["kernel"], "steps": 10, "warmup": 3}
+            torch.cuda.empty_cache()
+        result["config"]["secondary"] = secondary
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(N, H, L, E, M, seed, args.workload)
     print(json.dumps(result))

@@ -14,6 +14,7 @@
 #include <string.h>
 
 #include <algorithm>
+#include <atomic>
 #include <mutex>
 
 #include "ftc_common.h"
@@ -32,6 +33,37 @@ void note_kernel(const char *name) { g_kernel = name; }
 static thread_local bool g_plan_only = false;
 static thread_local char g_plan[2048] = "";
 bool plan_only() { return g_plan_only; }
+
+// ---- tuning aids from the environment, read once -------------------------------------------
+static Tuning g_tuning;
+static std::atomic<int> g_tuning_state{0};  // 0: not read, 1: being read, 2: ready
+static void read_tuning(Tuning &t) {
+    auto num = [](const char *name) -> int {
+        const char *env = getenv(name);
+        return env && *env ? atoi(env) : -1;
+    };
+    t.split = num("FTC_SPLIT"), t.pad = num("FTC_PAD"), t.wg = num("FTC_WG"), t.tp = num("FTC_TP");
+    t.tp_segs = num("FTC_TP_SEGS"), t.tpx = num("FTC_TPX"), t.tpx_segs = num("FTC_TPX_SEGS");
+    t.seg_chunks = num("FTC_SEG_CHUNKS"), t.group = num("FTC_GROUP"), t.dma = num("FTC_DMA");
+    t.tph = num("FTC_TPH");
+    const char *ratio = getenv("FTC_TP_RATIO");
+    t.tp_ratio = ratio && *ratio ? atof(ratio) : -1.0;
+    t.stamp_ptr = getenv("FTC_STAMP_PTR");
+}
+const Tuning &tuning() {
+    if (g_tuning_state.load(std::memory_order_acquire) != 2) {
+        int expected = 0;
+        if (g_tuning_state.compare_exchange_strong(expected, 1)) {
+            read_tuning(g_tuning);
+            g_tuning.generation = 1;
+            g_tuning_state.store(2, std::memory_order_release);
+        } else {
+            while (g_tuning_state.load(std::memory_order_acquire) != 2) {
+            }
+        }
+    }
+    return g_tuning;
+}
 void note_plan(const char *fmt, ...) {
     const size_t used = strlen(g_plan);
     if (used + 2 >= sizeof(g_plan)) return;
@@ -189,8 +221,7 @@ __global__ void zero_words_kernel(uint32_t *p, uint32_t words);
 // workspace that is then added to the first one's rows (add_rows_kernel).  fp32 rows, widths
 // multiples of 4.
 bool split_widths(int64_t D, int64_t F) {
-    if (const char *env = getenv("FTC_SPLIT"))  // tuning aid
-        if (atoi(env) == 0) return false;
+    if (tuning().split == 0) return false;  // tuning aid
     return D > 128 && D <= 512 && F >= 4 && F <= 512 && D % 4 == 0 && F % 4 == 0;
 }
 
@@ -486,8 +517,7 @@ int padded_scans(const ScanDesc *scans, int n, const bool *take, int64_t N, int6
 bool pad_eligible(const ScanDesc &sc, int64_t rows) {
     const int Dp = padded_rows(sc.a.width);
     if (Dp == 0 || rows < kPadMinRows) return false;
-    if (const char *env = getenv("FTC_PAD"))  // tuning aid
-        if (atoi(env) == 0) return false;
+    if (tuning().pad == 0) return false;  // tuning aid
     return padded_shape_ok(Dp, round_up(sc.v.width, 32));
 }
 
@@ -633,6 +663,15 @@ extern "C" {
 
 int ftc_version(void) { return 1000; }
 
+int ftc_tuning_reload(void) {
+    tuning();  // (makes sure the first read is over)
+    Tuning t;
+    read_tuning(t);
+    t.generation = g_tuning.generation + 1;
+    g_tuning = t;
+    return FTC_OK;
+}
+
 const char *ftc_last_error(void) { return g_error; }
 
 const char *ftc_last_kernel(void) { return g_kernel; }
@@ -765,9 +804,15 @@ int64_t ftc_causal_dot_backward_workspace_bytes(int64_t N, int64_t H, int64_t L,
         int64_t ws = 0;
         if (padded_rows(E)) ws = std::max(ws, scan_workspace_bytes(N, H, L, padded_rows(E), round_up(M, 32)));
         if (padded_rows(M)) ws = std::max(ws, scan_workspace_bytes(N, H, L, padded_rows(M), round_up(E, 32)));
-        need = std::max(need, std::max<int64_t>(round_up(ws, 256), FTC_WORKSPACE_CONTROL_BYTES) +
-                                  4 * round_up(N * H * L * round_up(E, 32) * 4, 256) +
-                                  3 * round_up(N * H * L * round_up(M, 32) * 4, 256));
+        int64_t copies = 4 * round_up(N * H * L * round_up(E, 32) * 4, 256) +
+                         3 * round_up(N * H * L * round_up(M, 32) * 4, 256);
+        // bf16 rows whose two state shapes lie on either side of 128 rows: the scans of the
+        // wide one run on fp32 copies, the others on bf16 ones, so the tensors that both
+        // read (queries and keys, at most the values as well) are copied once for each
+        if (bf16)
+            copies += 2 * round_up(N * H * L * round_up(E, 32) * 2, 256) +
+                      round_up(N * H * L * round_up(M, 32) * 2, 256);
+        need = std::max(need, std::max<int64_t>(round_up(ws, 256), FTC_WORKSPACE_CONTROL_BYTES) + copies);
     }
     return need;
 }

@@ -44,6 +44,17 @@ inline OperandOut as_operand_out(const ftc_tensor4 *t) {
 int fail(int code, const char *fmt, ...);
 // Records which kernel the last launch on this thread used (ftc_last_kernel()).
 void note_kernel(const char *name);
+// The FTC_* environment variables (tuning aids for measurements; none is needed in normal
+// use), read once when the library is first used and again only by ftc_tuning_reload():
+// -1 stands for "not set".
+struct Tuning {
+    int split, pad, wg, tp, tp_segs, tpx, tpx_segs, seg_chunks, group, dma, tph;
+    double tp_ratio;  // < 0: not set
+    const char *stamp_ptr;
+    uint64_t generation;  // counts the reloads: memoised plans are dropped when it changes
+};
+const Tuning &tuning();
+
 // Plan-only mode of the calling thread (ftc_causal_dot_plan): the scan functions describe the
 // launch they would make, one line each, instead of making it, and touch no GPU.
 bool plan_only();

@@ -17,7 +17,7 @@ struct MfmaPlan {
 // all-fp32 scans of these widths run as workgroups of F / 32 wavefronts (ftc_wg_kernel.h)
 bool use_wg_kernel(int64_t D, int64_t F, int nscans, int64_t L, bool all_f32) {
     if (!all_f32 || !scan_wg_covers((int)D, (int)F)) return false;
-    if (const char *env = getenv("FTC_WG")) return atoi(env) != 0;  // tuning aid
+    if (tuning().wg >= 0) return tuning().wg != 0;  // tuning aid
     // Measured: a single scan over long chains (the forward) is 2-7 % faster in workgroup
     // form (cfg3 forward 331 us against 349, N=8, H=16, L=4096: 164 against 177); launches of
     // three scans and short chains are faster with one wavefront per segment.
@@ -57,8 +57,8 @@ int tp_kernel_segments(int64_t units, int64_t L, bool wide, bool others) {
     // chunk costs about a third of a full one), as long as that fills at least half the GPU.
     const int64_t total_chunks = (L + kChunk - 1) / kChunk;
     int nseg = (int)std::max<int64_t>(1, std::min<int64_t>(std::min<int64_t>(4, 256 / units), total_chunks));
-    if (const char *env = getenv("FTC_TP_SEGS")) nseg = std::max(1, std::min(atoi(env), 16));  // tuning aid
-    if (const char *env = getenv("FTC_TP")) return atoi(env) != 0 ? nseg : 0;           // tuning aid
+    if (tuning().tp_segs >= 0) nseg = std::max(1, std::min(tuning().tp_segs, 16));  // tuning aid
+    if (tuning().tp >= 0) return tuning().tp != 0 ? nseg : 0;                       // tuning aid
     // Measured (forward, us, N=10 H=8): cfg2 (L=1000) 30 against 42 for the kernels that split
     // L and exchange states; L=3000: 75 against 84; L=4096: 100 against 108; L=8192: 201
     // against 201 -- cut chains pay off while the chunks that a workgroup walks for its
@@ -87,7 +87,7 @@ int tp_segment_starts(int64_t chunks, int nseg, int32_t *start) {
     const int groups = (int)((chunks + kTpAhead - 1) / kTpAhead);
     nseg = std::max(1, std::min(std::min(nseg, groups), kMaxTpSegments));
     double kStateOnly = 0.4;
-    if (const char *env = getenv("FTC_TP_RATIO")) kStateOnly = atof(env);  // tuning aid
+    if (tuning().tp_ratio >= 0) kStateOnly = tuning().tp_ratio;  // tuning aid
     // best[s][g]: smallest achievable longest time of segments s .. nseg-1 when segment s
     // starts at group g (dynamic programme from the last segment back)
     constexpr int kMaxGroups = 64;  // 256 chunks
@@ -122,8 +122,7 @@ int tp_segment_starts(int64_t chunks, int nseg, int32_t *start) {
 int tp_exchange_segments(int64_t units, int64_t L, bool wide, int *nseg) {
     const int64_t total_chunks = (L + kChunk - 1) / kChunk;
     *nseg = 0;
-    if (const char *env = getenv("FTC_TPX"))  // tuning aid
-        if (atoi(env) == 0) return 0;
+    if (tuning().tpx == 0) return 0;  // tuning aid
     // Up to 64 chunks the cut chains without an exchange are as fast (cfg2: 30 us either way)
     // and need no workspace.
     if (units < 1 || (units > 128 && !wide) || total_chunks <= 64) return 0;
@@ -143,7 +142,7 @@ int tp_exchange_segments(int64_t units, int64_t L, bool wide, int *nseg) {
         }
     }
     want = std::min<int64_t>(want, total_chunks / 8);
-    if (const char *env = getenv("FTC_TPX_SEGS")) want = std::max(1, atoi(env));  // tuning aid
+    if (tuning().tpx_segs >= 0) want = std::max(1, tuning().tpx_segs);  // tuning aid
     if (want < 2) return 0;
     const int64_t seg_chunks = ((total_chunks + want - 1) / want + kTpAhead - 1) / kTpAhead * kTpAhead;
     const int64_t n = (total_chunks + seg_chunks - 1) / seg_chunks;
@@ -158,8 +157,8 @@ int tp_exchange_segments(int64_t units, int64_t L, bool wide, int *nseg) {
 // The chain-parallel kernel's plan for `nscans` scans of a D x F state over chains x L rows:
 // *seg_chunks > 0: an exchange with *nseg segments of that many chunks; else *nseg > 0: chains
 // cut into *nseg segments that need no exchange; both 0: another kernel takes the launch.
-void tp_plan(int64_t D, int64_t F, int64_t chains, int nscans, int64_t L, int *nseg, int *seg_chunks,
-             bool forced = false) {
+void tp_plan_compute(int64_t D, int64_t F, int64_t chains, int nscans, int64_t L, int *nseg,
+                     int *seg_chunks, bool forced) {
     *nseg = *seg_chunks = 0;
     if (!tp_widths(D, F, forced)) return;
     const bool wide = D != 64 || F != 64 || forced;
@@ -190,8 +189,8 @@ int64_t tp_exchange_workspace_bytes(int64_t units, int nseg, int64_t D) {
 
 // `wg`: the plan is for workgroups of F / 32 wavefronts (each has its own flag words);
 // `norm`: for their fused attention form, with one more wavefront and state slab per unit
-MfmaPlan make_plan(int64_t N, int64_t H, int64_t L, int64_t D, int64_t F, int nscans, bool wg,
-                   bool norm = false) {
+MfmaPlan make_plan_compute(int64_t N, int64_t H, int64_t L, int64_t D, int64_t F, int nscans,
+                           bool wg, bool norm) {
     MfmaPlan pl;
     const int64_t flags_per_unit = wg ? F / 32 + (norm ? 1 : 0) : 1;
     const int64_t chains = std::max<int64_t>(1, N * H);
@@ -217,8 +216,8 @@ MfmaPlan make_plan(int64_t N, int64_t H, int64_t L, int64_t D, int64_t F, int ns
         }
     }
     // tuning aid: FTC_SEG_CHUNKS=<n> forces segments of n chunks
-    if (const char *env = getenv("FTC_SEG_CHUNKS")) {
-        const int64_t forced = atoll(env);
+    if (tuning().seg_chunks >= 0) {
+        const int64_t forced = tuning().seg_chunks;
         if (forced >= 1 && forced <= total_chunks) {
             const int64_t nseg = (total_chunks + forced - 1) / forced;
             if (chains * nseg * nscans * flags_per_unit <= kMaxWaves && nseg <= 4096) best_c = forced;
@@ -235,6 +234,55 @@ MfmaPlan make_plan(int64_t N, int64_t H, int64_t L, int64_t D, int64_t F, int ns
     pl.workspace_bytes += nscans * pl.waves * 128;  // time stamps (ftc_wg_kernel.h)
 #endif
     return pl;
+}
+
+// Plans depend on the sizes alone and a caller repeats the same sizes call after call (the
+// segment search walks up to 4096 candidates for a long sequence): the last plans of every
+// thread are kept, keyed by their arguments and by the generation of the tuning variables.
+template <typename Value>
+struct PlanMemo {
+    static constexpr int kEntries = 32;
+    struct Entry {
+        int64_t key[8];
+        uint64_t generation;
+        Value value;
+    };
+    Entry entry[kEntries] = {};
+    template <typename Compute>
+    Value get(const int64_t (&key)[8], Compute compute) {
+        uint64_t h = 1469598103934665603ull;
+        for (int64_t k : key) h = (h ^ (uint64_t)k) * 1099511628211ull;
+        Entry &e = entry[h % kEntries];
+        const uint64_t generation = tuning().generation;
+        bool hit = e.generation == generation;
+        for (int i = 0; i < 8 && hit; i++) hit = e.key[i] == key[i];
+        if (!hit) {
+            e.value = compute();
+            for (int i = 0; i < 8; i++) e.key[i] = key[i];
+            e.generation = generation;
+        }
+        return e.value;
+    }
+};
+struct TpPlan {
+    int nseg, seg_chunks;
+};
+void tp_plan(int64_t D, int64_t F, int64_t chains, int nscans, int64_t L, int *nseg, int *seg_chunks,
+             bool forced = false) {
+    static thread_local PlanMemo<TpPlan> memo;
+    const int64_t key[8] = {D, F, chains, nscans, L, forced ? 1 : 0, 0, 0};
+    const TpPlan pl = memo.get(key, [&]() {
+        TpPlan p;
+        tp_plan_compute(D, F, chains, nscans, L, &p.nseg, &p.seg_chunks, forced);
+        return p;
+    });
+    *nseg = pl.nseg, *seg_chunks = pl.seg_chunks;
+}
+MfmaPlan make_plan(int64_t N, int64_t H, int64_t L, int64_t D, int64_t F, int nscans, bool wg,
+                   bool norm = false) {
+    static thread_local PlanMemo<MfmaPlan> memo;
+    const int64_t key[8] = {N, H, L, D, F, nscans, wg ? 1 : 0, norm ? 1 : 0};
+    return memo.get(key, [&]() { return make_plan_compute(N, H, L, D, F, nscans, wg, norm); });
 }
 
 // every row must start on a 16-byte boundary (16-byte loads and stores)
@@ -442,7 +490,7 @@ int mfma_scan(const ScanDesc *scans, int nscans, int64_t N, int64_t H, int64_t L
     args.key_len = fused ? fused->key_lengths : nullptr;
 #ifdef FTC_TIMELINE
     if (tp)  // tuning aid: where the chain-parallel kernel writes its time stamps
-        if (const char *env = getenv("FTC_STAMP_PTR"))
+        if (const char *env = getenv("FTC_STAMP_PTR"))  // (a build for measurements only)
             args.key_len = (const int64_t *)(uintptr_t)strtoull(env, nullptr, 0);
 #endif
     args.H = (int32_t)H;
@@ -462,7 +510,7 @@ int mfma_scan(const ScanDesc *scans, int nscans, int64_t N, int64_t H, int64_t L
         while (args.group * args.group < pl.nseg) args.group++;
     }
     // tuning aid: FTC_GROUP=<n> forces groups of n steps
-    if (const char *env = getenv("FTC_GROUP")) args.group = std::max(1, atoi(env));
+    if (tuning().group >= 0) args.group = std::max(1, tuning().group);
     // a wavefront watches one flag per lane: at most 64 steps per group and 64 groups
     args.group = std::min(args.group, 64);
     while ((pl.nseg + args.group - 1) / args.group > 64) args.group++;
@@ -472,11 +520,11 @@ int mfma_scan(const ScanDesc *scans, int nscans, int64_t N, int64_t H, int64_t L
             return fail(FTC_ERR_INVALID, "scans of one launch must share widths and dtypes");
     // fp32 states of up to 64 rows: the kernel that feeds its fragments from LDS tiles
     bool dma = D <= 64 && combo == kFFFF;
-    if (const char *env = getenv("FTC_DMA")) dma = dma && atoi(env) != 0;  // tuning aid
+    if (tuning().dma >= 0) dma = dma && tuning().dma != 0;  // tuning aid
     // chain-parallel scans of states of up to 64 rows run on the fp16 matrix path
     // (ftc_tph_kernel.h: two scaled fp16 pieces per value), wider ones on three bf16 pieces
     bool half_pieces = tp && D <= 64;
-    if (const char *env = getenv("FTC_TPH")) half_pieces = half_pieces && atoi(env) != 0;  // tuning aid
+    if (tuning().tph >= 0) half_pieces = half_pieces && tuning().tph != 0;  // tuning aid
     note_kernel(tp ? (half_pieces ? (tpx_seg_chunks > 0 ? "scan_tph_kernel (exchange)" : "scan_tph_kernel")
                                   : (tpx_seg_chunks > 0 ? "scan_tp_kernel (exchange)" : "scan_tp_kernel"))
                 : wg ? (fused ? "scan_wg_kernel<NORM>" : "scan_wg_kernel")

@@ -133,12 +133,12 @@ __device__ __forceinline__ void split_pair_under_mfma(float x0, float x1, uint32
     }
 }
 
-// elu(x) + 1 = max(x, 0) + exp(min(x, 0)): five instructions, no select.  For x > 0 the
-// second term is exactly one.  For x <= 0 the exponent x log2(e) is rounded once, which costs
-// at most |x| 2^-24 ln 2 of relative accuracy -- in absolute terms never more than
+// elu(x) + 1 = x + 1 for x > 0, exp(x) otherwise (NaN stays NaN, as in the reference's
+// elu(x) + 1).  For x <= 0 the exponent x log2(e) is rounded once, which costs at most
+// |x| 2^-24 ln 2 of relative accuracy -- in absolute terms never more than
 // 2^-24 ln 2 max_x |x| e^x = 1.6e-8, a fraction of the rounding of a feature near one.
 __device__ __forceinline__ float feature_phi(float x) {
-    return fmaxf(x, 0.f) + __builtin_amdgcn_exp2f(fminf(x, 0.f) * 1.44269502f);
+    return x > 0.f ? x + 1.f : __builtin_amdgcn_exp2f(x * 1.44269502f);
 }
 // the feature map on four values of a row
 __device__ __forceinline__ u32x4 feature_quad(const u32x4 raw) {

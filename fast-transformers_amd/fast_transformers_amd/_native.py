@@ -22,6 +22,7 @@ EXPORTED_SYMBOLS = (
     "ftc_version",
     "ftc_last_error",
     "ftc_last_kernel",
+    "ftc_tuning_reload",
     "ftc_causal_dot_plan",
     "ftc_workspace_reset",
     "ftc_causal_dot_product_workspace_bytes",
@@ -65,6 +66,8 @@ def load():
     lib.ftc_last_error.argtypes = []
     lib.ftc_last_kernel.restype = ctypes.c_char_p
     lib.ftc_last_kernel.argtypes = []
+    lib.ftc_tuning_reload.restype = ctypes.c_int
+    lib.ftc_tuning_reload.argtypes = []
     for name in ("ftc_causal_dot_product_workspace_bytes",
                  "ftc_causal_dot_backward_workspace_bytes",
                  "ftc_causal_linear_attention_workspace_bytes"):

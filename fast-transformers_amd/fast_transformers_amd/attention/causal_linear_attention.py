@@ -159,7 +159,7 @@ class CausalLinearAttention(Module):
         if queries.shape[1] != keys.shape[1] or keys.shape[1] != values.shape[1]:
             return None
         qv, kv, vv = (t.permute(0, 2, 1, 3) for t in (queries, keys, values))
-        if not fused_attention_covers(qv, vv):
+        if not fused_attention_covers(qv, vv, kv):
             return None
         lengths = getattr(key_lengths, "lengths", None)
         if lengths is None:  # not a length mask: the composition multiplies by its matrix

@@ -16,6 +16,7 @@
   dtype) and the gradients have the dtype of their inputs (``__init__.py:59-61``).
 """
 import os
+import time
 
 import torch
 
@@ -53,11 +54,33 @@ def _check_out(t, name):
 # buffer is allocated zero-filled once and then handed to every later call on that stream.
 #
 # The error word of a workspace (byte 8 of the control block) is non-zero after a call that
-# was cut short.  Reading it means waiting for the GPU, so the wrapper does it where that is
-# cheap or asked for: before a cached workspace is replaced by a larger one, and after every
-# call when FTC_CHECK=1 is set in the environment (a debugging mode); ``check_workspaces()``
-# does it on demand.
+# was cut short.  Reading it means waiting for the GPU, so the wrapper does that only where it
+# is asked for (``check_workspaces()``; after every call when FTC_CHECK=1 is set in the
+# environment) or cheap (before a cached workspace is replaced by a larger one).  Between
+# those it watches without waiting: at most every ``_PROBE_INTERVAL_S`` seconds a call leaves
+# an asynchronous copy of the error word to pinned host memory behind it on its stream, and a
+# later call that finds the copy finished (an event query) reads the word and raises.
 _workspaces = {}
+_ws_bytes = {}            # (query, N, H, L, E, M, dtype code) -> bytes: sizes repeat call after call
+_probes = {}              # workspace key -> [pinned word, event or None, time of the last probe]
+_PROBE_INTERVAL_S = 0.01
+
+
+def _workspace_bytes(query, N, H, L, E, M, code):
+    key = (query, N, H, L, E, M, code)
+    nbytes = _ws_bytes.get(key)
+    if nbytes is None:
+        nbytes = _native.check(getattr(_native.load(), query)(N, H, L, E, M, code), query)
+        _ws_bytes[key] = nbytes
+    return nbytes
+
+
+def reload_tuning():
+    """Make the library read its FTC_* environment variables again (they are read once, at first
+    use) and forget the workspace sizes asked for under the old values.  A debugging aid: call
+    it with no work in flight."""
+    _native.check(_native.load().ftc_tuning_reload(), "ftc_tuning_reload")
+    _ws_bytes.clear()
 
 
 def _workspace(nbytes, device):
@@ -71,12 +94,39 @@ def _workspace(nbytes, device):
             check_workspaces()  # the old buffer's last word on the calls made with it
         ws = torch.zeros(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
         _workspaces[key] = ws
+        _probes.pop(key, None)
+    _watch(key, ws)
     return ws, ws.numel()
 
 
-def _after_call():
+def _watch(key, ws):
+    """Look at a finished probe of this workspace, if there is one; otherwise nothing."""
+    probe = _probes.get(key)
+    if probe is None or probe[1] is None or torch.cuda.is_current_stream_capturing():
+        return
+    if probe[1].query():
+        probe[1] = None
+        if int(probe[0].item()) != 0:
+            check_workspaces()   # synchronises, resets the control block and raises
+
+
+def _after_call(ws=None):
     if os.environ.get("FTC_CHECK", "0") not in ("", "0"):
         check_workspaces()
+        return
+    if ws is None or torch.cuda.is_current_stream_capturing():
+        return
+    # leave a probe behind this call when the last one is old enough and has been read
+    key = (ws.device.index, torch.cuda.current_stream(ws.device).cuda_stream)
+    now = time.monotonic()
+    probe = _probes.get(key)
+    if probe is None:
+        probe = _probes[key] = [torch.zeros(1, dtype=torch.int32).pin_memory(), None, 0.0]
+    if probe[1] is None and now - probe[2] >= _PROBE_INTERVAL_S:
+        probe[0].copy_(ws[8:12].view(torch.int32), non_blocking=True)
+        ev = torch.cuda.Event()
+        ev.record()
+        probe[1], probe[2] = ev, now
 
 
 def workspace_error_words():
@@ -87,9 +137,11 @@ def workspace_error_words():
 
 def check_workspaces():
     """Synchronise and raise if any cached workspace reports that a call was cut short.  The
-    control block of such a workspace is cleared first (``ftc_workspace_reset``), so calls
-    made after the exception start from a clean workspace again: a control block left
-    non-zero would make every later call on it stop early with its outputs unwritten."""
+    control block of such a workspace is cleared first (``ftc_workspace_reset``, on the current
+    stream of its device once that device is idle: the stream the workspace was cached for may
+    be gone by now), so calls made after the exception start from a clean workspace again: a
+    control block left non-zero would make every later call on it stop early with its outputs
+    unwritten."""
     bad = {key: word for key, word in workspace_error_words().items() if word != 0}
     if not bad:
         return
@@ -97,9 +149,12 @@ def check_workspaces():
     for (device_index, stream) in bad:
         ws = _workspaces[(device_index, stream)]
         with torch.cuda.device(device_index):
-            _native.check(lib.ftc_workspace_reset(ws.data_ptr(), ws.numel(), stream),
+            torch.cuda.synchronize()
+            _native.check(lib.ftc_workspace_reset(ws.data_ptr(), ws.numel(),
+                                                  torch.cuda.current_stream().cuda_stream),
                           "ftc_workspace_reset")
-    torch.cuda.synchronize()
+            torch.cuda.synchronize()
+        _probes.pop((device_index, stream), None)
     raise RuntimeError("causal_dot_product: a call was cut short on workspace(s) %s "
                        "(error words %s); its outputs are not valid.  The workspaces have "
                        "been reset." % (sorted(bad), [bad[k] for k in sorted(bad)]))
@@ -115,15 +170,14 @@ def causal_dot_product_hip(queries, keys, values, product):
     N, H, L, E = q.shape
     M = v.shape[3]
     with torch.cuda.device(q.device):
-        nbytes = _native.check(
-            lib.ftc_causal_dot_product_workspace_bytes(N, H, L, E, M, _native.dtype_code(q.dtype)),
-            "ftc_causal_dot_product_workspace_bytes")
+        nbytes = _workspace_bytes("ftc_causal_dot_product_workspace_bytes", N, H, L, E, M,
+                                  _native.dtype_code(q.dtype))
         ws, nbytes = _workspace(nbytes, q.device)
         dq, dk, dv, do = (_native.describe(t) for t in (q, k, v, out))
         rc = lib.ftc_causal_dot_product(dq, dk, dv, do, ws.data_ptr() if ws is not None else None,
                                         nbytes, torch.cuda.current_stream().cuda_stream)
-    _native.check(rc, "ftc_causal_dot_product")
-    _after_call()
+        _native.check(rc, "ftc_causal_dot_product")
+        _after_call(ws)
 
 
 def causal_dot_product_with_state(queries, keys, values, initial_state=None,
@@ -151,9 +205,8 @@ def causal_dot_product_with_state(queries, keys, values, initial_state=None,
     out = torch.empty((N, H, L, M), dtype=torch.float32, device=q.device)
     s1 = torch.empty((N, H, E, M), dtype=torch.float32, device=q.device) if return_state else None
     with torch.cuda.device(q.device):
-        nbytes = _native.check(
-            lib.ftc_causal_dot_product_workspace_bytes(N, H, L, E, M, _native.dtype_code(q.dtype)),
-            "ftc_causal_dot_product_workspace_bytes")
+        nbytes = _workspace_bytes("ftc_causal_dot_product_workspace_bytes", N, H, L, E, M,
+                                  _native.dtype_code(q.dtype))
         ws, nbytes = _workspace(nbytes, q.device)
         dq, dk, dv, do = (_native.describe(t) for t in (q, k, v, out))
         d0 = _native.describe(s0) if s0 is not None else None
@@ -161,8 +214,8 @@ def causal_dot_product_with_state(queries, keys, values, initial_state=None,
         rc = lib.ftc_causal_dot_product_state(dq, dk, dv, d0, do, d1,
                                               ws.data_ptr() if ws is not None else None, nbytes,
                                               torch.cuda.current_stream().cuda_stream)
-    _native.check(rc, "ftc_causal_dot_product_state")
-    _after_call()
+        _native.check(rc, "ftc_causal_dot_product_state")
+        _after_call(ws)
     return out, s1
 
 
@@ -183,27 +236,28 @@ def causal_dot_backward_hip(queries, keys, values, grad_out, grad_queries, grad_
     N, H, L, E = q.shape
     M = v.shape[3]
     with torch.cuda.device(q.device):
-        nbytes = _native.check(
-            lib.ftc_causal_dot_backward_workspace_bytes(N, H, L, E, M,
-                                                        _native.dtype_code(q.dtype)),
-            "ftc_causal_dot_backward_workspace_bytes")
+        nbytes = _workspace_bytes("ftc_causal_dot_backward_workspace_bytes", N, H, L, E, M,
+                                  _native.dtype_code(q.dtype))
         ws, nbytes = _workspace(nbytes, q.device)
         descs = [_native.describe(t) if t is not None else None for t in (q, k, v, g, gq, gk, gv)]
         rc = lib.ftc_causal_dot_backward(*descs, ws.data_ptr() if ws is not None else None,
                                          nbytes, torch.cuda.current_stream().cuda_stream)
-    _native.check(rc, "ftc_causal_dot_backward")
-    _after_call()
+        _native.check(rc, "ftc_causal_dot_backward")
+        _after_call(ws)
 
 
 FTC_ERR_UNSUPPORTED = -2
 
 
-def fused_attention_covers(queries, values):
+def fused_attention_covers(queries, values, keys=None):
     """True when ``ftc_causal_linear_attention`` has a kernel for tensors of these sizes and
-    element type ((N, H, L, E) queries, (N, H, L, M) values)."""
-    if queries.dtype != torch.float32 or values.dtype != torch.float32:
+    element type ((N, H, L, E) queries and keys, (N, H, L, M) values)."""
+    tensors = (queries, values) if keys is None else (queries, keys, values)
+    if any(t.dtype != torch.float32 or t.device != queries.device for t in tensors):
         return False
     if queries.device.type != "cuda":
+        return False
+    if keys is not None and keys.shape[3] != queries.shape[3]:
         return False
     return queries.shape[3] in (32, 64) and values.shape[3] in (32, 64)
 

@@ -81,6 +81,15 @@ const char *ftc_last_error(void);
 const char *ftc_last_kernel(void);
 
 /*
+ * The library reads its FTC_* environment variables (tuning aids for measurements: they force
+ * a kernel or a segment length; none is needed in normal use) once, when it is first used.
+ * This call reads them again.  Call it with no work in flight, and repeat the workspace
+ * queries afterwards: another route may need another workspace.  No counterpart in the
+ * reference.
+ */
+int ftc_tuning_reload(void);
+
+/*
  * What ftc_causal_dot_product (backward == 0) or ftc_causal_dot_backward (backward != 0,
  * all three gradients, dense outputs) would launch for tensors of these shapes, element
  * types and strides: one line of text per launch (kernel, state size, chains, segments, cuts,

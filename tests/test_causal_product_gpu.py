@@ -733,6 +733,17 @@ def test_dirty_control_block_is_reported_and_healed(cp):
         assert scale_error(out, want) <= 1e-4
     finally:
         del os.environ["FTC_CHECK"]
+    # without the debugging mode the wrapper watches the error word without waiting for the
+    # GPU: a probe left behind one call is read by a later one (within a few calls and 10 ms)
+    ws.view(torch.int32)[64 + max_waves] = 1000
+    torch.cuda.synchronize()
+    import time
+    with pytest.raises(RuntimeError, match="cut short"):
+        for _ in range(6):
+            hip_forward(cp, Q, K, V)
+            time.sleep(0.02)
+    out = hip_forward(cp, Q, K, V)             # reset by the check: works again
+    assert scale_error(out, want) <= 1e-4
     # and a workspace is checked before a larger one replaces it
     ws.view(torch.int32)[64 + max_waves] = 1000
     torch.cuda.synchronize()
@@ -938,6 +949,7 @@ def test_chain_parallel_kernel_cut_chains_equal_whole_chains(cp, widths):
     outs = []
     for segs in ("1", "2", "4"):
         os.environ["FTC_TP"], os.environ["FTC_TP_SEGS"] = "1", segs
+        cp.reload_tuning()      # (the library reads its tuning variables once)
         try:
             out = torch.empty(N, H, L, M, device="cuda")
             cp.causal_dot_product_hip(Q, K, V, out)
@@ -947,6 +959,7 @@ def test_chain_parallel_kernel_cut_chains_equal_whole_chains(cp, widths):
             outs.append([out] + grads)
         finally:
             del os.environ["FTC_TP"], os.environ["FTC_TP_SEGS"]
+            cp.reload_tuning()
     for other in outs[1:]:
         for a, b in zip(outs[0], other):
             assert torch.equal(a, b)

@@ -196,3 +196,27 @@ def test_module_takes_the_fused_path_without_grad_and_agrees_with_the_compositio
         cla.causal_linear_attention_hip = native
     assert scale_error(y_fused.permute(0, 2, 1, 3), y_composed.detach().permute(0, 2, 1, 3)) <= 1e-5
     gate(y_fused.cpu(), q.cpu(), k.cpu(), v.cpu(), torch.tensor([700, 301]), module.eps)
+
+
+def test_non_finite_inputs_propagate_as_in_the_composition(lib):
+    """The feature map elu(x) + 1 keeps NaN (and maps -inf to 0, +inf to +inf), in the fused
+    launch as in the composition of operator calls that training uses: the same rows come out
+    non-finite either way."""
+    from fast_transformers_amd import attention, masking
+    N, L, H, E, M = 1, 300, 2, 64, 64
+    q, k, v = (t.cuda() for t in inputs(N, L, H, E, M, seed=12))
+    q[0, 40, 0, 3] = float("nan")     # one query row of head 0
+    k[0, 200, 1, 5] = float("nan")    # a key of head 1: every row from 200 on
+    q[0, 10, 1, 7] = float("-inf")    # phi(-inf) = 0: harmless
+    full = masking.LengthMask(torch.full((N,), L).cuda(), max_len=L)
+    mask = masking.TriangularCausalMask(L, device="cuda")
+    module = attention.CausalLinearAttention(E).cuda()
+    with torch.no_grad():
+        y_fused = module(q, k, v, mask, full, full)
+    y_composed = module(q.clone().requires_grad_(True), k, v, mask, full, full).detach()
+    bad_fused, bad_composed = ~torch.isfinite(y_fused), ~torch.isfinite(y_composed)
+    assert torch.equal(bad_fused.any(dim=-1), bad_composed.any(dim=-1))
+    assert bad_fused[0, 40, 0].all() and bad_fused[0, 200:, 1].all()
+    assert not bad_fused[0, :40, 0].any() and not bad_fused[0, :200, 1].any()
+    ok = ~bad_fused
+    assert (y_fused[ok] - y_composed[ok]).abs().max() <= 1e-4 * y_composed[ok].abs().max()

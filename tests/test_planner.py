@@ -179,3 +179,27 @@ def test_the_workspace_query_covers_every_launch(backward):
             for line in lines((N, H, L, E), (N, H, L, M), dtype=dtype, backward=backward):
                 need = int(field(line, r"workspace (\d+) bytes")) if "workspace" in line else 0
                 assert need <= granted, (N, H, L, E, M, dtype, line, granted)
+
+
+@pytest.mark.parametrize("dtype", [_native.FTC_F32, _native.FTC_BF16], ids=["f32", "bf16"])
+def test_workspace_queries_cover_every_plan(dtype):
+    """Whatever route the planner takes, no launch of the plan needs more workspace than the
+    query of its entry point answers: widths on either side of every limit of the planner (32,
+    64, 128 rows; multiples of 4 and of 32 and neither), also bf16 rows whose two state shapes
+    call for copies of different element types."""
+    lib = _native.load()
+    widths = [10, 25, 32, 33, 48, 64, 65, 96, 100, 128, 129, 132, 200, 255, 256, 300]
+    worst = 0.0
+    for (N, H, L) in [(10, 8, 2048), (2, 3, 700), (1, 2, 8192), (40, 16, 64)]:
+        for E in widths:
+            for M in widths:
+                for backward in (False, True):
+                    text = lines((N, H, L, E), (N, H, L, M), backward=backward, dtype=dtype)
+                    need = max([int(x) for l in text for x in re.findall(r"workspace (\d+) bytes", l)]
+                               or [0])
+                    query = (lib.ftc_causal_dot_backward_workspace_bytes if backward else
+                             lib.ftc_causal_dot_product_workspace_bytes)(N, H, L, E, M, dtype)
+                    assert need <= query, ((N, H, L, E, M), backward, need, query, text)
+                    if query:
+                        worst = max(worst, need / query)
+    assert worst > 0.5   # (the queries are not wildly generous either)

@@ -73,11 +73,23 @@ def test_static_scratch_entry_point_matches_workspace_entry_point():
 
 
 def test_static_scratch_refuses_sizes_beyond_the_array():
+    import os
     from fast_transformers_amd import _native as native
     lib = native.load()
     N, H, L, E, M = 4, 4, 65536, 500, 500  # odd widths: segment states of 1 MB each
     need = lib.ftc_causal_dot_product_workspace_bytes(N, H, L, E, M, native.FTC_F32)
     assert need > (48 << 20)
+    # ... and so does the route without padded copies, which the entry point falls back to
+    # before it gives up (asked of the host alone, with the copies switched off): only then is
+    # it safe to hand the entry point descriptors whose pointers must never be read
+    os.environ["FTC_PAD"] = "0"
+    try:
+        assert lib.ftc_tuning_reload() == 0
+        bare = lib.ftc_causal_dot_product_workspace_bytes(N, H, L, E, M, native.FTC_F32)
+    finally:
+        del os.environ["FTC_PAD"]
+        assert lib.ftc_tuning_reload() == 0
+    assert bare > (48 << 20), "the sizes of this test no longer exceed the built-in array"
     # refused on the host before anything touches the device: the pointers are never read
     def fake(X):
         return native.Tensor4(256, native.FTC_F32, (N, H, L, X), (H * L * X, L * X, X, 1))
