@@ -138,10 +138,6 @@ def dtype_code(dtype):
 
 def describe(t):
     """``ftc_tensor4`` view of a 4-d device tensor (no copy)."""
-    d = Tensor4()
-    d.ptr = t.data_ptr() if t.numel() else None
-    d.dtype = dtype_code(t.dtype)
-    for i in range(4):
-        d.size[i] = t.shape[i]
-        d.stride[i] = t.stride(i)
-    return d
+    shape = t.shape
+    empty = shape[0] == 0 or shape[1] == 0 or shape[2] == 0 or shape[3] == 0
+    return Tensor4(None if empty else t.data_ptr(), dtype_code(t.dtype), tuple(shape), t.stride())

@@ -66,6 +66,25 @@ _probes = {}              # workspace key -> [pinned word, event or None, time o
 _PROBE_INTERVAL_S = 0.01
 
 
+class _NoGuard:
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        return False
+
+
+_NO_GUARD = _NoGuard()
+
+
+def _device_guard(device):
+    """Make `device` current for the call -- at no cost when it already is."""
+    index = device.index
+    if index is None or index == torch.cuda.current_device():
+        return _NO_GUARD
+    return torch.cuda.device(index)
+
+
 def _workspace_bytes(query, N, H, L, E, M, code):
     key = (query, N, H, L, E, M, code)
     nbytes = _ws_bytes.get(key)
@@ -83,11 +102,12 @@ def reload_tuning():
     _ws_bytes.clear()
 
 
-def _workspace(nbytes, device):
+def _workspace(nbytes, device, stream=None):
     if nbytes <= 0:
         return None, 0
-    key = (device.index if device.index is not None else torch.cuda.current_device(),
-           torch.cuda.current_stream(device).cuda_stream)
+    if stream is None:
+        stream = torch.cuda.current_stream(device).cuda_stream
+    key = (device.index if device.index is not None else torch.cuda.current_device(), stream)
     ws = _workspaces.get(key)
     if ws is None or ws.numel() < nbytes:
         if ws is not None:
@@ -102,31 +122,36 @@ def _workspace(nbytes, device):
 def _watch(key, ws):
     """Look at a finished probe of this workspace, if there is one; otherwise nothing."""
     probe = _probes.get(key)
-    if probe is None or probe[1] is None or torch.cuda.is_current_stream_capturing():
+    if probe is None or probe[1] is None:
         return
-    if probe[1].query():
+    if not torch.cuda.is_current_stream_capturing() and probe[1].query():
         probe[1] = None
         if int(probe[0].item()) != 0:
             check_workspaces()   # synchronises, resets the control block and raises
 
 
-def _after_call(ws=None):
+def _after_call(ws=None, stream=None):
     if os.environ.get("FTC_CHECK", "0") not in ("", "0"):
         check_workspaces()
         return
-    if ws is None or torch.cuda.is_current_stream_capturing():
+    if ws is None:
         return
     # leave a probe behind this call when the last one is old enough and has been read
-    key = (ws.device.index, torch.cuda.current_stream(ws.device).cuda_stream)
     now = time.monotonic()
+    if stream is None:
+        stream = torch.cuda.current_stream(ws.device).cuda_stream
+    key = (ws.device.index, stream)
     probe = _probes.get(key)
+    if probe is not None and (probe[1] is not None or now - probe[2] < _PROBE_INTERVAL_S):
+        return
+    if torch.cuda.is_current_stream_capturing():
+        return
     if probe is None:
         probe = _probes[key] = [torch.zeros(1, dtype=torch.int32).pin_memory(), None, 0.0]
-    if probe[1] is None and now - probe[2] >= _PROBE_INTERVAL_S:
-        probe[0].copy_(ws[8:12].view(torch.int32), non_blocking=True)
-        ev = torch.cuda.Event()
-        ev.record()
-        probe[1], probe[2] = ev, now
+    probe[0].copy_(ws[8:12].view(torch.int32), non_blocking=True)
+    ev = torch.cuda.Event()
+    ev.record()
+    probe[1], probe[2] = ev, now
 
 
 def workspace_error_words():
@@ -169,15 +194,16 @@ def causal_dot_product_hip(queries, keys, values, product):
     out = _check_out(product, "product")
     N, H, L, E = q.shape
     M = v.shape[3]
-    with torch.cuda.device(q.device):
+    with _device_guard(q.device):
+        stream = torch.cuda.current_stream().cuda_stream
         nbytes = _workspace_bytes("ftc_causal_dot_product_workspace_bytes", N, H, L, E, M,
                                   _native.dtype_code(q.dtype))
-        ws, nbytes = _workspace(nbytes, q.device)
+        ws, nbytes = _workspace(nbytes, q.device, stream)
         dq, dk, dv, do = (_native.describe(t) for t in (q, k, v, out))
         rc = lib.ftc_causal_dot_product(dq, dk, dv, do, ws.data_ptr() if ws is not None else None,
-                                        nbytes, torch.cuda.current_stream().cuda_stream)
+                                        nbytes, stream)
         _native.check(rc, "ftc_causal_dot_product")
-        _after_call(ws)
+        _after_call(ws, stream)
 
 
 def causal_dot_product_with_state(queries, keys, values, initial_state=None,
@@ -204,18 +230,19 @@ def causal_dot_product_with_state(queries, keys, values, initial_state=None,
                                "tensor of shape (N, H, E, M)")
     out = torch.empty((N, H, L, M), dtype=torch.float32, device=q.device)
     s1 = torch.empty((N, H, E, M), dtype=torch.float32, device=q.device) if return_state else None
-    with torch.cuda.device(q.device):
+    with _device_guard(q.device):
+        stream = torch.cuda.current_stream().cuda_stream
         nbytes = _workspace_bytes("ftc_causal_dot_product_workspace_bytes", N, H, L, E, M,
                                   _native.dtype_code(q.dtype))
-        ws, nbytes = _workspace(nbytes, q.device)
+        ws, nbytes = _workspace(nbytes, q.device, stream)
         dq, dk, dv, do = (_native.describe(t) for t in (q, k, v, out))
         d0 = _native.describe(s0) if s0 is not None else None
         d1 = _native.describe(s1) if s1 is not None else None
         rc = lib.ftc_causal_dot_product_state(dq, dk, dv, d0, do, d1,
                                               ws.data_ptr() if ws is not None else None, nbytes,
-                                              torch.cuda.current_stream().cuda_stream)
+                                              stream)
         _native.check(rc, "ftc_causal_dot_product_state")
-        _after_call(ws)
+        _after_call(ws, stream)
     return out, s1
 
 
@@ -235,15 +262,16 @@ def causal_dot_backward_hip(queries, keys, values, grad_out, grad_queries, grad_
                    (grad_values, "grad_values")))
     N, H, L, E = q.shape
     M = v.shape[3]
-    with torch.cuda.device(q.device):
+    with _device_guard(q.device):
+        stream = torch.cuda.current_stream().cuda_stream
         nbytes = _workspace_bytes("ftc_causal_dot_backward_workspace_bytes", N, H, L, E, M,
                                   _native.dtype_code(q.dtype))
-        ws, nbytes = _workspace(nbytes, q.device)
+        ws, nbytes = _workspace(nbytes, q.device, stream)
         descs = [_native.describe(t) if t is not None else None for t in (q, k, v, g, gq, gk, gv)]
         rc = lib.ftc_causal_dot_backward(*descs, ws.data_ptr() if ws is not None else None,
-                                         nbytes, torch.cuda.current_stream().cuda_stream)
+                                         nbytes, stream)
         _native.check(rc, "ftc_causal_dot_backward")
-        _after_call(ws)
+        _after_call(ws, stream)
 
 
 FTC_ERR_UNSUPPORTED = -2
