@@ -912,10 +912,19 @@ int64_t ftc_causal_linear_attention_workspace_bytes(int64_t N, int64_t H, int64_
     return fused_attention_workspace_bytes(N, H, L, E, M);
 }
 
-int ftc_causal_linear_attention(const ftc_tensor4 *queries, const ftc_tensor4 *keys,
-                                const ftc_tensor4 *values, const int64_t *key_lengths, float eps,
-                                const ftc_tensor4 *out, void *workspace, size_t workspace_bytes,
-                                void *stream) {
+static int check_denominators(const ftc_tensor4 *den, const Dims &d) {
+    if (den->dtype != FTC_F32) return fail(FTC_ERR_INVALID, "denominators must be float32");
+    if (den->size[0] != d.N || den->size[1] != d.H || den->size[2] != d.L || den->size[3] != 1)
+        return fail(FTC_ERR_INVALID, "denominators must have shape (N, H, L, 1)");
+    if (d.N * d.H * d.L > 0 && !den->ptr) return fail(FTC_ERR_INVALID, "denominators has a null data pointer");
+    return FTC_OK;
+}
+
+int ftc_causal_linear_attention_forward(const ftc_tensor4 *queries, const ftc_tensor4 *keys,
+                                        const ftc_tensor4 *values, const int64_t *key_lengths,
+                                        float eps, const ftc_tensor4 *out,
+                                        const ftc_tensor4 *denominators, void *workspace,
+                                        size_t workspace_bytes, void *stream) {
     Dims d;
     int rc = read_dims(queries, values, &d);
     if (rc) return rc;
@@ -923,6 +932,7 @@ int ftc_causal_linear_attention(const ftc_tensor4 *queries, const ftc_tensor4 *k
     if ((rc = check_tensor(keys, "keys", d.N, d.H, d.L, d.E, FTC_F32, FTC_F32))) return rc;
     if ((rc = check_tensor(values, "values", d.N, d.H, d.L, d.M, FTC_F32, FTC_F32))) return rc;
     if ((rc = check_tensor(out, "out", d.N, d.H, d.L, d.M, FTC_F32, FTC_F32))) return rc;
+    if (denominators && (rc = check_denominators(denominators, d))) return rc;
     if (!(eps == eps)) return fail(FTC_ERR_INVALID, "eps is not a number");
     if (!(d.E == 32 || d.E == 64) || !(d.M == 32 || d.M == 64))
         return fail(FTC_ERR_UNSUPPORTED,
@@ -933,9 +943,119 @@ int ftc_causal_linear_attention(const ftc_tensor4 *queries, const ftc_tensor4 *k
     if (!fused_attention_supported(fwd, d.L))
         return fail(FTC_ERR_UNSUPPORTED,
                     "the fused attention kernel needs 16-byte aligned rows that do not overlap");
-    const FusedAttention fused = {key_lengths, eps};
+    FusedAttention fused;
+    fused.key_lengths = key_lengths, fused.eps = eps;
+    if (denominators) {
+        if (denominators->stride[2] != 1)
+            return fail(FTC_ERR_INVALID, "denominators must be contiguous along L");
+        fused.denominators = (float *)denominators->ptr;
+        fused.den_sn = denominators->stride[0], fused.den_sh = denominators->stride[1];
+    }
     return mfma_scan(&fwd, 1, d.N, d.H, d.L, workspace, workspace_bytes, (hipStream_t)stream,
                      &fused);
+}
+
+int ftc_causal_linear_attention(const ftc_tensor4 *queries, const ftc_tensor4 *keys,
+                                const ftc_tensor4 *values, const int64_t *key_lengths, float eps,
+                                const ftc_tensor4 *out, void *workspace, size_t workspace_bytes,
+                                void *stream) {
+    return ftc_causal_linear_attention_forward(queries, keys, values, key_lengths, eps, out, nullptr,
+                                               workspace, workspace_bytes, stream);
+}
+
+// workspace of the backward: [scans][Qf][Kf][gz][dd][segment sums]
+static int64_t attention_backward_layout(int64_t N, int64_t H, int64_t L, int64_t E, int64_t M,
+                                         int64_t (&offset)[6]) {
+    const int64_t positions = N * H * L;
+    int64_t at = std::max<int64_t>(
+        round_up(std::max(scan_workspace_bytes(N, H, L, E, M, false), scan_workspace_bytes(N, H, L, M, E, false)), 256),
+        FTC_WORKSPACE_CONTROL_BYTES);
+    offset[0] = 0;
+    offset[1] = at, at += round_up(positions * E * 4, 256);   // Qf
+    offset[2] = at, at += round_up(positions * E * 4, 256);   // Kf
+    offset[3] = at, at += round_up(positions * M * 4, 256);   // gz
+    offset[4] = at, at += round_up(positions * 4, 256);       // dd
+    offset[5] = at, at += round_up(N * H * attention_backward_segments(L) * 2 * E * 4, 256);
+    return at;
+}
+
+int64_t ftc_causal_linear_attention_backward_workspace_bytes(int64_t N, int64_t H, int64_t L,
+                                                             int64_t E, int64_t M, int32_t dtype) {
+    if (N < 0 || H < 0 || L < 0 || E < 0 || M < 0) return fail(FTC_ERR_INVALID, "negative size");
+    if (dtype != FTC_F32 || !(E == 32 || E == 64) || !(M == 32 || M == 64))
+        return fail(FTC_ERR_UNSUPPORTED,
+                    "the fused attention backward takes fp32 rows with E, M in {32, 64}");
+    if (N * H * L == 0) return 0;
+    int64_t offset[6];
+    return attention_backward_layout(N, H, L, E, M, offset);
+}
+
+int ftc_causal_linear_attention_backward(const ftc_tensor4 *queries, const ftc_tensor4 *keys,
+                                         const ftc_tensor4 *values, const int64_t *key_lengths,
+                                         const ftc_tensor4 *out, const ftc_tensor4 *denominators,
+                                         const ftc_tensor4 *grad_out, const ftc_tensor4 *grad_queries,
+                                         const ftc_tensor4 *grad_keys, const ftc_tensor4 *grad_values,
+                                         void *workspace, size_t workspace_bytes, void *stream) {
+    Dims d;
+    int rc = read_dims(queries, values, &d);
+    if (rc) return rc;
+    if ((rc = check_tensor(queries, "queries", d.N, d.H, d.L, d.E, FTC_F32, FTC_F32))) return rc;
+    if ((rc = check_tensor(keys, "keys", d.N, d.H, d.L, d.E, FTC_F32, FTC_F32))) return rc;
+    if ((rc = check_tensor(values, "values", d.N, d.H, d.L, d.M, FTC_F32, FTC_F32))) return rc;
+    if ((rc = check_tensor(out, "out", d.N, d.H, d.L, d.M, FTC_F32, FTC_F32))) return rc;
+    if ((rc = check_tensor(grad_out, "grad_out", d.N, d.H, d.L, d.M, FTC_F32, FTC_F32))) return rc;
+    if (!denominators) return fail(FTC_ERR_INVALID, "denominators is null");
+    if ((rc = check_denominators(denominators, d))) return rc;
+    if (grad_queries && (rc = check_tensor(grad_queries, "grad_queries", d.N, d.H, d.L, d.E, FTC_F32, FTC_F32)))
+        return rc;
+    if (grad_keys && (rc = check_tensor(grad_keys, "grad_keys", d.N, d.H, d.L, d.E, FTC_F32, FTC_F32)))
+        return rc;
+    if (grad_values && (rc = check_tensor(grad_values, "grad_values", d.N, d.H, d.L, d.M, FTC_F32, FTC_F32)))
+        return rc;
+    if (!(d.E == 32 || d.E == 64) || !(d.M == 32 || d.M == 64))
+        return fail(FTC_ERR_UNSUPPORTED,
+                    "the fused attention backward takes fp32 rows with E, M in {32, 64}");
+    if (d.N * d.H * d.L == 0) return FTC_OK;
+    for (const ftc_tensor4 *t : {queries, keys, values, out, grad_out, grad_queries, grad_keys})
+        if (t && ((uintptr_t)t->ptr % 16 || t->stride[0] % 4 || t->stride[1] % 4 || t->stride[2] % 4))
+            return fail(FTC_ERR_UNSUPPORTED, "the fused attention backward needs 16-byte aligned rows");
+    int64_t offset[6];
+    const int64_t need = attention_backward_layout(d.N, d.H, d.L, d.E, d.M, offset);
+    if (!workspace || (int64_t)workspace_bytes < need || (uintptr_t)workspace % 256 != 0)
+        return fail(FTC_ERR_WORKSPACE, "workspace of %lld bytes (256-byte aligned) needed, %zu given",
+                    (long long)need, workspace_bytes);
+    hipStream_t s = (hipStream_t)stream;
+    char *base = (char *)workspace;
+    float *Qf = (float *)(base + offset[1]), *Kf = (float *)(base + offset[2]);
+    float *gz = (float *)(base + offset[3]), *dd = (float *)(base + offset[4]);
+    float *sums = (float *)(base + offset[5]);
+    Operand den{denominators->ptr, denominators->stride[0], denominators->stride[1],
+                denominators->stride[2], FTC_F32, 1};
+    launch_attention_backward_prep(as_operand(queries), as_operand(keys), as_operand(grad_out),
+                                   as_operand(out), den, key_lengths, d.N, d.H, d.L, (int)d.E, (int)d.M,
+                                   Qf, Kf, gz, dd, sums, s);
+    // the plain backward's three scans on (Qf, Kf, v, gz)
+    auto dense = [&](float *p, int64_t w) {
+        return Operand{p, d.H * d.L * w, d.L * w, w, FTC_F32, (int32_t)w};
+    };
+    const Operand qf = dense(Qf, d.E), kf = dense(Kf, d.E), gzo = dense(gz, d.M), v = as_operand(values);
+    ScanDesc scans[3];
+    int n = 0;
+    if (grad_queries) scans[n++] = ScanDesc{gzo, v, kf, as_operand_out(grad_queries), false};
+    if (grad_keys) scans[n++] = ScanDesc{v, gzo, qf, as_operand_out(grad_keys), true};
+    if (grad_values) scans[n++] = ScanDesc{kf, qf, gzo, as_operand_out(grad_values), true};
+    if (n > 0 && (rc = run_scans(scans, n, d.N, d.H, d.L, workspace, (size_t)offset[1], s))) return rc;
+    if (grad_queries || grad_keys) {
+        const OperandOut none{nullptr, 0, 0, 0, FTC_F32, (int32_t)d.E};
+        launch_attention_backward_finish(as_operand(queries), as_operand(keys), key_lengths, dd, sums,
+                                         d.N, d.H, d.L, (int)d.E,
+                                         grad_queries ? as_operand_out(grad_queries) : none,
+                                         grad_keys ? as_operand_out(grad_keys) : none, s);
+    }
+    hipError_t err = hipGetLastError();
+    if (err != hipSuccess) return fail(FTC_ERR_HIP, "attention backward launch failed: %s", hipGetErrorString(err));
+    note_kernel("attention backward: prep, three scans, prefix sums");
+    return FTC_OK;
 }
 
 }  // extern "C"

@@ -146,6 +146,10 @@ int64_t mfma_tp_workspace_bytes(int64_t N, int64_t H, int64_t L, int64_t D, int6
 struct FusedAttention {
     const int64_t *key_lengths;  // N values on the device, or nullptr (every key counts)
     float eps;
+    // optional: where the denominators (phi(a_l) . sum_{j <= l} phi(b_j) + eps) go, one float
+    // per position at denominators[n den_sn + h den_sh + l] (the backward needs them)
+    float *denominators = nullptr;
+    int64_t den_sn = 0, den_sh = 0;
 };
 bool fused_attention_supported(const ScanDesc &scan, int64_t L);
 int64_t fused_attention_workspace_bytes(int64_t N, int64_t H, int64_t L, int64_t D, int64_t F);
@@ -156,6 +160,22 @@ int mfma_scan(const ScanDesc *scans, int nscans, int64_t N, int64_t H, int64_t L
               void *workspace, size_t workspace_bytes, hipStream_t stream,
               const FusedAttention *fused = nullptr, bool may_chain_parallel = true,
               bool forced = false);
+
+// Backward of the fused attention (ftc_attention.hip): the kernels around the three scans.
+// prep: Qf = phi(q), Kf = phi(k) [l < key_len] (dense rows of E floats), gz = g / den (dense rows
+// of M floats), dd = -(g . out) / den (one float per position), and per (chain, segment of
+// positions) the totals of Kf and of dd Qf (`sums`: 2 E floats each).  finish: dq and dk, which
+// hold the scans' results, get the prefix sums that the denominator contributes and phi'.
+int64_t attention_backward_segments(int64_t L);
+void launch_attention_backward_prep(const Operand &q, const Operand &k, const Operand &g,
+                                    const Operand &out, const Operand &den, const int64_t *key_len,
+                                    int64_t N, int64_t H, int64_t L, int E, int M, float *Qf,
+                                    float *Kf, float *gz, float *dd, float *sums,
+                                    hipStream_t stream);
+void launch_attention_backward_finish(const Operand &q, const Operand &k, const int64_t *key_len,
+                                      const float *dd, const float *sums, int64_t N, int64_t H,
+                                      int64_t L, int E, const OperandOut &dq, const OperandOut &dk,
+                                      hipStream_t stream);
 
 // Fill every row of `out` with zeros (used for empty contractions).
 int zero_rows(const OperandOut &out, int64_t N, int64_t H, int64_t L, hipStream_t stream);

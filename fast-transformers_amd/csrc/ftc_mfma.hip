@@ -479,6 +479,8 @@ int mfma_scan(const ScanDesc *scans, int nscans, int64_t N, int64_t H, int64_t L
         o.s0_sn = sd.initial.stride_n, o.s0_sh = sd.initial.stride_h, o.s0_sd = sd.initial.stride_d;
         o.s_out = sd.final_.ptr;
         o.so_sn = sd.final_.stride_n, o.so_sh = sd.final_.stride_h, o.so_sd = sd.final_.stride_d;
+        if (fused && fused->denominators)  // (the fused form has no state to hand out)
+            o.s_out = fused->denominators, o.so_sn = fused->den_sn, o.so_sh = fused->den_sh, o.so_sd = 0;
         max_stride = std::max(max_stride, std::max(std::max(sd.a.stride_l, sd.b.stride_l),
                                                    std::max(sd.v.stride_l, sd.out.stride_l)));
     }

@@ -685,7 +685,14 @@ __global__ __launch_bounds__(512, 2) void scan_wg_kernel(uint32_t *__restrict__ 
             // lane (i = ln, g) holds f = 32 w + 8 q + 4 g + 0..3 in registers 4 q .. 4 q + 3
             if constexpr (NORM) {
                 if (is_den) {
-                    if (g == 0) den_sh[slot][c & 1][ln] = O[0] + p.eps;
+                    if (g == 0) {
+                        const float den = O[0] + p.eps;
+                        den_sh[slot][c & 1][ln] = den;
+                        // (the caller's copy of the denominators, for the backward)
+                        const int row = chunk_row0(c) + ln;
+                        if (op.s_out && row < rows)
+                            op.s_out[(int64_t)n * op.so_sn + (int64_t)h * op.so_sh + lo + row] = den;
+                    }
                 } else {
                     O_held = O;
                 }

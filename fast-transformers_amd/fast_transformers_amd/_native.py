@@ -33,6 +33,9 @@ EXPORTED_SYMBOLS = (
     "ftc_causal_dot_backward",
     "ftc_causal_linear_attention_workspace_bytes",
     "ftc_causal_linear_attention",
+    "ftc_causal_linear_attention_forward",
+    "ftc_causal_linear_attention_backward_workspace_bytes",
+    "ftc_causal_linear_attention_backward",
 )
 
 
@@ -70,7 +73,8 @@ def load():
     lib.ftc_tuning_reload.argtypes = []
     for name in ("ftc_causal_dot_product_workspace_bytes",
                  "ftc_causal_dot_backward_workspace_bytes",
-                 "ftc_causal_linear_attention_workspace_bytes"):
+                 "ftc_causal_linear_attention_workspace_bytes",
+                 "ftc_causal_linear_attention_backward_workspace_bytes"):
         f = getattr(lib, name)
         f.restype = ctypes.c_int64
         f.argtypes = [ctypes.c_int64] * 5 + [ctypes.c_int32]
@@ -91,6 +95,13 @@ def load():
     lib.ftc_causal_linear_attention.argtypes = [t4] * 3 + [ctypes.c_void_p, ctypes.c_float, t4,
                                                            ctypes.c_void_p, ctypes.c_size_t,
                                                            ctypes.c_void_p]
+    lib.ftc_causal_linear_attention_forward.restype = ctypes.c_int
+    lib.ftc_causal_linear_attention_forward.argtypes = [t4] * 3 + [ctypes.c_void_p, ctypes.c_float, t4,
+                                                                   t4, ctypes.c_void_p,
+                                                                   ctypes.c_size_t, ctypes.c_void_p]
+    lib.ftc_causal_linear_attention_backward.restype = ctypes.c_int
+    lib.ftc_causal_linear_attention_backward.argtypes = [t4] * 3 + [ctypes.c_void_p] + [t4] * 6 + [
+        ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]
     lib.ftc_causal_dot_plan.restype = ctypes.c_int
     lib.ftc_causal_dot_plan.argtypes = [t4] * 3 + [ctypes.c_int, ctypes.c_char_p, ctypes.c_size_t]
     _lib = lib

@@ -17,14 +17,16 @@ this stack cost ten and fifty times the operator itself).
 When nothing has to be differentiated (eval, ``torch.no_grad``) and the feature map is the
 default one, the whole body of ``forward`` -- both feature maps, the key-length mask, the
 product, the normaliser and the final scale -- is one launch of
-``ftc_causal_linear_attention`` (head dimensions 32 or 64, float32).  Training keeps the
-composition above, whose pieces autograd differentiates.
+``ftc_causal_linear_attention`` (head dimensions 32 or 64, float32), and training on
+``CausalLinearAttentionFunction``, whose backward is one launch sequence of its own
+(``ftc_causal_linear_attention_backward``).  Other sizes and feature maps keep the composition
+above, whose pieces autograd differentiates.
 """
 import torch
 from torch.nn import Module
 
 from ..causal_product import causal_dot_product_hip, causal_dot_backward_hip, \
-    causal_linear_attention_hip, fused_attention_covers
+    causal_linear_attention_hip, fused_attention_covers, CausalLinearAttentionFunction
 
 
 class ActivationFunctionFeatureMap(Module):
@@ -147,11 +149,9 @@ class CausalLinearAttention(Module):
 
     def _fused_forward(self, queries, keys, values, key_lengths):
         """The whole forward in one launch (feature map, key-length mask, product,
-        normaliser), when nothing has to be differentiated and a fused kernel covers the
-        sizes; None otherwise."""
-        if torch.is_grad_enabled() and (queries.requires_grad or keys.requires_grad
-                                        or values.requires_grad):
-            return None
+        normaliser) when a fused kernel covers the sizes -- with its own backward (one
+        element-wise pass, the three gradient scans, one prefix-sum pass) when something has
+        to be differentiated; None otherwise."""
         fm = self.feature_map
         if not (isinstance(fm, ActivationFunctionFeatureMap)
                 and fm.activation_function is _elu_plus_one):
@@ -165,6 +165,9 @@ class CausalLinearAttention(Module):
         if lengths is None:  # not a length mask: the composition multiplies by its matrix
             return None
         lengths = lengths.to(device=queries.device, dtype=torch.int64).contiguous()
+        if torch.is_grad_enabled() and (queries.requires_grad or keys.requires_grad
+                                        or values.requires_grad):
+            return CausalLinearAttentionFunction.apply(qv, kv, vv, lengths, self.eps).permute(0, 2, 1, 3)
         N, L, H, _ = queries.shape
         out = torch.empty((N, L, H, values.shape[3]), device=queries.device, dtype=torch.float32)
         causal_linear_attention_hip(qv, kv, vv, lengths, self.eps, out.permute(0, 2, 1, 3))

@@ -290,37 +290,103 @@ def fused_attention_covers(queries, values, keys=None):
     return queries.shape[3] in (32, 64) and values.shape[3] in (32, 64)
 
 
-def causal_linear_attention_hip(queries, keys, values, key_lengths, eps, out):
+def _check_key_lengths(key_lengths, q):
+    if key_lengths is not None:
+        if key_lengths.dtype != torch.int64 or key_lengths.device != q.device or \
+                key_lengths.shape != (q.shape[0],) or not key_lengths.is_contiguous():
+            raise RuntimeError("causal_linear_attention: key_lengths must be a contiguous int64 "
+                               "tensor of N values on the device of the queries")
+
+
+def causal_linear_attention_hip(queries, keys, values, key_lengths, eps, out, denominators=None):
     """In-place fused forward of causally masked linear attention with the feature map
     ``elu(x) + 1``: replaces the body of the reference module's forward
     (``attention/causal_linear_attention.py:71-104``) in one launch.  ``queries``, ``keys``:
     raw (N, H, L, E) projections; ``values``, ``out``: (N, H, L, M); ``key_lengths``: int64
-    tensor of N lengths on the same device, or None.  Raises ``RuntimeError`` for sizes
-    without a fused kernel (see ``fused_attention_covers``)."""
+    tensor of N lengths on the same device, or None; ``denominators``: None, or a float32
+    (N, H, L) tensor that receives the normaliser's denominators (the backward needs them).
+    Raises ``RuntimeError`` for sizes without a fused kernel (see ``fused_attention_covers``)."""
     lib = _native.load()
     q, k, v = (_prepare(t, n) for t, n in
                ((queries, "queries"), (keys, "keys"), (values, "values")))
     o = _check_out(out, "out")
     N, H, L, E = q.shape
     M = v.shape[3]
-    if key_lengths is not None:
-        if key_lengths.dtype != torch.int64 or key_lengths.device != q.device or \
-                key_lengths.shape != (N,) or not key_lengths.is_contiguous():
-            raise RuntimeError("causal_linear_attention: key_lengths must be a contiguous int64 "
-                               "tensor of N values on the device of the queries")
-    with torch.cuda.device(q.device):
-        nbytes = _native.check(
-            lib.ftc_causal_linear_attention_workspace_bytes(N, H, L, E, M,
-                                                            _native.dtype_code(q.dtype)),
-            "ftc_causal_linear_attention_workspace_bytes")
-        ws, nbytes = _workspace(nbytes, q.device)
+    _check_key_lengths(key_lengths, q)
+    with _device_guard(q.device):
+        stream = torch.cuda.current_stream().cuda_stream
+        nbytes = _workspace_bytes("ftc_causal_linear_attention_workspace_bytes", N, H, L, E, M,
+                                  _native.dtype_code(q.dtype))
+        ws, nbytes = _workspace(nbytes, q.device, stream)
         dq, dk, dv, do = (_native.describe(t) for t in (q, k, v, o))
-        rc = lib.ftc_causal_linear_attention(
+        dden = _native.describe(denominators.unsqueeze(3)) if denominators is not None else None
+        rc = lib.ftc_causal_linear_attention_forward(
             dq, dk, dv, key_lengths.data_ptr() if key_lengths is not None else None, float(eps),
-            do, ws.data_ptr() if ws is not None else None, nbytes,
-            torch.cuda.current_stream().cuda_stream)
-    _native.check(rc, "ftc_causal_linear_attention")
-    _after_call()
+            do, dden, ws.data_ptr() if ws is not None else None, nbytes, stream)
+        _native.check(rc, "ftc_causal_linear_attention_forward")
+        _after_call(ws, stream)
+
+
+def causal_linear_attention_backward_hip(queries, keys, values, key_lengths, out, denominators,
+                                         grad_out, grad_queries, grad_keys, grad_values):
+    """In-place backward of ``causal_linear_attention_hip``: gradients with respect to the raw
+    queries, keys and values (any of the three may be None) from ``grad_out``, the forward's
+    ``out`` and its ``denominators``.  Replaces what autograd does in the reference for the body
+    of ``CausalLinearAttention.forward`` (``attention/causal_linear_attention.py:71-104``)."""
+    lib = _native.load()
+    q, k, v, o, g = (_prepare(t, n) for t, n in
+                     ((queries, "queries"), (keys, "keys"), (values, "values"), (out, "out"),
+                      (grad_out, "grad_out")))
+    gq, gk, gv = (_check_out(t, n) if t is not None else None for t, n in
+                  ((grad_queries, "grad_queries"), (grad_keys, "grad_keys"),
+                   (grad_values, "grad_values")))
+    N, H, L, E = q.shape
+    M = v.shape[3]
+    _check_key_lengths(key_lengths, q)
+    with _device_guard(q.device):
+        stream = torch.cuda.current_stream().cuda_stream
+        nbytes = _workspace_bytes("ftc_causal_linear_attention_backward_workspace_bytes", N, H, L,
+                                  E, M, _native.dtype_code(q.dtype))
+        ws, nbytes = _workspace(nbytes, q.device, stream)
+        descs = [_native.describe(t) if t is not None else None
+                 for t in (q, k, v, o, denominators.unsqueeze(3), g, gq, gk, gv)]
+        rc = lib.ftc_causal_linear_attention_backward(
+            descs[0], descs[1], descs[2],
+            key_lengths.data_ptr() if key_lengths is not None else None, *descs[3:],
+            ws.data_ptr() if ws is not None else None, nbytes, stream)
+        _native.check(rc, "ftc_causal_linear_attention_backward")
+        _after_call(ws, stream)
+
+
+class CausalLinearAttentionFunction(torch.autograd.Function):
+    """``out = causal linear attention(queries, keys, values)`` with the feature map
+    ``elu(x) + 1``, the key-length mask and the normaliser inside, one fused launch forward
+    and one launch sequence backward.  Tensors in the operator's (N, H, L, X) layout (permuted
+    views of the module's (N, L, H, X) tensors are fine)."""
+
+    @staticmethod
+    def forward(ctx, queries, keys, values, key_lengths, eps):
+        N, H, L, _ = queries.shape
+        M = values.shape[3]
+        # (N, L, H, M) storage, as the module hands its result on
+        out = torch.empty((N, L, H, M), device=queries.device, dtype=torch.float32).permute(0, 2, 1, 3)
+        den = torch.empty((N, H, L), device=queries.device, dtype=torch.float32)
+        causal_linear_attention_hip(queries, keys, values, key_lengths, eps, out, den)
+        ctx.save_for_backward(queries, keys, values, out, den)
+        ctx.key_lengths = key_lengths
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        queries, keys, values, out, den = ctx.saved_tensors
+        need = ctx.needs_input_grad
+        like = lambda t: torch.empty_like(t.permute(0, 2, 1, 3)).permute(0, 2, 1, 3)
+        gq = like(queries) if need[0] else None
+        gk = like(keys) if need[1] else None
+        gv = like(values) if need[2] else None
+        causal_linear_attention_backward_hip(queries, keys, values, ctx.key_lengths, out, den,
+                                             grad_out, gq, gk, gv)
+        return gq, gk, gv, None, None
 
 
 def _cpu_args(name, *tensors):

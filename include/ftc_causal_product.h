@@ -213,6 +213,52 @@ int ftc_causal_linear_attention(const ftc_tensor4 *queries, const ftc_tensor4 *k
                                 const ftc_tensor4 *out, void *workspace, size_t workspace_bytes,
                                 void *stream);
 
+/*
+ * The same forward, for training: it also writes, when `denominators` is not NULL, the
+ * denominators of the formula above (eps included), one float per position, which the
+ * backward below needs: (N,H,L,1), FTC_F32, unit stride along L.  Workspace:
+ * ftc_causal_linear_attention_workspace_bytes.  The reference keeps the corresponding tensor
+ * (Z, attention/causal_linear_attention.py:95) alive through autograd.
+ */
+int ftc_causal_linear_attention_forward(const ftc_tensor4 *queries, const ftc_tensor4 *keys,
+                                        const ftc_tensor4 *values, const int64_t *key_lengths,
+                                        float eps, const ftc_tensor4 *out,
+                                        const ftc_tensor4 *denominators, void *workspace,
+                                        size_t workspace_bytes, void *stream);
+
+/*
+ * Scratch bytes ftc_causal_linear_attention_backward needs (>= 0), FTC_ERR_UNSUPPORTED when the
+ * sizes are not covered, or another negative ftc_status.
+ */
+int64_t ftc_causal_linear_attention_backward_workspace_bytes(int64_t N, int64_t H, int64_t L,
+                                                             int64_t E, int64_t M, int32_t dtype);
+
+/*
+ * Gradients of ftc_causal_linear_attention_forward with respect to the raw queries, keys and
+ * values, given grad_out = d loss / d out.  Replaces what autograd does in the reference for
+ * CausalLinearAttention.forward (attention/causal_linear_attention.py:71-104): the backward
+ * of the two feature-map passes, of the key-length mask, of cumsum and einsum for the
+ * normaliser, of the final scale, and causal_dot_backward twice.  With Qf, Kf as above,
+ * gz_l = grad_out_l / den_l and dd_l = -(grad_out_l . out_l) / den_l:
+ *
+ *   dQf_l = sum_{j<=l} (gz_l . v_j) Kf_j + dd_l sum_{j<=l} Kf_j
+ *   dKf_j = sum_{l>=j} (v_j . gz_l) Qf_l + sum_{l>=j} dd_l Qf_l
+ *   grad_values_j = sum_{l>=j} (Kf_j . Qf_l) gz_l
+ *   grad_queries = dQf phi'(queries);  grad_keys_j = dKf_j phi'(keys_j) if j < key_lengths[n] else 0
+ *   phi'(x) = x > 0 ? 1 : exp(x)
+ *
+ * out, denominators: what the forward wrote.  All tensors FTC_F32 with 16-byte aligned rows;
+ * a gradient that is not wanted may be passed as NULL.  Sizes: E, M in {32, 64}.  The launch
+ * sequence: one element-wise pass (feature maps, gz, dd into the workspace), the three scans
+ * of ftc_causal_dot_backward on them, and a prefix-sum pass over grad_queries and grad_keys.
+ */
+int ftc_causal_linear_attention_backward(const ftc_tensor4 *queries, const ftc_tensor4 *keys,
+                                         const ftc_tensor4 *values, const int64_t *key_lengths,
+                                         const ftc_tensor4 *out, const ftc_tensor4 *denominators,
+                                         const ftc_tensor4 *grad_out, const ftc_tensor4 *grad_queries,
+                                         const ftc_tensor4 *grad_keys, const ftc_tensor4 *grad_values,
+                                         void *workspace, size_t workspace_bytes, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -173,7 +173,41 @@ def test_sizes_without_a_fused_kernel_are_refused(lib):
     assert rc == -2 and "fused" in _native.last_error()
 
 
-def test_module_takes_the_fused_path_without_grad_and_agrees_with_the_composition(lib):
+def _count_backward_calls():
+    """Context that counts the calls of the fused backward (autograd runs it on a thread of its
+    own, where ftc_last_kernel() of this thread does not see it)."""
+    import contextlib
+    from fast_transformers_amd import causal_product as cpm
+
+    @contextlib.contextmanager
+    def counting():
+        calls = []
+        native = cpm.causal_linear_attention_backward_hip
+        cpm.causal_linear_attention_backward_hip = lambda *a: (calls.append(1), native(*a))[1]
+        try:
+            yield calls
+        finally:
+            cpm.causal_linear_attention_backward_hip = native
+    return counting()
+
+
+def _composition(cla):
+    """Context that makes the module compose its result from operator calls (what sizes and
+    feature maps without a fused kernel get)."""
+    import contextlib
+
+    @contextlib.contextmanager
+    def off():
+        covers = cla.fused_attention_covers
+        cla.fused_attention_covers = lambda *a: False
+        try:
+            yield
+        finally:
+            cla.fused_attention_covers = covers
+    return off()
+
+
+def test_module_takes_the_fused_path_and_agrees_with_the_composition(lib):
     from fast_transformers_amd import attention, masking
     from fast_transformers_amd.attention import causal_linear_attention as cla
     N, L, H, E, M = 2, 700, 4, 64, 64
@@ -189,13 +223,138 @@ def test_module_takes_the_fused_path_without_grad_and_agrees_with_the_compositio
         with torch.no_grad():
             y_fused = module(q, k, v, mask, full, lengths)
         assert calls == [1]
-        qg = q.clone().requires_grad_(True)
-        y_composed = module(qg, k, v, mask, full, lengths)
+        with _composition(cla):
+            y_composed = module(q.clone().requires_grad_(True), k, v, mask, full, lengths)
         assert calls == [1] and y_composed.requires_grad
     finally:
         cla.causal_linear_attention_hip = native
     assert scale_error(y_fused.permute(0, 2, 1, 3), y_composed.detach().permute(0, 2, 1, 3)) <= 1e-5
     gate(y_fused.cpu(), q.cpu(), k.cpu(), v.cpu(), torch.tensor([700, 301]), module.eps)
+
+
+def _dense_attention(q, k, v, lengths, eps):
+    """The closed form of the reference's API test (tests/causal_product/test_causal_product.py:
+    34-40) with the feature map and the key-length mask of the module, on (N, L, H, X) tensors
+    of any float type: differentiable, so that autograd gives the gradients to compare with."""
+    Q = torch.nn.functional.elu(q) + 1
+    K = torch.nn.functional.elu(k) + 1
+    L = q.shape[1]
+    keep = (torch.arange(L, device=q.device)[None, :] < lengths[:, None]).to(q.dtype)
+    K = K * keep[:, :, None, None]
+    QK = torch.einsum("nlhe,nshe->nhls", Q, K)
+    QK = QK * torch.tril(torch.ones(L, L, dtype=q.dtype, device=q.device))
+    Z = 1 / (QK.sum(dim=-1) + eps)                       # (N, H, L)
+    return torch.einsum("nhls,nshm->nlhm", QK, v) * Z.permute(0, 2, 1)[..., None]
+
+
+BACKWARD_SHAPES = [
+    # N, L, H, E, M, key lengths
+    (2, 300, 3, 64, 64, [300, 117]), (1, 1000, 8, 64, 64, [1000]), (3, 257, 2, 32, 32, [257, 40, 200]),
+    (2, 513, 2, 64, 32, [513, 400]), (2, 200, 4, 32, 64, [0, 200]), (1, 33, 1, 64, 64, [33]),
+]
+
+
+@pytest.mark.parametrize("shape", BACKWARD_SHAPES, ids=lambda s: "n%d_l%d_h%d_e%d_m%d" % s[:5])
+def test_backward_against_autograd_in_float64(lib, shape):
+    """ftc_causal_linear_attention_backward (through the autograd Function the module uses)
+    against autograd through the dense closed form in float64; the same closed form in
+    float32 shows what that arithmetic alone costs."""
+    from fast_transformers_amd.causal_product import CausalLinearAttentionFunction
+    N, L, H, E, M, lens = shape
+    q, k, v = inputs(N, L, H, E, M, seed=31 + L)
+    g = torch.randn(N, L, H, M, generator=torch.Generator().manual_seed(32 + L))
+    lengths = torch.tensor(lens)
+    eps = 1e-6
+
+    def grads(dtype, device):
+        qq, kk, vv = (t.to(device=device, dtype=dtype).requires_grad_(True) for t in (q, k, v))
+        out = _dense_attention(qq, kk, vv, lengths.to(device), eps)
+        out.backward(g.to(device=device, dtype=dtype))
+        return [out.detach().cpu()] + [t.grad.cpu() for t in (qq, kk, vv)]
+
+    exact = grads(torch.float64, "cpu")
+    plain = grads(torch.float32, "cuda")
+    qd, kd, vd = (t.cuda().requires_grad_(True) for t in (q, k, v))
+    nlh = lambda t: t.permute(0, 2, 1, 3)
+    out = CausalLinearAttentionFunction.apply(nlh(qd), nlh(kd), nlh(vd), lengths.cuda(), eps)
+    assert lib.ftc_last_kernel().startswith(b"scan_wg_kernel")
+    with _count_backward_calls() as calls:
+        nlh(out).backward(g.cuda())
+    assert calls == [1]
+    torch.cuda.synchronize()
+    got = [nlh(out).detach().cpu()] + [t.grad.cpu() for t in (qd, kd, vd)]
+    for name, a, b, c in zip(("out", "grad_queries", "grad_keys", "grad_values"), got, plain, exact):
+        assert torch.isfinite(a).all(), name
+        nlhx = lambda t: t.permute(0, 2, 1, 3).double()
+        e_hip, e_plain = scale_error(nlhx(a), nlhx(c)), scale_error(nlhx(b), nlhx(c))
+        print("%-13s vs float64: hip %.3e  dense fp32 autograd %.3e" % (name, e_hip, e_plain), flush=True)
+        assert e_hip <= max(4 * e_plain, 5e-6), name
+    # keys at or beyond the key length have no gradient, as in the reference (their features
+    # are multiplied by zero)
+    for n_, len_ in enumerate(lens):
+        assert (got[2][n_, len_:] == 0).all()
+
+
+def test_backward_finite_differences(lib):
+    """Directional derivatives of sum(out * w) along random directions, by central differences
+    of the float64 closed form, against the fused backward's gradients."""
+    from fast_transformers_amd.causal_product import CausalLinearAttentionFunction
+    N, L, H, E, M = 1, 150, 2, 64, 64
+    q, k, v = inputs(N, L, H, E, M, seed=41)
+    w = torch.randn(N, L, H, M, generator=torch.Generator().manual_seed(42))
+    lengths = torch.tensor([131])
+    eps = 1e-6
+    qd, kd, vd = (t.cuda().requires_grad_(True) for t in (q, k, v))
+    nlh = lambda t: t.permute(0, 2, 1, 3)
+    out = CausalLinearAttentionFunction.apply(nlh(qd), nlh(kd), nlh(vd), lengths.cuda(), eps)
+    (nlh(out) * w.cuda()).sum().backward()
+    f = lambda a, b, c: (_dense_attention(a.double(), b.double(), c.double(), lengths, eps) * w.double()).sum()
+    gen = torch.Generator().manual_seed(43)
+    for name, base, grad in (("queries", 0, qd.grad), ("keys", 1, kd.grad), ("values", 2, vd.grad)):
+        for _ in range(3):
+            args = [q, k, v]
+            direction = torch.randn(args[base].shape, generator=gen)
+            h = 1e-4
+            plus, minus = list(args), list(args)
+            plus[base] = args[base].double() + h * direction.double()
+            minus[base] = args[base].double() - h * direction.double()
+            fd = ((f(*plus) - f(*minus)) / (2 * h)).item()
+            an = (grad.cpu().double() * direction.double()).sum().item()
+            print("d/d%s: finite difference %.6e, backward %.6e" % (name, fd, an), flush=True)
+            assert abs(fd - an) <= 1e-4 * max(1.0, abs(fd))
+
+
+def test_module_trains_through_the_fused_backward(lib):
+    """Under grad the module runs the fused forward and its backward, and the parameters'
+    gradients agree with those of the composition of operator calls."""
+    from fast_transformers_amd import attention, masking
+    from fast_transformers_amd.attention import causal_linear_attention as cla
+    N, L, H, E, M = 2, 400, 4, 64, 64
+    q, k, v = (t.cuda() for t in inputs(N, L, H, E, M, seed=51))
+    lengths = masking.LengthMask(torch.tensor([400, 255]).cuda(), max_len=L)
+    full = masking.LengthMask(torch.full((N,), L).cuda(), max_len=L)
+    mask = masking.TriangularCausalMask(L, device="cuda")
+    module = attention.CausalLinearAttention(E).cuda()
+    w = torch.randn(N, L, H, M, generator=torch.Generator().manual_seed(52)).cuda()
+
+    def run():
+        leaves = [t.clone().requires_grad_(True) for t in (q, k, v)]
+        y = module(*leaves, mask, full, lengths)
+        (y * w).sum().backward()
+        return y.detach(), [t.grad for t in leaves]
+
+    with _count_backward_calls() as calls:
+        y_fused, g_fused = run()
+        assert calls == [1]
+        with _composition(cla):
+            y_comp, g_comp = run()
+        assert calls == [1]
+    nlh = lambda t: t.permute(0, 2, 1, 3)
+    assert scale_error(nlh(y_fused), nlh(y_comp)) <= 1e-5
+    for name, a, b in zip(("queries", "keys", "values"), g_fused, g_comp):
+        err = scale_error(nlh(a), nlh(b))
+        print("grad %s: fused against composition %.3e" % (name, err), flush=True)
+        assert err <= 2e-5, name
 
 
 def test_non_finite_inputs_propagate_as_in_the_composition(lib):
