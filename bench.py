@@ -16,7 +16,8 @@ reads Q,K,V and writes the product; backward reads Q,K,V,G and writes dQ,dK,dV),
 flops 14*E*M/2, over the mean of the two launch durations, timed with events on the stream
 the kernels are launched on; both the HBM and the matrix-core fraction are given and the one
 with the larger minimum time is named as the bound.  With the default workload the line also
-carries a few timed steps of cfg3 and cfg5 (``config.secondary``).  ``cpu_baseline`` times
+carries a few timed steps of cfg3 and cfg5 and of the attention module's training step at
+config 4's attention shape (``config.secondary``).  ``cpu_baseline`` times
 the reference's own CPU extension (or, when it is not built, its C restatement) on this box's
 host cores over a bounded number of calls of the same workload.
 """
@@ -347,10 +348,55 @@ def main():
                 "hbm_frac": r["roofline"]["hbm"]["frac"], "mfma_frac": r["roofline"]["mfma"]["frac"],
                 "kernels": r["roofline"]["kernel"], "steps": 10, "warmup": 3}
             torch.cuda.empty_cache()
+        secondary["cfg4_attention_training"] = attention_training_step()
         result["config"]["secondary"] = secondary
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(N, H, L, E, M, seed, args.workload)
     print(json.dumps(result))
+
+
+def attention_training_step(steps=10, warmup=3):
+    """Forward + backward of the CausalLinearAttention module on the attention shape of
+    config 4 (N=10, L=4096, 8 heads, E=M=64, fp32): through the fused entry points (one launch
+    forward; element-wise pass, three scans and prefix-sum pass backward) and through the
+    composition of operator calls that autograd differentiates piece by piece.  Wall clock
+    over `steps` calls after `warmup`, inputs resident."""
+    import torch
+    from fast_transformers_amd import attention, masking
+    from fast_transformers_amd.attention import causal_linear_attention as cla
+
+    N, L, H, E, M = 10, 4096, 8, 64, 64
+    gen = torch.Generator(device="cuda").manual_seed(4)
+    q, k, v, w = (torch.randn(N, L, H, d, device="cuda", generator=gen) for d in (E, E, M, M))
+    lengths = masking.LengthMask(torch.full((N,), L, device="cuda"), max_len=L)
+    mask = masking.TriangularCausalMask(L, device="cuda")
+    module = attention.CausalLinearAttention(E).cuda()
+
+    def step():
+        leaves = [t.detach().requires_grad_(True) for t in (q, k, v)]
+        module(*leaves, mask, lengths, lengths).backward(w)
+
+    def timed():
+        for _ in range(warmup):
+            step()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            step()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) * 1e3 / steps
+
+    fused_ms = timed()
+    covers = cla.fused_attention_covers
+    cla.fused_attention_covers = lambda *a, **kw: False
+    try:
+        composed_ms = timed()
+    finally:
+        cla.fused_attention_covers = covers
+    return {"workload": "CausalLinearAttention forward + backward, N=10 L=4096 H=8 E=M=64 fp32",
+            "fused_ms_per_step": round(fused_ms, 4), "composition_ms_per_step": round(composed_ms, 4),
+            "fused_Mtokens_per_s": round(N * L / (fused_ms * 1e-3) / 1e6, 2),
+            "steps": steps, "warmup": warmup}
 
 
 def encoder_workload(args):
