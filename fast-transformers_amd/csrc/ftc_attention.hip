@@ -26,8 +26,9 @@
 namespace ftc {
 namespace {
 
-constexpr int kRun = 8;                // consecutive positions per thread of the finish kernel
-constexpr int kSegment = 16 * kRun;    // positions per workgroup: 16 groups of 16 lanes
+constexpr int kRun = 4;                    // consecutive positions per thread of the finish kernel
+constexpr int kGroups = 32;                // ... whose workgroup has this many groups of 16 lanes
+constexpr int kSegment = kGroups * kRun;   // positions per workgroup
 
 __device__ __forceinline__ float phi(float x) {
     return x > 0.f ? x + 1.f : __builtin_amdgcn_exp2f(x * 1.44269502f);
@@ -69,10 +70,11 @@ __global__ __launch_bounds__(256) void attn_bwd_prep_kernel(
     int E, int M, int nseg, float *__restrict__ Qf, float *__restrict__ Kf, float *__restrict__ gz,
     float *__restrict__ dd, float *__restrict__ sums) {
     __shared__ float4 part[2][16][16];
-    const int64_t chain = blockIdx.x / nseg;
-    const int seg = blockIdx.x % nseg;
+    // (the heads of one batch entry and segment in neighbouring workgroups: with heads
+    // interleaved in memory their rows lie side by side)
+    const int h = blockIdx.x % H, seg = (blockIdx.x / H) % nseg, n = blockIdx.x / (H * nseg);
+    const int64_t chain = (int64_t)n * H + h;
     const int r = threadIdx.x >> 4, c = threadIdx.x & 15;
-    const int n = (int)(chain / H), h = (int)(chain % H);
     const int len = key_len ? (int)min<int64_t>(key_len[n], L) : L;
     const bool has_e = 4 * c < E, has_m = 4 * c < M;
     const int ce = has_e ? 4 * c : 0, cm = has_m ? 4 * c : 0;
@@ -116,19 +118,20 @@ __global__ __launch_bounds__(256) void attn_bwd_prep_kernel(
     }
 }
 
-// One workgroup per (chain, segment); 16 lanes per position as above, and group r takes the
+// One workgroup of 32 groups per (chain, segment); 16 lanes per position as above, and group r takes the
 // run of kRun consecutive positions seg kSegment + r kRun ...  dq and dk hold the scans'
 // results on entry:
 //   dq[l] = (dq[l] + dd[l] sum_{j <= l} Kf[j]) phi'(q[l])
 //   dk[j] = (dk[j] + sum_{l >= j} dd[l] Qf[l]) phi'(k[j]) [j < key_len]
-__global__ __launch_bounds__(256) void attn_bwd_finish_kernel(
+__global__ __launch_bounds__(16 * kGroups) void attn_bwd_finish_kernel(
     Rows q, Rows k, const int64_t *__restrict__ key_len, const float *__restrict__ dd,
     const float *__restrict__ sums, int H, int L, int E, int nseg, RowsOut dq, RowsOut dk) {
-    __shared__ float4 total[2][16][16];
-    const int64_t chain = blockIdx.x / nseg;
-    const int seg = blockIdx.x % nseg;
+    __shared__ float4 total[2][kGroups][16];
+    // (the heads of one batch entry and segment in neighbouring workgroups: with heads
+    // interleaved in memory their rows lie side by side)
+    const int h = blockIdx.x % H, seg = (blockIdx.x / H) % nseg, n = blockIdx.x / (H * nseg);
+    const int64_t chain = (int64_t)n * H + h;
     const int r = threadIdx.x >> 4, c = threadIdx.x & 15;
-    const int n = (int)(chain / H), h = (int)(chain % H);
     const int len = key_len ? (int)min<int64_t>(key_len[n], L) : L;
     const bool has_e = 4 * c < E;
     const int ce = has_e ? 4 * c : 0;
@@ -166,7 +169,7 @@ __global__ __launch_bounds__(256) void attn_bwd_finish_kernel(
     __syncthreads();
     // and the runs before and after this one in the segment
     for (int i = 0; i < r; i++) ck = ck + total[0][i][c];
-    for (int i = 15; i > r; i--) cq = cq + total[1][i][c];
+    for (int i = kGroups - 1; i > r; i--) cq = cq + total[1][i][c];
     if (!has_e) return;
     if (dq.ptr) {
         float *row = dq.ptr + n * dq.sn + h * dq.sh + ce;
@@ -216,7 +219,7 @@ void launch_attention_backward_finish(const Operand &q, const Operand &k, const 
                                       int64_t L, int E, const OperandOut &dq, const OperandOut &dk,
                                       hipStream_t stream) {
     const int nseg = (int)attention_backward_segments(L);
-    hipLaunchKernelGGL(attn_bwd_finish_kernel, dim3((unsigned)(N * H * nseg)), dim3(256), 0, stream,
+    hipLaunchKernelGGL(attn_bwd_finish_kernel, dim3((unsigned)(N * H * nseg)), dim3(16 * kGroups), 0, stream,
                        rows_of(q), rows_of(k), key_len, dd, sums, (int)H, (int)L, E, nseg, rows_of(dq),
                        rows_of(dk));
 }
