@@ -125,9 +125,10 @@ int tp_exchange_segments(int64_t units, int64_t L, bool wide, int *nseg) {
     if (tuning().tpx == 0) return 0;  // tuning aid
     // Up to 64 chunks the cut chains without an exchange are as fast (cfg2: 30 us either way)
     // and need no workspace.
-    if (units < 1 || (units > 128 && !wide) || total_chunks <= 64) return 0;
+    const bool force = tuning().tpx_segs >= 2;  // tuning aid: also where the rules below say no
+    if (!force && (units < 1 || (units > 128 && !wide) || total_chunks <= 64)) return 0;
     // (wide states: also with more workgroups than CUs, where chains are too long to walk whole)
-    if (units > 128 && total_chunks <= 256) return 0;
+    if (!force && units > 128 && total_chunks <= 256) return 0;
     int64_t want = 256 / units;
     if (wide && units * want != 256) {
         // Workgroups that do not fill whole rounds of 256: the number of segments with the
@@ -157,13 +158,21 @@ int tp_exchange_segments(int64_t units, int64_t L, bool wide, int *nseg) {
 // The chain-parallel kernel's plan for `nscans` scans of a D x F state over chains x L rows:
 // *seg_chunks > 0: an exchange with *nseg segments of that many chunks; else *nseg > 0: chains
 // cut into *nseg segments that need no exchange; both 0: another kernel takes the launch.
+// `mixed`: rows with bf16 among them (the fp16-piece form of the kernel takes those; the plans
+// are those of fp32 rows where the kernel is used at all).
 void tp_plan_compute(int64_t D, int64_t F, int64_t chains, int nscans, int64_t L, int *nseg,
-                     int *seg_chunks, bool forced) {
+                     int *seg_chunks, bool forced, bool mixed) {
     *nseg = *seg_chunks = 0;
     if (!tp_widths(D, F, forced)) return;
     const bool wide = D != 64 || F != 64 || forced;
     const bool others = !forced && mfma_scan_supported_widths(D, F);
     const int64_t units = chains * nscans * tp_fblocks(F);
+    // A single scan over bf16 rows: the kernels that split L multiply such rows as they are,
+    // one matrix instruction per product, and win until there are workgroups for every CU
+    // (forward, 64 x 64, N*H = 80: 33 against 38 us at L=1000, 69 against 110 at L=4096;
+    // N*H = 256: 56 against 47 at L=1000).  The three scans of a backward call are faster
+    // here for up to 128 chains (L=1000, N*H = 80: 50 against 101 us).
+    if (mixed && nscans == 1 && others && units < 256) return;
     // Shapes of the other kernels with 32 rows or columns (a workgroup here has half of its
     // matrix work or half of its consumers to spare for them): measured at N=8, H=16, L=4096,
     // forward + backward, 32 x 128 0.62 against 0.80 ms and 128 x 32 0.76 against 0.78 on whole
@@ -268,12 +277,12 @@ struct TpPlan {
     int nseg, seg_chunks;
 };
 void tp_plan(int64_t D, int64_t F, int64_t chains, int nscans, int64_t L, int *nseg, int *seg_chunks,
-             bool forced = false) {
+             bool forced = false, bool mixed = false) {
     static thread_local PlanMemo<TpPlan> memo;
-    const int64_t key[8] = {D, F, chains, nscans, L, forced ? 1 : 0, 0, 0};
+    const int64_t key[8] = {D, F, chains, nscans, L, forced ? 1 : 0, mixed ? 1 : 0, 0};
     const TpPlan pl = memo.get(key, [&]() {
         TpPlan p;
-        tp_plan_compute(D, F, chains, nscans, L, &p.nseg, &p.seg_chunks, forced);
+        tp_plan_compute(D, F, chains, nscans, L, &p.nseg, &p.seg_chunks, forced, mixed);
         return p;
     });
     *nseg = pl.nseg, *seg_chunks = pl.seg_chunks;
@@ -291,6 +300,13 @@ bool aligned16(const void *ptr, int64_t s0, int64_t s1, int64_t s2, int dtype) {
     return ((uintptr_t)ptr % 16 == 0) && s0 % per16 == 0 && s1 % per16 == 0 && s2 % per16 == 0;
 }
 
+// what the chain-parallel kernel asks of rows: fp32 rows on 16-byte boundaries, bf16 rows (which
+// it reads and writes four values at a time) on 8-byte boundaries
+bool aligned_quads(const void *ptr, int64_t s0, int64_t s1, int64_t s2, int dtype) {
+    if (dtype == FTC_F32) return aligned16(ptr, s0, s1, s2, dtype);
+    return ((uintptr_t)ptr % 8 == 0) && s0 % 4 == 0 && s1 % 4 == 0 && s2 % 4 == 0;
+}
+
 // element-type combinations with a compiled kernel: (a, b, v, out)
 enum Combo { kNone = 0, kFFFF, kBBBF, kFBBB, kBFBB, kBBFB };
 Combo combo_of(const ScanDesc &sd) {
@@ -302,6 +318,12 @@ Combo combo_of(const ScanDesc &sd) {
     if (a == B16 && b == F32 && v == B16 && o == B16) return kBFBB;  // bf16 dK (b = grad_out)
     if (a == B16 && b == B16 && v == F32 && o == B16) return kBBFB;  // bf16 dV (v = grad_out)
     return kNone;
+}
+
+// chain-parallel scans of states of up to 64 rows run on the fp16 matrix path
+// (ftc_tph_kernel.h: two scaled fp16 pieces per value), wider ones on three bf16 pieces
+bool tph_takes_rows(int64_t D) {
+    return D <= 64 && tuning().tph != 0;  // (FTC_TPH=0: tuning aid)
 }
 
 // rows must not overlap (the descriptor's end marks the first row outside the segment) and
@@ -384,16 +406,21 @@ bool mfma_tp_takes(const ScanDesc *scans, int nscans, int64_t N, int64_t H, int6
     const int D = scans[0].a.width, F = scans[0].v.width;
     if (nscans < 1 || nscans > kMaxScans || !tp_widths(D, F, forced)) return false;
     int64_t widest_stride = 0;
+    bool mixed = false;
     for (int i = 0; i < nscans; i++) {
         const ScanDesc &sd = scans[i];
-        if (combo_of(sd) != kFFFF || sd.a.width != D || sd.v.width != F) return false;
+        const Combo combo = combo_of(sd);
+        mixed = mixed || combo != kFFFF;
+        // rows with bf16 among them: the fp16-piece form of the kernel only
+        if (combo == kNone || (combo != kFFFF && !tph_takes_rows(D))) return false;
+        if (sd.a.width != D || sd.v.width != F) return false;
         if (L > 1 && !(stride_ok(sd.a.stride_l, D) && stride_ok(sd.b.stride_l, D) &&
                        stride_ok(sd.v.stride_l, F) && stride_ok(sd.out.stride_l, F)))
             return false;
-        if (!(aligned16(sd.a.ptr, sd.a.stride_n, sd.a.stride_h, sd.a.stride_l, FTC_F32) &&
-              aligned16(sd.b.ptr, sd.b.stride_n, sd.b.stride_h, sd.b.stride_l, FTC_F32) &&
-              aligned16(sd.v.ptr, sd.v.stride_n, sd.v.stride_h, sd.v.stride_l, FTC_F32) &&
-              aligned16(sd.out.ptr, sd.out.stride_n, sd.out.stride_h, sd.out.stride_l, FTC_F32)))
+        if (!(aligned_quads(sd.a.ptr, sd.a.stride_n, sd.a.stride_h, sd.a.stride_l, sd.a.dtype) &&
+              aligned_quads(sd.b.ptr, sd.b.stride_n, sd.b.stride_h, sd.b.stride_l, sd.b.dtype) &&
+              aligned_quads(sd.v.ptr, sd.v.stride_n, sd.v.stride_h, sd.v.stride_l, sd.v.dtype) &&
+              aligned_quads(sd.out.ptr, sd.out.stride_n, sd.out.stride_h, sd.out.stride_l, sd.out.dtype)))
             return false;
         widest_stride = std::max(widest_stride, std::max(std::max(sd.a.stride_l, sd.b.stride_l),
                                                          std::max(sd.v.stride_l, sd.out.stride_l)));
@@ -402,7 +429,7 @@ bool mfma_tp_takes(const ScanDesc *scans, int nscans, int64_t N, int64_t H, int6
     if ((L + 2 * kChunk) * std::max<int64_t>(widest_stride, std::max(D, F)) * 4 >= 0x7fffffffLL)
         return false;
     int nseg = 0, seg_chunks = 0;
-    tp_plan(D, F, std::max<int64_t>(1, N * H), nscans, L, &nseg, &seg_chunks, forced);
+    tp_plan(D, F, std::max<int64_t>(1, N * H), nscans, L, &nseg, &seg_chunks, forced, mixed);
     return nseg > 0;
 }
 
@@ -428,7 +455,9 @@ int mfma_scan(const ScanDesc *scans, int nscans, int64_t N, int64_t H, int64_t L
     const int64_t fblocks = tp_shape ? tp_fblocks(F) : 1;
     int tpx_nseg = 0, tpx_seg_chunks = 0, tp_nseg = 0;
     if (tp_shape) {
-        tp_plan(D, F, chains, nscans, L, &tpx_nseg, &tpx_seg_chunks, forced);
+        bool any_bf16 = false;
+        for (int i = 0; i < nscans; i++) any_bf16 = any_bf16 || combo_of(scans[i]) != kFFFF;
+        tp_plan(D, F, chains, nscans, L, &tpx_nseg, &tpx_seg_chunks, forced, any_bf16);
         if (tpx_seg_chunks == 0) tp_nseg = tpx_nseg, tpx_nseg = 0;
     }
     const bool tp = tp_nseg > 0 || tpx_seg_chunks > 0;
@@ -474,7 +503,9 @@ int mfma_scan(const ScanDesc *scans, int nscans, int64_t N, int64_t H, int64_t L
         o.v_sn = sd.v.stride_n, o.v_sh = sd.v.stride_h, o.v_sl = row_stride(sd.v.stride_l, F);
         o.o_sn = sd.out.stride_n, o.o_sh = sd.out.stride_h, o.o_sl = row_stride(sd.out.stride_l, F);
         o.rev = sd.reverse ? 1 : 0;
-        o.pad = 0;
+        // (element types of the rows, for the kernel that takes them scan by scan)
+        o.pad = (sd.a.dtype == FTC_BF16 ? kRowsBf16A : 0) | (sd.b.dtype == FTC_BF16 ? kRowsBf16B : 0) |
+                (sd.v.dtype == FTC_BF16 ? kRowsBf16V : 0) | (sd.out.dtype == FTC_BF16 ? kRowsBf16Out : 0);
         o.s0 = sd.initial.ptr;
         o.s0_sn = sd.initial.stride_n, o.s0_sh = sd.initial.stride_h, o.s0_sd = sd.initial.stride_d;
         o.s_out = sd.final_.ptr;
@@ -517,16 +548,16 @@ int mfma_scan(const ScanDesc *scans, int nscans, int64_t N, int64_t H, int64_t L
     args.group = std::min(args.group, 64);
     while ((pl.nseg + args.group - 1) / args.group > 64) args.group++;
 
-    for (int i = 1; i < nscans; i++)
-        if (combo_of(scans[i]) != combo || scans[i].a.width != D || scans[i].v.width != F)
+    const bool half_pieces = tp && tph_takes_rows(D);
+    bool mixed = false;  // rows with bf16 among them
+    for (int i = 0; i < nscans; i++) {
+        mixed = mixed || combo_of(scans[i]) != kFFFF;
+        if ((!half_pieces && combo_of(scans[i]) != combo) || scans[i].a.width != D || scans[i].v.width != F)
             return fail(FTC_ERR_INVALID, "scans of one launch must share widths and dtypes");
+    }
     // fp32 states of up to 64 rows: the kernel that feeds its fragments from LDS tiles
     bool dma = D <= 64 && combo == kFFFF;
     if (tuning().dma >= 0) dma = dma && tuning().dma != 0;  // tuning aid
-    // chain-parallel scans of states of up to 64 rows run on the fp16 matrix path
-    // (ftc_tph_kernel.h: two scaled fp16 pieces per value), wider ones on three bf16 pieces
-    bool half_pieces = tp && D <= 64;
-    if (tuning().tph >= 0) half_pieces = half_pieces && tuning().tph != 0;  // tuning aid
     note_kernel(tp ? (half_pieces ? (tpx_seg_chunks > 0 ? "scan_tph_kernel (exchange)" : "scan_tph_kernel")
                                   : (tpx_seg_chunks > 0 ? "scan_tp_kernel (exchange)" : "scan_tp_kernel"))
                 : wg ? (fused ? "scan_wg_kernel<NORM>" : "scan_wg_kernel")
@@ -547,7 +578,7 @@ int mfma_scan(const ScanDesc *scans, int nscans, int64_t N, int64_t H, int64_t L
     }
     if (tp) {
         if (half_pieces)
-            launch_scan_tph(workspace, args, stream);
+            launch_scan_tph(workspace, args, mixed, stream);
         else
             launch_scan_tp(workspace, args, stream);
     } else if (wg) {

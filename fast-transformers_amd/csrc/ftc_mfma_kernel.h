@@ -400,6 +400,9 @@ struct StateExchange {
 // One scan of a launch.  A launch runs up to kMaxScans independent scans of the same
 // (D, F, N, H, L) side by side (the three gradients of a backward call, the column slices
 // of a wide output), so that their launch gaps and wait times overlap.
+// element types of a scan's rows as ScanOperands::pad carries them: bits set for bf16 rows
+constexpr int kRowsBf16A = 1, kRowsBf16B = 2, kRowsBf16V = 4, kRowsBf16Out = 8;
+
 struct ScanOperands {
     const void *a, *b, *v;
     void *out;
@@ -408,7 +411,7 @@ struct ScanOperands {
     int64_t v_sn, v_sh, v_sl;
     int64_t o_sn, o_sh, o_sl;
     int32_t rev;  // 0: j <= l, walk up; 1: j >= l, walk down
-    int32_t pad;
+    int32_t pad;  // kRowsBf16* bits (read by the kernel that takes rows of either type scan by scan)
     // optional D x F fp32 states per chain (null: none): the state the scan starts from and
     // the state after its last position; strides in elements, unit stride along F
     const float *s0;

@@ -1,6 +1,8 @@
-// Chain-parallel form of the MFMA causal scan for gfx950 on the fp16 matrix path: all-fp32
-// rows, states of up to 64 x 64 per workgroup (output columns beyond 64 have a workgroup of
-// their own, widths that do not fill the block are clipped).
+// Chain-parallel form of the MFMA causal scan for gfx950 on the fp16 matrix path: fp32 rows
+// (or, in the MIX form of the kernel, any operand in bf16: such rows are widened as they arrive
+// and rounded to nearest even as they leave; their low pieces are zero), states of up to
+// 64 x 64 per workgroup (output columns beyond 64 have a workgroup of their own, widths that do
+// not fill the block are clipped).
 //
 //   out[c, l, f] = sum_{j <= l} (a[c,l,:] . b[c,j,:]) * v[c,j,f]      (REV: j >= l)
 //
@@ -176,9 +178,15 @@ __device__ __forceinline__ void raise_slot(lds_u32_t *slots, int k, int pos, con
     }
 }
 
+// four bf16 values in two words -> the same values as fp32 bit patterns
+__device__ __forceinline__ u32x4 widen_bf16_quad(const u32x4 r) {
+    return u32x4{r.x << 16, r.x & 0xffff0000u, r.y << 16, r.y & 0xffff0000u};
+}
+
 // KS: groups of 32 rows of the state (1: a state of up to 32 rows, which skips the matrix
-// instructions and fragment reads of the empty half)
-template <int KS>
+// instructions and fragment reads of the empty half).  MIX: rows of either element type, as
+// ScanOperands::pad says scan by scan (false: all rows fp32).
+template <int KS, bool MIX>
 __global__ __launch_bounds__(768, 3) void scan_tph_kernel(uint32_t *__restrict__ ws_ptr, ScanArgs p) {
     constexpr int D = 64, F = 64;              // one block of state rows and of output columns
     constexpr int T = 512;                     // producer lanes (eight wavefronts)
@@ -284,18 +292,21 @@ __global__ __launch_bounds__(768, 3) void scan_tph_kernel(uint32_t *__restrict__
     if (producer) {
         // =========================== producers ===========================
         const int ptid = (wave - 4) * 64 + lane;
-        const uint32_t a_slb = (uint32_t)op.a_sl * 4, b_slb = (uint32_t)op.b_sl * 4,
-                       v_slb = (uint32_t)op.v_sl * 4;
-        const char *a_seg = (const char *)op.a + ((int64_t)n * op.a_sn + (int64_t)h * op.a_sh) * 4;
-        const char *b_seg = (const char *)op.b + ((int64_t)n * op.b_sn + (int64_t)h * op.b_sh) * 4;
+        const bool a_bf = MIX && (op.pad & kRowsBf16A), b_bf = MIX && (op.pad & kRowsBf16B),
+                   v_bf = MIX && (op.pad & kRowsBf16V);
+        const uint32_t a_es = a_bf ? 2 : 4, b_es = b_bf ? 2 : 4, v_es = v_bf ? 2 : 4;  // bytes
+        const uint32_t a_slb = (uint32_t)op.a_sl * a_es, b_slb = (uint32_t)op.b_sl * b_es,
+                       v_slb = (uint32_t)op.v_sl * v_es;
+        const char *a_seg = (const char *)op.a + ((int64_t)n * op.a_sn + (int64_t)h * op.a_sh) * a_es;
+        const char *b_seg = (const char *)op.b + ((int64_t)n * op.b_sn + (int64_t)h * op.b_sh) * b_es;
         const char *v_seg = (const char *)op.v +
-                            ((int64_t)n * op.v_sn + (int64_t)h * op.v_sh + F * fb) * 4;
+                            ((int64_t)n * op.v_sn + (int64_t)h * op.v_sh + F * fb) * v_es;
         const __amdgpu_buffer_rsrc_t a_rs = __builtin_amdgcn_make_buffer_rsrc(
-            (void *)a_seg, 0, (rows - 1) * a_slb + Dw * 4, kRsrcFlags);
+            (void *)a_seg, 0, (rows - 1) * a_slb + Dw * a_es, kRsrcFlags);
         const __amdgpu_buffer_rsrc_t b_rs = __builtin_amdgcn_make_buffer_rsrc(
-            (void *)b_seg, 0, (rows - 1) * b_slb + Dw * 4, kRsrcFlags);
+            (void *)b_seg, 0, (rows - 1) * b_slb + Dw * b_es, kRsrcFlags);
         const __amdgpu_buffer_rsrc_t v_rs = __builtin_amdgcn_make_buffer_rsrc(
-            (void *)v_seg, 0, (rows - 1) * v_slb + fw * 4, kRsrcFlags);
+            (void *)v_seg, 0, (rows - 1) * v_slb + fw * v_es, kRsrcFlags);
         // One quad (four columns of one row) of every operand per lane and position.  Widths
         // that do not fill the block: a lane whose four columns lie beyond the width asks
         // outside the descriptor and cuts zeros (widths are multiples of 4).
@@ -303,16 +314,30 @@ __global__ __launch_bounds__(768, 3) void scan_tph_kernel(uint32_t *__restrict__
         const int prow = ptid / QA, pc4 = ptid % QA;
         const bool ab_in = 4 * pc4 < Dw;
         const bool v_in = 4 * pc4 < fw;
-        const uint32_t a_goff = (uint32_t)prow * a_slb + 16u * pc4,
-                       b_goff = (uint32_t)prow * b_slb + 16u * pc4,
-                       v_goff = (uint32_t)prow * v_slb + 16u * pc4;
+        const uint32_t a_goff = (uint32_t)prow * a_slb + 4u * a_es * pc4,
+                       b_goff = (uint32_t)prow * b_slb + 4u * b_es * pc4,
+                       v_goff = (uint32_t)prow * v_slb + 4u * v_es * pc4;
         const int a_waddr = TpSwizzle<RBA>::addr(prow, 8 * pc4),
                   b_waddr = TpSwizzle<RBA>::addr(prow, 2 * b_tile_column(4 * pc4)),
                   v_waddr = TpSwizzle<RBV>::addr(prow, 8 * pc4);
-        struct Raw {
+        struct Raw {  // (bf16 rows: the quad in the first two words)
             u32x4 a, b, v;
         };
         Raw raw[PF];
+        // (MIX: the same two 8-byte requests whatever the type -- no branch around a request,
+        // which would end the run of requests in flight; the second one of a bf16 quad asks
+        // outside the descriptor)
+        auto load_quad = [&](const __amdgpu_buffer_rsrc_t rs, uint32_t off, bool bf) -> u32x4 {
+            if (!MIX) return __builtin_amdgcn_raw_buffer_load_b128(rs, off, 0, 0);
+            const u32x2 lo = __builtin_amdgcn_raw_buffer_load_b64(rs, off, 0, 0);
+            const u32x2 hi = __builtin_amdgcn_raw_buffer_load_b64(rs, bf ? kNoRow : off + 8u, 0, 0);
+            return u32x4{lo.x, lo.y, hi.x, hi.y};
+        };
+        auto widen = [&](const u32x4 r, bool bf) -> u32x4 {
+            if (!MIX) return r;
+            const u32x4 wide = widen_bf16_quad(r);
+            return u32x4{bf ? wide.x : r.x, bf ? wide.y : r.y, bf ? wide.z : r.z, bf ? wide.w : r.w};
+        };
         // Every request is made every time, whether its rows exist or not (a chunk walked for
         // its state alone needs no rows of a; positions past the end of the walk have no
         // rows): a request outside the descriptor costs no memory traffic and reads as zero,
@@ -321,25 +346,23 @@ __global__ __launch_bounds__(768, 3) void scan_tph_kernel(uint32_t *__restrict__
         auto fetch = [&](Raw &r, int v) {  // v: position of the walk
             const int row0 = v < nwalk ? chunk_row0(walk_chunk(v)) : -2 * kChunk;
             const int row0_x = v >= n1 ? row0 : -2 * kChunk;
-            r.a = __builtin_amdgcn_raw_buffer_load_b128(
-                a_rs, ab_in ? a_goff + (uint32_t)row0_x * a_slb : kNoRow, 0, 0);
-            r.b = __builtin_amdgcn_raw_buffer_load_b128(
-                b_rs, ab_in ? b_goff + (uint32_t)row0 * b_slb : kNoRow, 0, 0);
-            r.v = __builtin_amdgcn_raw_buffer_load_b128(
-                v_rs, v_in ? v_goff + (uint32_t)row0 * v_slb : kNoRow, 0, 0);
+            r.a = load_quad(a_rs, ab_in ? a_goff + (uint32_t)row0_x * a_slb : kNoRow, a_bf);
+            r.b = load_quad(b_rs, ab_in ? b_goff + (uint32_t)row0 * b_slb : kNoRow, b_bf);
+            r.v = load_quad(v_rs, v_in ? v_goff + (uint32_t)row0 * v_slb : kNoRow, v_bf);
         };
         // the largest magnitudes of the rows of a position against the ceilings (rows that
         // were not asked for read as zeros); k: that position's slot
         auto look_ahead = [&](const Raw &r, int k, int pos) {
-            raise_slot(slots, k, pos, ce, max_abs4(r.a, 0.f), max_abs4(r.b, 0.f), max_abs4(r.v, 0.f), lane);
+            raise_slot(slots, k, pos, ce, max_abs4(widen(r.a, a_bf), 0.f), max_abs4(widen(r.b, b_bf), 0.f),
+                       max_abs4(widen(r.v, v_bf), 0.f), lane);
         };
         // A position of the walk goes to its LDS buffer through register set (position % PF).
         // The first n1 positions only feed the state: no piece of a.
         auto cut = [&](const Raw &r, int buf, bool own) {
             lds_char *const pc = unit_pc + buf * kBufBytes;
-            if (own) cut_quad_to_lds(r.a, ce.scale_a(), pc, kTileA, a_waddr);
-            cut_quad_to_lds(r.b, ce.scale_b(), pc + kOffB, kTileA, b_waddr);
-            cut_quad_to_lds(r.v, ce.scale_v(), pc + kOffV, kTileV, v_waddr);
+            if (own) cut_quad_to_lds(widen(r.a, a_bf), ce.scale_a(), pc, kTileA, a_waddr);
+            cut_quad_to_lds(widen(r.b, b_bf), ce.scale_b(), pc + kOffB, kTileA, b_waddr);
+            cut_quad_to_lds(widen(r.v, v_bf), ce.scale_v(), pc + kOffV, kTileV, v_waddr);
             if (!own) asm volatile("" ::"v"(r.a));
         };
 #pragma unroll
@@ -390,10 +413,12 @@ __global__ __launch_bounds__(768, 3) void scan_tph_kernel(uint32_t *__restrict__
 
     // =========================== consumers ===========================
     const int ln = lane & 15, g = lane >> 4;
-    const uint32_t o_slb = (uint32_t)op.o_sl * 4;
-    char *o_seg = (char *)op.out + ((int64_t)n * op.o_sn + (int64_t)h * op.o_sh + F * fb) * 4;
+    const bool o_bf = MIX && (op.pad & kRowsBf16Out);
+    const uint32_t o_es = o_bf ? 2 : 4;  // bytes
+    const uint32_t o_slb = (uint32_t)op.o_sl * o_es;
+    char *o_seg = (char *)op.out + ((int64_t)n * op.o_sn + (int64_t)h * op.o_sh + F * fb) * o_es;
     const __amdgpu_buffer_rsrc_t o_rs =
-        __builtin_amdgcn_make_buffer_rsrc((void *)o_seg, 0, (rows - 1) * o_slb + fw * 4, kRsrcFlags);
+        __builtin_amdgcn_make_buffer_rsrc((void *)o_seg, 0, (rows - 1) * o_slb + fw * o_es, kRsrcFlags);
     // Pt quadrant of this wavefront (see scan_tp_kernel)
     const int jh = w == 0 ? 0 : w == 1 ? 1 : ((w == 2) == REV ? 1 : 0);
     const int ih = w == 0 ? 0 : w == 1 ? 1 : 1 - jh;
@@ -432,7 +457,7 @@ __global__ __launch_bounds__(768, 3) void scan_tph_kernel(uint32_t *__restrict__
     uint32_t o_lane[2];
 #pragma unroll
     for (int x = 0; x < 2; x++)
-        o_lane[x] = (uint32_t)(16 * (x ^ ih) + ln) * o_slb + 4u * (16 * w + 4 * g);
+        o_lane[x] = (uint32_t)(16 * (x ^ ih) + ln) * o_slb + o_es * (16 * w + 4 * g);
     const bool o_in = 16 * w + 4 * g < fw;  // (columns beyond the width are not stored)
 
     constexpr int NT = 2 * KS;  // state tiles of 16 rows
@@ -613,11 +638,18 @@ __global__ __launch_bounds__(768, 3) void scan_tph_kernel(uint32_t *__restrict__
     int Xo = 0;
     uint32_t o_off = 0x80000000u;
     auto store_rows = [&](int x) {
-        const u32x4 r = {__float_as_uint(__builtin_amdgcn_ldexpf(O[x][0], Xo)),
-                         __float_as_uint(__builtin_amdgcn_ldexpf(O[x][1], Xo)),
-                         __float_as_uint(__builtin_amdgcn_ldexpf(O[x][2], Xo)),
-                         __float_as_uint(__builtin_amdgcn_ldexpf(O[x][3], Xo))};
-        __builtin_amdgcn_raw_buffer_store_b128(r, o_rs, o_in ? o_off + o_lane[x] : kNoRow, 0, 0);
+        const float y0 = __builtin_amdgcn_ldexpf(O[x][0], Xo), y1 = __builtin_amdgcn_ldexpf(O[x][1], Xo),
+                    y2 = __builtin_amdgcn_ldexpf(O[x][2], Xo), y3 = __builtin_amdgcn_ldexpf(O[x][3], Xo);
+        const uint32_t at = o_in ? o_off + o_lane[x] : kNoRow;
+        if (!MIX) {
+            buffer_store_out(o_rs, at, y0, y1, y2, y3, (float *)nullptr);
+        } else {  // two 8-byte stores whatever the type; the second one of a bf16 quad goes nowhere
+            const u32x2 first = {o_bf ? pack_bf16_rne(y0, y1) : __float_as_uint(y0),
+                                 o_bf ? pack_bf16_rne(y2, y3) : __float_as_uint(y1)};
+            const u32x2 second = {__float_as_uint(y2), __float_as_uint(y3)};
+            __builtin_amdgcn_raw_buffer_store_b64(first, o_rs, at, 0, 0);
+            __builtin_amdgcn_raw_buffer_store_b64(second, o_rs, o_bf ? kNoRow : at + 8u, 0, 0);
+        }
     };
     const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
     // One chunk, in LDS buffer B (a compile-time number, so that every LDS access of the body

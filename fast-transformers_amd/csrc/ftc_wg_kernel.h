@@ -754,7 +754,8 @@ bool scan_wg_norm_covers(int D, int F);
 // chain-parallel form (ftc_tp_kernel.h): one workgroup per chain of a 64 x 64 all-fp32 scan
 void launch_scan_tp(void *ws, const ScanArgs &args, hipStream_t stream);
 // the same on the fp16 matrix path (ftc_tph_kernel.h): states of up to 64 rows
-void launch_scan_tph(void *ws, const ScanArgs &args, hipStream_t stream);
+// `mixed`: some rows are bf16 (ScanOperands::pad of every scan says which)
+void launch_scan_tph(void *ws, const ScanArgs &args, bool mixed, hipStream_t stream);
 
 }  // namespace mfma
 }  // namespace ftc

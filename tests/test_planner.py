@@ -63,7 +63,19 @@ def test_what_the_chain_parallel_kernel_leaves_to_the_others():
     assert lines((10, 8, 1000, 32), (10, 8, 1000, 128))[0].startswith("scan_tph_kernel:")
     assert lines((4, 16, 16384, 32), (4, 16, 16384, 128))[0].startswith("scan_dma_kernel")
     assert lines((1, 3, 500, 128), (1, 3, 500, 128))[0].startswith("scan_mfma_kernel")  # few chains
-    assert lines((4, 8, 1000, 64), (4, 8, 1000, 64), dtype=_native.FTC_BF16)[0] \
+    # bf16 rows: a single scan stays with the kernels that multiply such rows as they are
+    # until there is a workgroup for every CU; the three scans of a backward call, and widths
+    # that those kernels would only take as padded copies, go to the chain-parallel kernel
+    bf16 = dict(dtype=_native.FTC_BF16)
+    assert lines((4, 8, 1000, 64), (4, 8, 1000, 64), **bf16)[0].startswith("scan_mfma_kernel")
+    assert lines((10, 8, 1000, 64), (10, 8, 1000, 64), **bf16)[0].startswith("scan_mfma_kernel")
+    assert lines((16, 16, 1000, 64), (16, 16, 1000, 64), **bf16)[0].startswith("scan_tph_kernel:")
+    assert lines((10, 8, 1000, 64), (10, 8, 1000, 64), backward=True, **bf16)[0] \
+        .startswith("scan_tph_kernel: 3 scans")
+    assert lines((6, 8, 257, 48), (6, 8, 257, 40), **bf16)[0].startswith("scan_tph_kernel:")
+    assert lines((8, 8, 130, 20), (8, 8, 130, 20), **bf16)[0].startswith("scan_tph_kernel:")
+    # (rows of 128 values: no fp16-piece form, and the bf16-piece form takes fp32 rows only)
+    assert lines((10, 8, 1000, 128), (10, 8, 1000, 128), backward=True, **bf16)[0] \
         .startswith("scan_mfma_kernel")
     # odd widths: zero-padded dense copies for the matrix-core kernels when there are enough
     # rows to pay for the extra launches; states of more than 128 rows stay generic
