@@ -31,7 +31,7 @@ static thread_local char g_error[512] = "";
 static thread_local const char *g_kernel = "";
 void note_kernel(const char *name) { g_kernel = name; }
 static thread_local bool g_plan_only = false;
-static thread_local char g_plan[2048] = "";
+static thread_local char g_plan[16384] = "";
 bool plan_only() { return g_plan_only; }
 
 // ---- tuning aids from the environment, read once -------------------------------------------
@@ -239,6 +239,17 @@ __global__ __launch_bounds__(256) void add_rows_kernel(float *strided, int64_t s
         Vec *row = (Vec *)(strided + (chain / H) * sn + (chain % H) * sh + (int64_t)l * sl + c0);
         *row += *(const Vec *)(dense + (chain * L + l) * w + c0);
     }
+}
+
+// the same for rows of any width and alignment, one value at a time
+__global__ __launch_bounds__(256) void add_rows_any_kernel(float *strided, int64_t sn, int64_t sh,
+                                                           int64_t sl, int64_t H, int64_t L,
+                                                           int64_t chains, int w, const float *dense) {
+    const uint32_t j = blockIdx.x * 256u + threadIdx.x;
+    if (j >= (uint32_t)L * (uint32_t)w) return;
+    const uint32_t l = j / (uint32_t)w, c = j % (uint32_t)w;
+    for (int64_t chain = blockIdx.y; chain < chains; chain += gridDim.y)
+        strided[(chain / H) * sn + (chain % H) * sh + (int64_t)l * sl + c] += dense[(chain * L + l) * w + c];
 }
 
 // workspace of the launches of a split (the largest need among them) and of the buffers that
@@ -513,6 +524,87 @@ int padded_scans(const ScanDesc *scans, int n, const bool *take, int64_t N, int6
     return FTC_OK;
 }
 
+// ---- rows of more than 512 values: column slices and row parts of at most 512 ---------------
+//
+// Output columns are independent of each other, and out_l = sum_d a[l, d] (...) is a sum over d:
+// a scan whose v rows are wider than 512 is run slice by slice of the columns, one whose a and
+// b rows are wider than 512 part by part of those columns, all parts but the first into a
+// buffer in the workspace that is then added to the first one's rows.  Every piece is a scan
+// of at most 512 x 512 and goes through run_scans like any other.  fp32 rows only.
+constexpr int64_t kWidestRows = kGenericMaxDim;
+bool wide_shape(int64_t D, int64_t F) { return D > kWidestRows || F > kWidestRows; }
+// the pieces: equal widths (multiples of 4 of a and b, of 32 of v and out), the last one shorter
+int64_t wide_part_width(int64_t W, int64_t multiple) {
+    const int64_t parts = (W + kWidestRows - 1) / kWidestRows;
+    return std::min<int64_t>(kWidestRows, round_up((W + parts - 1) / parts, multiple));
+}
+// workspace of a wide scan: that of its largest piece, then the buffer of the later row parts
+int64_t wide_scan_workspace_bytes(int64_t N, int64_t H, int64_t L, int64_t D, int64_t F,
+                                  int64_t *piece_bytes) {
+    const int64_t dw = wide_part_width(D, 4), fw = wide_part_width(F, 32);
+    int64_t ws = FTC_WORKSPACE_CONTROL_BYTES;
+    for (int64_t d : {dw, D % dw})
+        for (int64_t f : {fw, F % fw})
+            if (d > 0 && f > 0) ws = std::max(ws, scan_workspace_bytes(N, H, L, d, f));
+    ws = round_up(ws, 256);
+    if (piece_bytes) *piece_bytes = ws;
+    return ws + (D > dw ? round_up(N * H * L * fw * 4, 256) : 0);
+}
+
+int wide_scan(const ScanDesc &scan, int64_t N, int64_t H, int64_t L, void *workspace,
+              size_t workspace_bytes, hipStream_t stream) {
+    const int64_t D = scan.a.width, F = scan.v.width;
+    if (scan.a.dtype != FTC_F32 || scan.b.dtype != FTC_F32 || scan.v.dtype != FTC_F32 ||
+        scan.out.dtype != FTC_F32)
+        return fail(FTC_ERR_UNSUPPORTED, "rows of more than %d values must be fp32", (int)kWidestRows);
+    const int64_t dw = wide_part_width(D, 4), fw = wide_part_width(F, 32);
+    int64_t ws_piece = 0;
+    const int64_t need = wide_scan_workspace_bytes(N, H, L, D, F, &ws_piece);
+    if (!plan_only() && (!workspace || (int64_t)workspace_bytes < need || (uintptr_t)workspace % 256 != 0))
+        return fail(FTC_ERR_WORKSPACE, "workspace of %lld bytes (256-byte aligned) needed, %zu given",
+                    (long long)need, workspace_bytes);
+    float *later = (float *)((char *)workspace + ws_piece);
+    for (int64_t col = 0; col < F; col += fw) {
+        const int64_t f = std::min(fw, F - col);
+        for (int64_t row = 0; row < D; row += dw) {
+            const int64_t d = std::min(dw, D - row);
+            ScanDesc piece = scan;
+            piece.a.ptr = (const float *)scan.a.ptr + row, piece.a.width = (int32_t)d;
+            piece.b.ptr = (const float *)scan.b.ptr + row, piece.b.width = (int32_t)d;
+            piece.v.ptr = (const float *)scan.v.ptr + col, piece.v.width = (int32_t)f;
+            piece.out.ptr = (float *)scan.out.ptr + col, piece.out.width = (int32_t)f;
+            if (piece.initial.ptr) piece.initial.ptr += row * piece.initial.stride_d + col;
+            if (piece.final_.ptr) piece.final_.ptr += row * piece.final_.stride_d + col;
+            if (row > 0) piece.out = OperandOut{later, H * L * f, L * f, f, FTC_F32, (int32_t)f};
+            const int rc = run_scans(&piece, 1, N, H, L, workspace, (size_t)ws_piece, stream, true);
+            if (rc) return rc;
+            if (row == 0) continue;
+            if (plan_only()) {
+                note_plan("add_rows_kernel: rows %lld .. of the state, columns %lld ..: result added to "
+                          "the first part's, workspace %lld bytes", (long long)row, (long long)col,
+                          (long long)need);
+                continue;
+            }
+            float *first = (float *)scan.out.ptr + col;
+            const unsigned chains_y = (unsigned)std::min<int64_t>(N * H, 65535);
+            const bool quads = f % 4 == 0 && (uintptr_t)first % 16 == 0 && scan.out.stride_n % 4 == 0 &&
+                               scan.out.stride_h % 4 == 0 && scan.out.stride_l % 4 == 0;
+            if (L * f >= 0x7fffffffLL) return fail(FTC_ERR_UNSUPPORTED, "L x M beyond 31 bits");
+            if (quads)
+                hipLaunchKernelGGL(add_rows_kernel, dim3((unsigned)((L * (f / 4) + 255) / 256), chains_y),
+                                   dim3(256), 0, stream, first, scan.out.stride_n, scan.out.stride_h,
+                                   scan.out.stride_l, H, L, N * H, (int)f, (const float *)later);
+            else
+                hipLaunchKernelGGL(add_rows_any_kernel, dim3((unsigned)((L * f + 255) / 256), chains_y),
+                                   dim3(256), 0, stream, first, scan.out.stride_n, scan.out.stride_h,
+                                   scan.out.stride_l, H, L, N * H, (int)f, (const float *)later);
+            const hipError_t err = hipGetLastError();
+            if (err != hipSuccess) return fail(FTC_ERR_HIP, "add launch failed: %s", hipGetErrorString(err));
+        }
+    }
+    return FTC_OK;
+}
+
 // whether a scan that the matrix-core kernels do not take as it is may go the padded way
 bool pad_eligible(const ScanDesc &sc, int64_t rows) {
     const int Dp = padded_rows(sc.a.width);
@@ -533,6 +625,12 @@ int run_scans(const ScanDesc *scans, int n, int64_t N, int64_t H, int64_t L, voi
     // The scans of one shape go to the chain-parallel kernel together where it takes them
     // (whole scans: a column slice made below is never offered to it).
     bool offered[kMfmaMaxScans] = {};
+    for (int i = 0; i < n; i++) {
+        if (!wide_shape(scans[i].a.width, scans[i].v.width)) continue;
+        const int rc = wide_scan(scans[i], N, H, L, workspace, workspace_bytes, stream);
+        if (rc) return rc;
+        offered[i] = taken[i] = true;
+    }
     for (int i = 0; i < n; i++) {
         if (offered[i]) continue;
         ScanDesc group[kMfmaMaxScans];
@@ -609,6 +707,7 @@ int run_scans(const ScanDesc *scans, int n, int64_t N, int64_t H, int64_t L, voi
 // needs at the least (without them such a scan runs on the generic kernel).
 int64_t scan_workspace_bytes(int64_t N, int64_t H, int64_t L, int64_t D, int64_t F, bool with_pad,
                              bool bf16) {
+    if (wide_shape(D, F)) return wide_scan_workspace_bytes(N, H, L, D, F, nullptr);
     int64_t need = generic_scan_workspace_bytes(N, H, L, D, F);
     int widths[kMfmaMaxSlices];
     const int nslices = mfma_slice_widths(D, F, widths);
@@ -681,8 +780,8 @@ int64_t ftc_causal_dot_product_workspace_bytes(int64_t N, int64_t H, int64_t L, 
     if (N < 0 || H < 0 || L < 0 || E < 0 || M < 0) return fail(FTC_ERR_INVALID, "negative size");
     if (dtype != FTC_F32 && dtype != FTC_BF16) return fail(FTC_ERR_INVALID, "unknown dtype");
     if (N * H * L == 0 || M == 0 || E == 0) return 0;
-    if (E > kGenericMaxDim || M > kGenericMaxDim)
-        return fail(FTC_ERR_UNSUPPORTED, "E and M must be at most %d", kGenericMaxDim);
+    if ((E > kGenericMaxDim || M > kGenericMaxDim) && dtype != FTC_F32)
+        return fail(FTC_ERR_UNSUPPORTED, "rows of more than %d values must be fp32", kGenericMaxDim);
     return scan_workspace_bytes(N, H, L, E, M, true, dtype == FTC_BF16);
 }
 
@@ -793,8 +892,8 @@ int64_t ftc_causal_dot_backward_workspace_bytes(int64_t N, int64_t H, int64_t L,
     if (N < 0 || H < 0 || L < 0 || E < 0 || M < 0) return fail(FTC_ERR_INVALID, "negative size");
     if (dtype != FTC_F32 && dtype != FTC_BF16) return fail(FTC_ERR_INVALID, "unknown dtype");
     if (N * H * L == 0 || M == 0 || E == 0) return 0;
-    if (E > kGenericMaxDim || M > kGenericMaxDim)
-        return fail(FTC_ERR_UNSUPPORTED, "E and M must be at most %d", kGenericMaxDim);
+    if ((E > kGenericMaxDim || M > kGenericMaxDim) && dtype != FTC_F32)
+        return fail(FTC_ERR_UNSUPPORTED, "rows of more than %d values must be fp32", kGenericMaxDim);
     const bool bf16 = dtype == FTC_BF16;
     int64_t need = std::max(scan_workspace_bytes(N, H, L, E, M, true, bf16),
                             scan_workspace_bytes(N, H, L, M, E, true, bf16));

@@ -122,7 +122,7 @@ def plan(shape_q, shape_v, dtype=FTC_F32, backward=False, strides=None):
         return d
     st = strides or (None, None, None)
     q, k, v = dense(shape_q, st[0]), dense(shape_q, st[1]), dense(shape_v, st[2])
-    buf = ctypes.create_string_buffer(4096)
+    buf = ctypes.create_string_buffer(16384)
     rc = load().ftc_causal_dot_plan(ctypes.byref(q), ctypes.byref(k), ctypes.byref(v),
                                     1 if backward else 0, buf, len(buf))
     check(rc, "ftc_causal_dot_plan")

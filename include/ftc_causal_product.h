@@ -118,7 +118,10 @@ int64_t ftc_causal_dot_product_workspace_bytes(int64_t N, int64_t H, int64_t L, 
  * product[n,h,l,:] = sum_{j<=l} (queries[n,h,l,:] . keys[n,h,j,:]) values[n,h,j,:]
  * Replaces causal_dot_product(queries, keys, values, product)
  * (causal_product_cpu.cpp:82-124, causal_product_cuda.cu:1273-1285).
- * queries, keys: (N,H,L,E); values, product: (N,H,L,M).
+ * queries, keys: (N,H,L,E); values, product: (N,H,L,M).  Any E and M for fp32 tensors, like
+ * the reference's fallback kernels (causal_product_cuda.cu:1243-1269): beyond 512 the call
+ * runs piece by piece of the columns and needs the workspace of the query above; bf16
+ * tensors: E, M <= 512 (FTC_ERR_UNSUPPORTED beyond).
  */
 int ftc_causal_dot_product(const ftc_tensor4 *queries, const ftc_tensor4 *keys,
                            const ftc_tensor4 *values, const ftc_tensor4 *product,

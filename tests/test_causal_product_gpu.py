@@ -95,6 +95,50 @@ def test_reference_gpu_protocol(cp, trial):
         assert torch.allclose(got, ref, rtol=1e-4, atol=1e-5)
 
 
+WIDE_SHAPES = {
+    # name: (N, H, L, E, M, seed) -- rows of more than 512 values (the reference's fallback kernels
+    # have no limit, causal_product_cuda.cu:1243-1269, 1404-1433): column slices and row parts
+    "e600_m520": (1, 2, 300, 600, 520, 81),
+    "e513_m33": (2, 2, 100, 513, 33, 82),       # a last part of odd width, rows added one by one
+    "e1100_m40": (1, 1, 64, 1100, 40, 83),      # three parts of the state's rows
+    "e64_m1030": (1, 2, 256, 64, 1030, 84),     # three column slices forward, three row parts backward
+}
+
+
+@pytest.mark.parametrize("name", sorted(WIDE_SHAPES))
+def test_rows_of_more_than_512_values(cp, name):
+    """The reference's own bar (relative error below 1e-5 of the largest value, allclose with
+    1e-4 / 1e-5, tests/causal_product/test_causal_product_gpu.py:42-84) on positive uniform
+    draws, as in the reference's test."""
+    N, H, L, E, M, seed = WIDE_SHAPES[name]
+    print("wide rows", name, (N, H, L, E, M), flush=True)
+    Q, K, V, G = oracle.make_inputs(N, H, L, E, M, seed=seed, positive_uniform=True)
+    out = hip_forward(cp, Q, K, V)
+    want = oracle.forward(Q, K, V)
+    assert max_relative_error(want, out) < 1e-5
+    assert torch.allclose(out, want, rtol=1e-4, atol=1e-5)
+    grads = hip_backward(cp, Q, K, V, G)
+    for got, ref in zip(grads, oracle.backward(Q, K, V, G)):
+        assert max_relative_error(ref, got) < 1e-5
+        assert torch.allclose(got, ref, rtol=1e-4, atol=1e-5)
+
+
+def test_wide_rows_with_states_handed_in_and_out(cp):
+    """The stateful forward over rows of 600 and 520 values: two pieces against the whole, and
+    the state against the sum of outer products in float64."""
+    N, H, L, E, M = 1, 2, 200, 600, 520
+    Q, K, V, _ = oracle.make_inputs(N, H, L, E, M, seed=85, positive_uniform=True)
+    q, k, v = Q.cuda(), K.cuda(), V.cuda()
+    cut = 120
+    first, state = cp.causal_dot_product_with_state(q[:, :, :cut], k[:, :, :cut], v[:, :, :cut])
+    second, last = cp.causal_dot_product_with_state(q[:, :, cut:], k[:, :, cut:], v[:, :, cut:], state)
+    got = torch.cat([first, second], dim=2).cpu()
+    want = oracle.forward(Q, K, V)
+    assert max_relative_error(want, got) < 1e-5
+    want_state = torch.einsum("nhle,nhlm->nhem", K.double(), V.double())
+    assert scale_error(last.cpu(), want_state) <= 2e-6
+
+
 CONFIG_SHAPES = {
     # BASELINE configs 1 and 2 at full size
     "cfg1": (2, 4, 512, 64, 64, 1),
@@ -976,8 +1020,8 @@ def test_errors_and_empty_inputs(cp):
     with pytest.raises(RuntimeError):
         cp.causal_dot_product_hip(Q, Q, V, out.double())            # product must be fp32
     with pytest.raises(RuntimeError):
-        big = torch.rand(1, 1, 4, 600, device="cuda")
-        cp.causal_dot_product_hip(big, big, V[:, :1, :4], out[:, :1, :4])  # E > 512
+        big = torch.rand(1, 1, 8, 600, device="cuda").bfloat16()               # E > 512 in bf16
+        cp.causal_dot_product_hip(big, big, V[:, :1].bfloat16(), out[:, :1])
     # zero-length sequence and empty batch are no-ops
     e = torch.empty(0, 2, 8, 4, device="cuda")
     cp.causal_dot_product_hip(e, e, torch.empty(0, 2, 8, 6, device="cuda"),

@@ -215,3 +215,24 @@ def test_workspace_queries_cover_every_plan(dtype):
                     if query:
                         worst = max(worst, need / query)
     assert worst > 0.5   # (the queries are not wildly generous either)
+
+
+def test_rows_of_more_than_512_values_are_cut_into_pieces():
+    """fp32 rows wider than 512: column slices of v and out, row parts of a and b whose results
+    are added; every piece is planned like a scan of its own and the queries cover the lot."""
+    lib = _native.load()
+    fwd = lines((1, 2, 300, 600), (1, 2, 300, 520))
+    # two row parts of 300 for each of two column slices of 288 and 232
+    assert sum("state 128 x 288" in l for l in fwd) == 4 and sum("state 44 x 232" in l for l in fwd) == 2
+    assert sum(l.startswith("add_rows_kernel: rows 300 ..") for l in fwd) == 2
+    for (N, H, L, E, M) in [(1, 2, 300, 600, 520), (2, 2, 100, 513, 33), (1, 1, 64, 1100, 40),
+                            (1, 2, 256, 64, 1030), (3, 4, 2048, 700, 900)]:
+        for backward in (False, True):
+            text = lines((N, H, L, E), (N, H, L, M), backward=backward)
+            need = max(int(x) for l in text for x in re.findall(r"workspace (\d+) bytes", l))
+            query = (lib.ftc_causal_dot_backward_workspace_bytes if backward else
+                     lib.ftc_causal_dot_product_workspace_bytes)(N, H, L, E, M, _native.FTC_F32)
+            assert 0 < need <= query, ((N, H, L, E, M), backward, need, query)
+    # bf16 rows of that width: refused, by the queries as by the calls
+    assert lib.ftc_causal_dot_product_workspace_bytes(1, 2, 300, 600, 520, _native.FTC_BF16) < 0
+    assert b"fp32" in lib.ftc_last_error()
