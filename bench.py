@@ -44,9 +44,10 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 matrix, published
 # carries it only while the sources are unchanged, otherwise null.
 MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {
     # workload: (bytes, kernel source hash at the time of the measurement)
-    "cfg2": (137391756, "3e8d53cbcaa977a7"),
-    "cfg3": (3137663994, "3e8d53cbcaa977a7"),
-    "wide": (1877406822, "3e8d53cbcaa977a7"),
+    "cfg2": (137195143, "e4f7800f471c5d94"),
+    "cfg3": (3140424873, "e4f7800f471c5d94"),
+    "cfg5": (5516251577, "e4f7800f471c5d94"),
+    "wide": (1877445109, "e4f7800f471c5d94"),
 }
 
 WORKLOADS = {
