@@ -54,7 +54,7 @@ int tp_kernel_segments(int64_t units, int64_t L, bool wide, bool others) {
     // One workgroup per CU at a time.  A workgroup that takes a whole chain reads every row
     // once; with fewer chains than CUs a chain is cut into up to four segments whose
     // workgroups each rebuild the state before their segment by themselves (a state-only
-    // chunk costs about a third of a full one), as long as that fills at least half the GPU.
+    // chunk costs a bit more than half of a full one), as long as that fills at least half the GPU.
     const int64_t total_chunks = (L + kChunk - 1) / kChunk;
     int nseg = (int)std::max<int64_t>(1, std::min<int64_t>(std::min<int64_t>(4, 256 / units), total_chunks));
     if (tuning().tp_segs >= 0) nseg = std::max(1, std::min(tuning().tp_segs, 16));  // tuning aid
@@ -79,14 +79,15 @@ int tp_kernel_segments(int64_t units, int64_t L, bool wide, bool others) {
 
 // Where to cut a chain of `chunks` chunks into (at most) `nseg` segments for the
 // chain-parallel kernel.  The workgroup of a segment first rebuilds the state before its
-// segment from the chunks in front of it (measured: 0.35 to 0.45 of the time of a chunk that
-// also produces rows), so later segments are made shorter until all workgroups finish together:
+// segment from the chunks in front of it (measured: 0.55 to 0.6 of the time of a chunk that
+// also produces rows -- 0.75 against 1.3 us on the fp16-piece kernel with every workgroup
+// streaming rows), so later segments are made shorter until all workgroups finish together:
 // the starts (multiples of kTpAhead chunks, what the producers request ahead) that minimise the
 // longest workgroup.  Returns the number of segments; start[0 .. n] filled (start[n] = chunks).
 int tp_segment_starts(int64_t chunks, int nseg, int32_t *start) {
     const int groups = (int)((chunks + kTpAhead - 1) / kTpAhead);
     nseg = std::max(1, std::min(std::min(nseg, groups), kMaxTpSegments));
-    double kStateOnly = 0.4;
+    double kStateOnly = 0.6;
     if (tuning().tp_ratio >= 0) kStateOnly = tuning().tp_ratio;  // tuning aid
     // best[s][g]: smallest achievable longest time of segments s .. nseg-1 when segment s
     // starts at group g (dynamic programme from the last segment back)
