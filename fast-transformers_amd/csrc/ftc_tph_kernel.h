@@ -34,12 +34,16 @@
 //    position); after the
 //    workgroup barrier all twelve wavefronts read the slot.  All of them thus know the same
 //    three exponents for every position, and they depend on the rows alone: however a chain
-//    is cut into segments, the results are the same bit for bit.
+//    is cut into segments, the results are the same bit for bit (as long as the state stays
+//    below 2^14 units, s = 0; beyond that the chunk where s rises depends on the cut, and
+//    results agree to the rounding of the state's pieces, 2^-22).
 //  * The state is kept in the units of the scaled rows (2^(e_b + e_v - 8)); when a ceiling
 //    rises it is rescaled (exactly).  It is cut into pieces with one more power of two,
-//    2^-s, chosen so that no element exceeds 2^15: s rises when the largest element of the
-//    state before the previous chunk exceeds 2^(14 + s) (a chunk adds at most 2^13).  The
-//    chunk product needs no scale: |Pt| <= 64 * 16 * 16 = 2^14.
+//    2^-s, chosen so that no element leaves fp16's range: every third chunk s rises if an
+//    element of the state exceeds 2^(14 + s) (a chunk adds at most 2^13: three more chunks
+//    stay below 2^14 + 3 x 2^13 < 65504).  As long as s = 0, the rule, the cut is plain
+//    (one packed conversion per pair for the high pieces).  The chunk product needs no scale:
+//    |Pt| <= 64 * 16 * 16 = 2^14.
 //  * Ot = (S^T a^T) 2^s + v^T Pt is summed in the units of the chunk and leaves the
 //    accumulator through one v_ldexp_f32 per value.
 #pragma once
@@ -111,29 +115,47 @@ constexpr uint32_t kExpFloor = 28, kExpCeil = 248;
 __device__ __forceinline__ float pow2_field(int field) {  // 2^(field - 127), field clamped
     return __uint_as_float((uint32_t)max(1, min(254, field)) << 23);
 }
-// the ceiling exponent of a non-negative float (inf and NaN: the largest)
-__device__ __forceinline__ uint32_t ceiling_of(float m) {
-    const uint32_t be = (__float_as_uint(m) >> 23) & 0xffu;  // m < 2^(be - 126)
-    return max(kExpFloor, min(kExpCeil, be + 2u));
+// wave-uniform integer maxima and minima on the scalar unit (written out: the compiler would
+// merge them into three-operand vector instructions)
+__device__ __forceinline__ uint32_t scalar_max(uint32_t a, uint32_t b) {
+    uint32_t r;
+    asm("s_max_u32 %0, %1, %2" : "=s"(r) : "s"(a), "s"(b) : "scc");
+    return r;
+}
+__device__ __forceinline__ uint32_t scalar_min(uint32_t a, uint32_t b) {
+    uint32_t r;
+    asm("s_min_u32 %0, %1, %2" : "=s"(r) : "s"(a), "s"(b) : "scc");
+    return r;
+}
+// the ceiling exponent of a non-negative float, given as its bits in a scalar register (inf and
+// NaN: the largest)
+__device__ __forceinline__ uint32_t ceiling_of(uint32_t bits) {
+    const uint32_t be = (bits >> 23) & 0xffu;  // the value is below 2^(be - 126)
+    return scalar_max(kExpFloor, scalar_min(kExpCeil, be + 2u));
 }
 // The largest of a non-negative float over the wavefront (wave-uniform): four steps inside
 // the rows of 16 lanes on the data-parallel path, then one lane of every row.
+// (non-negative floats order like their bit patterns: an integer maximum needs no
+// canonicalising copy of the lane it reads across, and folds into one instruction)
 template <int CTRL>
-__device__ __forceinline__ float max_with_dpp(float x) {
-    return fmaxf(x, __uint_as_float((uint32_t)__builtin_amdgcn_update_dpp(
-                        0, (int)__float_as_uint(x), CTRL, 0xf, 0xf, true)));
+__device__ __forceinline__ uint32_t max_with_dpp(uint32_t x) {
+    return max(x, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, CTRL, 0xf, 0xf, true));
 }
-__device__ __forceinline__ float wave_max(float m) {
-    m = max_with_dpp<0xb1>(m);   // quad_perm [1, 0, 3, 2]
-    m = max_with_dpp<0x4e>(m);   // quad_perm [2, 3, 0, 1]
-    m = max_with_dpp<0x141>(m);  // row_half_mirror
-    m = max_with_dpp<0x140>(m);  // row_mirror
-    const uint32_t b = __float_as_uint(m);
-    const uint32_t r = max(max((uint32_t)__builtin_amdgcn_readlane((int)b, 0),
-                               (uint32_t)__builtin_amdgcn_readlane((int)b, 16)),
-                           max((uint32_t)__builtin_amdgcn_readlane((int)b, 32),
-                               (uint32_t)__builtin_amdgcn_readlane((int)b, 48)));
-    return __uint_as_float(r);  // (non-negative floats order like their bit patterns)
+// ... over each row of 16 lanes (every lane of a row gets the row's maximum)
+__device__ __forceinline__ uint32_t row_max_bits(float m) {
+    uint32_t b = __float_as_uint(m);
+    b = max_with_dpp<0xb1>(b);   // quad_perm [1, 0, 3, 2]
+    b = max_with_dpp<0x4e>(b);   // quad_perm [2, 3, 0, 1]
+    b = max_with_dpp<0x141>(b);  // row_half_mirror
+    b = max_with_dpp<0x140>(b);  // row_mirror
+    return b;
+}
+__device__ __forceinline__ uint32_t wave_max(float m) {  // (the bits of the largest value)
+    const uint32_t b = row_max_bits(m);
+    return scalar_max(scalar_max((uint32_t)__builtin_amdgcn_readlane((int)b, 0),
+                                 (uint32_t)__builtin_amdgcn_readlane((int)b, 16)),
+                      scalar_max((uint32_t)__builtin_amdgcn_readlane((int)b, 32),
+                                 (uint32_t)__builtin_amdgcn_readlane((int)b, 48)));
 }
 
 // The running ceilings of a, b and v as one wavefront knows them (wave-uniform).
@@ -159,8 +181,9 @@ __device__ __forceinline__ void read_slot(const lds_u32_t *slots, int k, Ceiling
     c.Ev = max(c.Ev, (uint32_t)__builtin_amdgcn_readfirstlane(s.z));
 }
 // Lane maxima of the rows of position `pos` (slot k) against the ceilings of the position
-// before it.  a: every wavefront that holds rows enters the ceiling of its own rows.  b, v:
-// whoever finds a value at or above the running ceiling raises the slot.
+// before it.  a: every row of 16 lanes enters the ceiling of its own values (one lane per row:
+// four atomics on one word per wavefront, no trip through scalar registers).  b, v: whoever
+// finds a value at or above the running ceiling raises the slot.
 __device__ __forceinline__ void raise_slot(lds_u32_t *slots, int k, int pos, const Ceilings &c,
                                            float ma, float mb, float mv, int lane) {
     lds_u32_t *const s = slots + 4 * k;
@@ -346,6 +369,7 @@ __global__ __launch_bounds__(768, 3) void scan_tph_kernel(uint32_t *__restrict__
         auto fetch = [&](Raw &r, int v) {  // v: position of the walk
             const int row0 = v < nwalk ? chunk_row0(walk_chunk(v)) : -2 * kChunk;
             const int row0_x = v >= n1 ? row0 : -2 * kChunk;
+            // (the sums wrap: a chunk that starts before the first row has its later rows in place)
             r.a = load_quad(a_rs, ab_in ? a_goff + (uint32_t)row0_x * a_slb : kNoRow, a_bf);
             r.b = load_quad(b_rs, ab_in ? b_goff + (uint32_t)row0 * b_slb : kNoRow, b_bf);
             r.v = load_quad(v_rs, v_in ? v_goff + (uint32_t)row0 * v_slb : kNoRow, v_bf);
@@ -617,18 +641,28 @@ __global__ __launch_bounds__(768, 3) void scan_tph_kernel(uint32_t *__restrict__
         while (s < 100 && __builtin_amdgcn_ballot_w64(m > pow2_field(127 + 14 + s)) != 0) s++;
     }
     float kappa = pow2_field(127 + dU - s);  // scale of the cut of S
+    bool plain_cut = dU - s == 0;            // ... which is one as a rule: a cheaper cut
     int s_cut = s;                            // ... and the s that went into it
     float mS = 0.f;                           // largest |S| seen while cutting
     Frag sf[2][2];
     // tile 2 ks + u of S_w -> words 2 u, 2 u + 1 of the fragments of k-step ks
-    auto cut_s = [&](int ks, int u) {
+    // (`track`: also note the largest magnitude.  One state in three is looked at, the one
+    // cut for the chunks in LDS buffer 0: s then rises when an element exceeds 2^(14 + s)
+    // units, three more chunks add at most 3 x 2^13, and 2^14 + 3 x 2^13 is below what fp16
+    // holds.)
+    auto cut_s = [&](int ks, int u, bool track) {
         const f32x4 x = S[2 * ks + u];
-        mS = fmaxf(fmaxf(fmaxf(fabsf(x[0]), fabsf(x[1])), fmaxf(fabsf(x[2]), fabsf(x[3]))), mS);
-        cut_quad_f16(x[0], x[1], x[2], x[3], kappa, sf[ks][0].w[2 * u], sf[ks][0].w[2 * u + 1],
-                     sf[ks][1].w[2 * u], sf[ks][1].w[2 * u + 1]);
+        if (track)
+            mS = fmaxf(fmaxf(fmaxf(fabsf(x[0]), fabsf(x[1])), fmaxf(fabsf(x[2]), fabsf(x[3]))), mS);
+        if (plain_cut)
+            cut_quad_f16_unscaled(x[0], x[1], x[2], x[3], sf[ks][0].w[2 * u], sf[ks][0].w[2 * u + 1],
+                                  sf[ks][1].w[2 * u], sf[ks][1].w[2 * u + 1]);
+        else
+            cut_quad_f16(x[0], x[1], x[2], x[3], kappa, sf[ks][0].w[2 * u], sf[ks][0].w[2 * u + 1],
+                         sf[ks][1].w[2 * u], sf[ks][1].w[2 * u + 1]);
     };
-    cut_s(0, 0);
-    cut_s(0, 1);
+    cut_s(0, 0, true);
+    cut_s(0, 1, true);
 
     // Ot_w of the chunk before in the units of that chunk (exponent Xo), and where its rows
     // go (before the first chunk: nowhere)
@@ -662,7 +696,7 @@ __global__ __launch_bounds__(768, 3) void scan_tph_kernel(uint32_t *__restrict__
         const lds_char *pn = unit_pc + BN * kBufBytes;
         lds_char *const ptc = pt_pc + B * (2 * kTileP);
         Frag pf[2][2];
-        f32x4 P = zero;
+        f32x4 P;  // (cleared by the first matrix instruction of its sum)
         if (c == c0 + 4) FTC_STAMP(0);
         __builtin_amdgcn_sched_barrier(0);
         // phase 1: (1) the quadrant in turn with (2b) Ot_w = S_w^T a^T for rows 0 .. 31 of
@@ -673,9 +707,9 @@ __global__ __launch_bounds__(768, 3) void scan_tph_kernel(uint32_t *__restrict__
             const int m = i % 3, ks = i / 3, x = i % 2, mo = i / 2;
             if (i == 0) store_rows(0);
             if (i == 1) store_rows(1);
-            if (ks < KS) P = mfma16h(bfr[ks][kPa[m]], af[0][ks][kPb[m]], P);
+            if (ks < KS) P = mfma16h(bfr[ks][kPa[m]], af[0][ks][kPb[m]], i == 0 ? zero : P);
             O[x] = mfma16h(sf[0][kPa[mo]], af[x][0][kPb[mo]], mo == 0 ? zero : O[x]);
-            if ((i == 1 || i == 3) && KS > 1) cut_s(1, i / 2);
+            if ((i == 1 || i == 3) && KS > 1) cut_s(1, i / 2, B == 0);
             tr_frag_into(bt, vf, pc, i);
             if (i < 4) tr_frag_into(bt, vf, pc, 6 + i);
             __builtin_amdgcn_sched_barrier(0);
@@ -688,8 +722,10 @@ __global__ __launch_bounds__(768, 3) void scan_tph_kernel(uint32_t *__restrict__
             s = max(0, s + dU);
             Ucur -= dU;
         }
-        while (s < 100 && __builtin_amdgcn_ballot_w64(mS > pow2_field(127 + 14 + s)) != 0) s++;
-        mS = 0.f;
+        if (B == 0) {
+            while (s < 100 && __builtin_amdgcn_ballot_w64(mS > pow2_field(127 + 14 + s)) != 0) s++;
+            mS = 0.f;
+        }
         if (c == c0 + 4) FTC_STAMP(2);
         __builtin_amdgcn_sched_barrier(0);
         // phase 2: (2b) for rows 32 .. 63 in turn with (3) S_w += b^T v_w for tiles 0 and 1;
@@ -746,13 +782,14 @@ __global__ __launch_bounds__(768, 3) void scan_tph_kernel(uint32_t *__restrict__
         ce.Ev = max(ce.Ev, (uint32_t)__builtin_amdgcn_readfirstlane(slot_next.z));
         dU = Ucur - ce.state_exp();
         kappa = pow2_field(127 + dU - s);
+        plain_cut = dU - s == 0;
         s_cut = s;
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int i = 0; i < 6; i++) {
             const int x = i % 2, m = i / 2;
             O[x] = mfma16h(vf[kPa[m]], pf[x][kPb[m]], O[x]);
-            if (i == 1 || i == 3) cut_s(0, i / 2);
+            if (i == 1 || i == 3) cut_s(0, i / 2, BN == 0);
             __builtin_amdgcn_sched_barrier(0);
         }
         o_off = (uint32_t)chunk_row0(c) * o_slb;
