@@ -44,10 +44,10 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 matrix, published
 # carries it only while the sources are unchanged, otherwise null.
 MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {
     # workload: (bytes, kernel source hash at the time of the measurement)
-    "cfg2": (138942178, "26b31c124e45a728"),
-    "cfg3": (3135513417, "26b31c124e45a728"),
-    "cfg5": (5516742527, "26b31c124e45a728"),
-    "wide": (1877401844, "26b31c124e45a728"),
+    "cfg2": (139473943, "a41fe8b16f136f54"),
+    "cfg3": (3143569854, "a41fe8b16f136f54"),
+    "cfg5": (5516330946, "a41fe8b16f136f54"),
+    "wide": (1877412303, "a41fe8b16f136f54"),
 }
 
 WORKLOADS = {
