@@ -44,10 +44,10 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 matrix, published
 # carries it only while the sources are unchanged, otherwise null.
 MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {
     # workload: (bytes, kernel source hash at the time of the measurement)
-    "cfg2": (139473943, "a41fe8b16f136f54"),
-    "cfg3": (3143569854, "a41fe8b16f136f54"),
-    "cfg5": (5516330946, "a41fe8b16f136f54"),
-    "wide": (1877412303, "a41fe8b16f136f54"),
+    "cfg2": (139029571, "c57677d557112d87"),
+    "cfg3": (3142773087, "c57677d557112d87"),
+    "cfg5": (5517273469, "c57677d557112d87"),
+    "wide": (1877080083, "c57677d557112d87"),
 }
 
 WORKLOADS = {

@@ -8,9 +8,10 @@
 //
 // Division of labour, chunking, LDS tiles, swizzles, segments and the exchange of segment
 // sums are those of ftc_tp_kernel.h (one workgroup walks one chain; four consumer wavefronts
-// hold the state as slabs of 16 columns and share the chunk product Pt through LDS; four
-// producer wavefronts fetch rows four chunks ahead and cut them into piece tiles).  What
-// differs is the arithmetic that stands for an fp32 product:
+// hold the state as slabs of 16 columns and share the chunk product Pt through LDS; producer
+// wavefronts -- eight here, one quad of every operand per lane and position -- fetch rows
+// four chunks ahead and cut them into piece tiles).  What differs is the arithmetic that
+// stands for an fp32 product:
 //
 //  * Every fp32 value x is scaled by a power of two and cut into TWO fp16 pieces, both rounded
 //    to nearest: hi = fp16(x s), lo = fp16(x s - hi).  hi + lo carries 22 significand bits of

@@ -207,7 +207,8 @@ int64_t ftc_causal_linear_attention_workspace_bytes(int64_t N, int64_t H, int64_
  * queries, keys: (N,H,L,E) raw projections (before the feature map); values, out:
  * (N,H,L,M); all FTC_F32, any N/H/L strides with 16-byte aligned rows (the module's
  * (N,L,H,X) tensors are passed as permuted views).  key_lengths: N int64 values on the
- * device, or NULL when every key counts.  Forward only.  Sizes: E, M in {32, 64};
+ * device, or NULL when every key counts.  (For training see
+ * ftc_causal_linear_attention_forward and ..._backward below.)  Sizes: E, M in {32, 64};
  * anything else returns FTC_ERR_UNSUPPORTED and the caller composes the result from
  * ftc_causal_dot_product as before.
  */
