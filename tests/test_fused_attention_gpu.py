@@ -379,3 +379,46 @@ def test_non_finite_inputs_propagate_as_in_the_composition(lib):
     assert not bad_fused[0, :40, 0].any() and not bad_fused[0, :200, 1].any()
     ok = ~bad_fused
     assert (y_fused[ok] - y_composed[ok]).abs().max() <= 1e-4 * y_composed[ok].abs().max()
+
+
+def test_forward_and_backward_replay_in_a_graph(lib):
+    """Both entry points only enqueue kernels (fill kernels instead of memsets, nothing
+    allocated), so a forward + backward pair can be captured in a HIP graph.  Every replay,
+    with direct launches on other data in between, reproduces the direct results bit for bit."""
+    from fast_transformers_amd import causal_product as cp
+    N, L, H, E, M = 2, 600, 4, 64, 64
+    nlh = lambda t: t.permute(0, 2, 1, 3)
+    q, k, v = (nlh(t.cuda()) for t in inputs(N, L, H, E, M, seed=71))
+    q2, k2, v2 = (nlh(t.cuda()) for t in inputs(N, L, H, E, M, seed=72))
+    g = nlh(torch.randn(N, L, H, M, generator=torch.Generator().manual_seed(73)).cuda())
+    lengths = torch.tensor([600, 431]).cuda()
+    out = nlh(torch.empty(N, L, H, M, device="cuda"))
+    den = torch.empty(N, H, L, device="cuda")
+    grads = [nlh(torch.empty(N, L, H, X, device="cuda")) for X in (E, E, M)]
+
+    def pair():
+        cp.causal_linear_attention_hip(q, k, v, lengths, 1e-6, out, den)
+        cp.causal_linear_attention_backward_hip(q, k, v, lengths, out, den, g, *grads)
+
+    pair()
+    torch.cuda.synchronize()
+    want = [t.clone() for t in [out] + grads]
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):  # the wrapper's workspace for this stream exists before capture
+        pair()
+    side.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        pair()
+    other = nlh(torch.empty(N, L, H, M, device="cuda"))
+    for replay in range(4):
+        for t in [out, den] + grads:
+            t.fill_(float("nan"))
+        cp.causal_linear_attention_hip(q2, k2, v2, None, 1e-6, other)   # the program's own work
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for name, got, ref in zip(("out", "dq", "dk", "dv"), [out] + grads, want):
+            assert torch.equal(got, ref), (replay, name)
+    assert torch.isfinite(other).all()
