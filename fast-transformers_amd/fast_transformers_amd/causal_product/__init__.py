@@ -132,7 +132,10 @@ def _watch(key, ws):
 
 def _after_call(ws=None, stream=None):
     if os.environ.get("FTC_CHECK", "0") not in ("", "0"):
-        check_workspaces()
+        # the check synchronises, which a capturing stream does not allow: a captured call is
+        # checked by the first eager call after the replays, or by check_workspaces()
+        if not torch.cuda.is_current_stream_capturing():
+            check_workspaces()
         return
     if ws is None:
         return

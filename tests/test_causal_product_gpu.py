@@ -744,11 +744,12 @@ def test_zz_no_wavefront_gave_up_waiting(cp):
     assert all(w == 0 for w in words.values()), words
 
 
-def test_dirty_control_block_is_reported_and_healed(cp):
+def test_dirty_control_block_is_reported_and_healed(cp, monkeypatch):
     """A control block that is not zero when a call starts (here: a ticket counter set from
     the host) makes the wavefronts of that chain stop early; every kernel still ends
     normally.  check_workspaces() reports it and resets the workspace, after which calls work
     again."""
+    monkeypatch.delenv("FTC_CHECK", raising=False)   # the steps below say when it is on
     N, H, L, E, M = 2, 2, 1500, 64, 64
     Q, K, V, _ = oracle.make_inputs(N, H, L, E, M, seed=77)
     want = oracle.forward(Q, K, V)
@@ -769,14 +770,12 @@ def test_dirty_control_block_is_reported_and_healed(cp):
     # the debugging mode reads the error word after every call
     ws.view(torch.int32)[64 + max_waves] = 1000
     torch.cuda.synchronize()
-    os.environ["FTC_CHECK"] = "1"
-    try:
-        with pytest.raises(RuntimeError, match="cut short"):
-            hip_forward(cp, Q, K, V)
-        out = hip_forward(cp, Q, K, V)         # reset by the check: works again
-        assert scale_error(out, want) <= 1e-4
-    finally:
-        del os.environ["FTC_CHECK"]
+    monkeypatch.setenv("FTC_CHECK", "1")
+    with pytest.raises(RuntimeError, match="cut short"):
+        hip_forward(cp, Q, K, V)
+    out = hip_forward(cp, Q, K, V)         # reset by the check: works again
+    assert scale_error(out, want) <= 1e-4
+    monkeypatch.delenv("FTC_CHECK")
     # without the debugging mode the wrapper watches the error word without waiting for the
     # GPU: a probe left behind one call is read by a later one (within a few calls and 10 ms)
     ws.view(torch.int32)[64 + max_waves] = 1000
