@@ -16,11 +16,12 @@
 //   dq = dQf phi'(q) ;  dk_j = dKf_j phi'(k_j) [j < key_len] ;  phi'(x) = x > 0 ? 1 : exp(x)
 //
 // The first sums are the three scans of the plain backward on (Qf, Kf, v, gz).  The second
-// ones are prefix sums along the chain of rows weighted by a scalar.  Both kernels here give a
-// workgroup one segment of 128 positions of one chain: attn_bwd_prep_kernel also leaves the
-// segment's totals, and attn_bwd_finish_kernel, one more pass over dq and dk, adds the prefix
-// sums (totals of the other segments, then of the other threads' runs, then its own run) and
-// multiplies by phi'.  Qf and Kf are recomputed there from q and k, which phi' needs anyway.
+// ones are prefix sums along the chain of rows weighted by a scalar.  The two large kernels here
+// give a workgroup one segment of 128 positions of one chain: attn_bwd_prep_kernel also leaves
+// the segment's totals, attn_bwd_totals_kernel turns those into the sums over the segments
+// before and after each one, and attn_bwd_finish_kernel, one more pass over dq and dk, adds the
+// prefix sums (those of the other segments, then of the other threads' runs, then its own run)
+// and multiplies by phi'.  Qf and Kf are recomputed there from q and k, which phi' needs anyway.
 #include "ftc_common.h"
 
 namespace ftc {
@@ -118,6 +119,32 @@ __global__ __launch_bounds__(256) void attn_bwd_prep_kernel(
     }
 }
 
+// The segments' totals -> what the segments before (Kf) and after (dd Qf) each one add up to,
+// in place, each sum in the fixed order that a walk along the chain would take (ascending for
+// the first kind, descending for the second).  One workgroup per chain, one lane per kind and
+// column; eight totals are in flight at a time.
+__global__ __launch_bounds__(128) void attn_bwd_totals_kernel(float *__restrict__ sums, int E, int nseg) {
+    const int which = threadIdx.x >> 6, col = threadIdx.x & 63;
+    if (col >= E) return;
+    float *s = sums + ((int64_t)blockIdx.x * nseg * 2 + which) * E + col;
+    const int64_t step = 2 * (int64_t)E;
+    float run = 0.f;
+    for (int i0 = 0; i0 < nseg; i0 += 8) {
+        float x[8];
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const int i = which == 0 ? i0 + j : nseg - 1 - (i0 + j);
+            x[j] = i0 + j < nseg ? s[i * step] : 0.f;
+        }
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const int i = which == 0 ? i0 + j : nseg - 1 - (i0 + j);
+            if (i0 + j < nseg) s[i * step] = run;
+            run += x[j];
+        }
+    }
+}
+
 // One workgroup of 32 groups per (chain, segment); 16 lanes per position as above, and group r takes the
 // run of kRun consecutive positions seg kSegment + r kRun ...  dq and dk hold the scans'
 // results on entry:
@@ -161,11 +188,9 @@ __global__ __launch_bounds__(16 * kGroups) void attn_bwd_finish_kernel(
     for (int i = kRun - 2; i >= 0; i--) qd[i] = qd[i] + qd[i + 1];
     total[0][r][c] = kf[kRun - 1];
     total[1][r][c] = qd[0];
-    // what the segments before (for dq) and after (for dk) this one add, in a fixed order
-    float4 ck = zero4(), cq = zero4();
-    const float *s = sums + (chain * nseg * 2) * E + ce;
-    for (int i = 0; i < seg; i++) ck = ck + *(const float4 *)(s + (int64_t)i * 2 * E);
-    for (int i = nseg - 1; i > seg; i--) cq = cq + *(const float4 *)(s + (int64_t)i * 2 * E + E);
+    // what the segments before (for dq) and after (for dk) this one add (attn_bwd_totals_kernel)
+    const float *s = sums + ((chain * nseg + seg) * 2) * E + ce;
+    float4 ck = *(const float4 *)s, cq = *(const float4 *)(s + E);
     __syncthreads();
     // and the runs before and after this one in the segment
     for (int i = 0; i < r; i++) ck = ck + total[0][i][c];
@@ -215,13 +240,14 @@ void launch_attention_backward_prep(const Operand &q, const Operand &k, const Op
 }
 
 void launch_attention_backward_finish(const Operand &q, const Operand &k, const int64_t *key_len,
-                                      const float *dd, const float *sums, int64_t N, int64_t H,
+                                      const float *dd, float *sums, int64_t N, int64_t H,
                                       int64_t L, int E, const OperandOut &dq, const OperandOut &dk,
                                       hipStream_t stream) {
     const int nseg = (int)attention_backward_segments(L);
+    hipLaunchKernelGGL(attn_bwd_totals_kernel, dim3((unsigned)(N * H)), dim3(128), 0, stream, sums, E, nseg);
     hipLaunchKernelGGL(attn_bwd_finish_kernel, dim3((unsigned)(N * H * nseg)), dim3(16 * kGroups), 0, stream,
-                       rows_of(q), rows_of(k), key_len, dd, sums, (int)H, (int)L, E, nseg, rows_of(dq),
-                       rows_of(dk));
+                       rows_of(q), rows_of(k), key_len, dd, (const float *)sums, (int)H, (int)L, E, nseg,
+                       rows_of(dq), rows_of(dk));
 }
 
 }  // namespace ftc

@@ -173,7 +173,7 @@ void launch_attention_backward_prep(const Operand &q, const Operand &k, const Op
                                     float *Kf, float *gz, float *dd, float *sums,
                                     hipStream_t stream);
 void launch_attention_backward_finish(const Operand &q, const Operand &k, const int64_t *key_len,
-                                      const float *dd, const float *sums, int64_t N, int64_t H,
+                                      const float *dd, float *sums, int64_t N, int64_t H,
                                       int64_t L, int E, const OperandOut &dq, const OperandOut &dk,
                                       hipStream_t stream);
 
