@@ -44,10 +44,10 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 matrix, published
 # carries it only while the sources are unchanged, otherwise null.
 MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {
     # workload: (bytes, kernel source hash at the time of the measurement)
-    "cfg2": (139529078, "7180d170abc13a66"),
-    "cfg3": (3139695269, "7180d170abc13a66"),
-    "cfg5": (5517084383, "7180d170abc13a66"),
-    "wide": (1877447160, "7180d170abc13a66"),
+    "cfg2": (139428186, "476fbf2993f72fc7"),
+    "cfg3": (3139837732, "476fbf2993f72fc7"),
+    "cfg5": (4971962191, "476fbf2993f72fc7"),
+    "wide": (1877415730, "476fbf2993f72fc7"),
 }
 
 WORKLOADS = {

@@ -46,11 +46,11 @@ bool mfma_scan_supported_widths(int64_t D, int64_t F) {
 // other than 64 x 64, for which the kernels that split L are half as fast as for 64 x 64;
 // `others`: one of those kernels takes this shape (else the choice is the VALU kernel).
 // Returns the number of segments per chain (0: another kernel takes the launch).
-int tp_kernel_segments(int64_t units, int64_t L, bool wide, bool others) {
+int tp_kernel_segments(int64_t units, int64_t L, bool wide, bool others, bool long_chains = false) {
     // a chain is walked by one workgroup from end to end: beyond 256 chunks the split of L
     // of the other kernels is faster, and its segment sums also keep the rounding of a long
-    // running state in check
-    if (L > 256 * kChunk) return 0;
+    // running state in check (`long_chains`: the caller knows better, see tp_plan_compute)
+    if (L > (long_chains ? 1024 : 256) * kChunk) return 0;
     // One workgroup per CU at a time.  A workgroup that takes a whole chain reads every row
     // once; with fewer chains than CUs a chain is cut into up to four segments whose
     // workgroups each rebuild the state before their segment by themselves (a state-only
@@ -161,19 +161,25 @@ int tp_exchange_segments(int64_t units, int64_t L, bool wide, int *nseg) {
 // cut into *nseg segments that need no exchange; both 0: another kernel takes the launch.
 // `mixed`: rows with bf16 among them (the fp16-piece form of the kernel takes those; the plans
 // are those of fp32 rows where the kernel is used at all).
+// `mixed`: kMixedRows: rows with bf16 among them; kMixedGradValues: a single scan of bf16 a and b
+// whose values are fp32 (the dV scan of a bf16 backward)
+constexpr int kMixedRows = 1, kMixedGradValues = 2;
 void tp_plan_compute(int64_t D, int64_t F, int64_t chains, int nscans, int64_t L, int *nseg,
-                     int *seg_chunks, bool forced, bool mixed) {
+                     int *seg_chunks, bool forced, int mixed) {
     *nseg = *seg_chunks = 0;
     if (!tp_widths(D, F, forced)) return;
     const bool wide = D != 64 || F != 64 || forced;
     const bool others = !forced && mfma_scan_supported_widths(D, F);
     const int64_t units = chains * nscans * tp_fblocks(F);
     // A single scan over bf16 rows: the kernels that split L multiply such rows as they are,
-    // one matrix instruction per product, and win until there are workgroups for every CU
-    // (forward, 64 x 64, N*H = 80: 33 against 38 us at L=1000, 69 against 110 at L=4096;
-    // N*H = 256: 56 against 47 at L=1000).  The three scans of a backward call are faster
+    // one matrix instruction per product, and win while this kernel has workgroups for fewer
+    // than half of the CUs (forward, 64 x 64, L=1000, N*H = 80: 32 against 36 us, 96: 33
+    // against 36, 112: 38 against 36, 128: 42 against 37, 192: 53 against 42) or would need
+    // an exchange (N*H = 128, L=4096: 114 against 132 us; L=8192: 208 against 241; without one,
+    // N*H = 192, L=4096: 160 against 140).  The three scans of a backward call are faster
     // here for up to 128 chains (L=1000, N*H = 80: 50 against 101 us).
-    if (mixed && nscans == 1 && others && units < 256) return;
+    const bool lone_mixed = mixed && nscans == 1 && others;
+    if (lone_mixed && units < 112) return;
     // Shapes of the other kernels with 32 rows or columns (a workgroup here has half of its
     // matrix work or half of its consumers to spare for them): measured at N=8, H=16, L=4096,
     // forward + backward, 32 x 128 0.62 against 0.80 ms and 128 x 32 0.76 against 0.78 on whole
@@ -188,7 +194,18 @@ void tp_plan_compute(int64_t D, int64_t F, int64_t chains, int nscans, int64_t L
     if (narrow && units > 512) return;
     if (!forced && D <= 64 && F <= 64 && units > 512 && L <= 2 * kChunk) return;
     if (!narrow) *seg_chunks = tp_exchange_segments(units, L, wide, nseg);
-    if (*seg_chunks == 0) *nseg = tp_kernel_segments(units, L, wide, others);
+    if (lone_mixed && units < 256 && *seg_chunks > 0) {
+        *nseg = *seg_chunks = 0;
+        return;
+    }
+    // The dV scan of a bf16 backward with a state of at most 32 rows and a workgroup for every
+    // CU is walked whole however long the chain: what the kernels that split L read twice there
+    // is the fp32 gradient, the widest operand by far (N=4, H=32, L=16384, 32 x 128: 0.485
+    // against 0.629 ms; the forward of the same shape, whose wide operand is the fp32 result
+    // that either kernel writes once, loses: 0.656 against 0.495).  bf16 results make the
+    // rounding of a long running fp32 state a non-issue.
+    const bool long_chains = mixed == kMixedGradValues && D <= 32 && units == 256;
+    if (*seg_chunks == 0) *nseg = tp_kernel_segments(units, L, wide, others, long_chains);
 }
 
 // workspace of the exchange: control block, then two state slots (own sum, group total) of
@@ -278,9 +295,9 @@ struct TpPlan {
     int nseg, seg_chunks;
 };
 void tp_plan(int64_t D, int64_t F, int64_t chains, int nscans, int64_t L, int *nseg, int *seg_chunks,
-             bool forced = false, bool mixed = false) {
+             bool forced = false, int mixed = 0) {
     static thread_local PlanMemo<TpPlan> memo;
-    const int64_t key[8] = {D, F, chains, nscans, L, forced ? 1 : 0, mixed ? 1 : 0, 0};
+    const int64_t key[8] = {D, F, chains, nscans, L, forced ? 1 : 0, mixed, 0};
     const TpPlan pl = memo.get(key, [&]() {
         TpPlan p;
         tp_plan_compute(D, F, chains, nscans, L, &p.nseg, &p.seg_chunks, forced, mixed);
@@ -407,11 +424,11 @@ bool mfma_tp_takes(const ScanDesc *scans, int nscans, int64_t N, int64_t H, int6
     const int D = scans[0].a.width, F = scans[0].v.width;
     if (nscans < 1 || nscans > kMaxScans || !tp_widths(D, F, forced)) return false;
     int64_t widest_stride = 0;
-    bool mixed = false;
+    int mixed = nscans == 1 && combo_of(scans[0]) == kBBFB ? kMixedGradValues : 0;
     for (int i = 0; i < nscans; i++) {
         const ScanDesc &sd = scans[i];
         const Combo combo = combo_of(sd);
-        mixed = mixed || combo != kFFFF;
+        if (combo != kFFFF && mixed == 0) mixed = kMixedRows;
         // rows with bf16 among them: the fp16-piece form of the kernel only
         if (combo == kNone || (combo != kFFFF && !tph_takes_rows(D))) return false;
         if (sd.a.width != D || sd.v.width != F) return false;
@@ -456,8 +473,9 @@ int mfma_scan(const ScanDesc *scans, int nscans, int64_t N, int64_t H, int64_t L
     const int64_t fblocks = tp_shape ? tp_fblocks(F) : 1;
     int tpx_nseg = 0, tpx_seg_chunks = 0, tp_nseg = 0;
     if (tp_shape) {
-        bool any_bf16 = false;
-        for (int i = 0; i < nscans; i++) any_bf16 = any_bf16 || combo_of(scans[i]) != kFFFF;
+        int any_bf16 = nscans == 1 && combo == kBBFB ? kMixedGradValues : 0;
+        for (int i = 0; i < nscans; i++)
+            if (combo_of(scans[i]) != kFFFF && any_bf16 == 0) any_bf16 = kMixedRows;
         tp_plan(D, F, chains, nscans, L, &tpx_nseg, &tpx_seg_chunks, forced, any_bf16);
         if (tpx_seg_chunks == 0) tp_nseg = tpx_nseg, tpx_nseg = 0;
     }

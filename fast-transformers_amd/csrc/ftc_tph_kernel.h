@@ -678,12 +678,11 @@ __global__ __launch_bounds__(768, 3) void scan_tph_kernel(uint32_t *__restrict__
         const uint32_t at = o_in ? o_off + o_lane[x] : kNoRow;
         if (!MIX) {
             buffer_store_out(o_rs, at, y0, y1, y2, y3, (float *)nullptr);
-        } else {  // two 8-byte stores whatever the type; the second one of a bf16 quad goes nowhere
-            const u32x2 first = {o_bf ? pack_bf16_rne(y0, y1) : __float_as_uint(y0),
-                                 o_bf ? pack_bf16_rne(y2, y3) : __float_as_uint(y1)};
-            const u32x2 second = {__float_as_uint(y2), __float_as_uint(y3)};
-            __builtin_amdgcn_raw_buffer_store_b64(first, o_rs, at, 0, 0);
-            __builtin_amdgcn_raw_buffer_store_b64(second, o_rs, o_bf ? kNoRow : at + 8u, 0, 0);
+        } else if (o_bf) {  // (a branch that the whole launch takes one way: no request hangs on it)
+            const u32x2 packed = {pack_bf16_rne(y0, y1), pack_bf16_rne(y2, y3)};
+            __builtin_amdgcn_raw_buffer_store_b64(packed, o_rs, at, 0, 0);
+        } else {
+            buffer_store_out(o_rs, at, y0, y1, y2, y3, (float *)nullptr);
         }
     };
     const f32x4 zero = {0.f, 0.f, 0.f, 0.f};

@@ -64,12 +64,26 @@ def test_what_the_chain_parallel_kernel_leaves_to_the_others():
     assert lines((4, 16, 16384, 32), (4, 16, 16384, 128))[0].startswith("scan_dma_kernel")
     assert lines((1, 3, 500, 128), (1, 3, 500, 128))[0].startswith("scan_mfma_kernel")  # few chains
     # bf16 rows: a single scan stays with the kernels that multiply such rows as they are
-    # until there is a workgroup for every CU; the three scans of a backward call, and widths
-    # that those kernels would only take as padded copies, go to the chain-parallel kernel
+    # until the chain-parallel kernel has workgroups for about half of the CUs, and wherever
+    # it would need an exchange; the three scans of a backward call, and widths that those
+    # kernels would only take as padded copies, go to the chain-parallel kernel
     bf16 = dict(dtype=_native.FTC_BF16)
     assert lines((4, 8, 1000, 64), (4, 8, 1000, 64), **bf16)[0].startswith("scan_mfma_kernel")
     assert lines((10, 8, 1000, 64), (10, 8, 1000, 64), **bf16)[0].startswith("scan_mfma_kernel")
+    assert lines((14, 8, 1000, 64), (14, 8, 1000, 64), **bf16)[0].startswith("scan_tph_kernel:")
+    assert lines((16, 8, 1000, 64), (16, 8, 1000, 64), **bf16)[0].startswith("scan_tph_kernel:")
+    assert lines((16, 8, 4096, 64), (16, 8, 4096, 64), **bf16)[0].startswith("scan_mfma_kernel")
+    assert lines((24, 8, 4096, 64), (24, 8, 4096, 64), **bf16)[0].startswith("scan_tph_kernel:")
     assert lines((16, 16, 1000, 64), (16, 16, 1000, 64), **bf16)[0].startswith("scan_tph_kernel:")
+    # config 5: the dV scan (fp32 values, a state of 32 rows) walks its chains whole, however
+    # long; the forward and the scans with a state of 128 rows stay where they were
+    cfg5 = lines((4, 32, 16384, 32), (4, 32, 16384, 128), backward=True, **bf16)
+    assert len(cfg5) == 3 and sum(l.startswith("scan_mfma_kernel") for l in cfg5) == 2
+    dv = [l for l in cfg5 if l.startswith("scan_tph_kernel:")]
+    assert len(dv) == 1 and "state 32 x 128" in dv[0] and "1 segment of 16384 rows" in dv[0]
+    assert lines((4, 32, 16384, 32), (4, 32, 16384, 128), **bf16)[0].startswith("scan_mfma_kernel")
+    assert all(l.startswith("scan_mfma_kernel")
+               for l in lines((2, 32, 16384, 32), (2, 32, 16384, 128), backward=True, **bf16))
     assert lines((10, 8, 1000, 64), (10, 8, 1000, 64), backward=True, **bf16)[0] \
         .startswith("scan_tph_kernel: 3 scans")
     assert lines((6, 8, 257, 48), (6, 8, 257, 40), **bf16)[0].startswith("scan_tph_kernel:")
