@@ -221,9 +221,11 @@ __device__ __forceinline__ void buffer_store_out(__amdgpu_buffer_rsrc_t rsrc, ui
     const u32x4 r = {__float_as_uint(x), __float_as_uint(y), __float_as_uint(z), __float_as_uint(w)};
     __builtin_amdgcn_raw_buffer_store_b128(r, rsrc, byte_offset, 0, 0);
 }
+// (as a conversion of a pair, so that it becomes one v_cvt_pk_bf16_f32)
 __device__ __forceinline__ uint32_t pack_bf16_rne(float lo, float hi) {
-    return (uint32_t)__builtin_bit_cast(uint16_t, (__bf16)lo) |
-           ((uint32_t)__builtin_bit_cast(uint16_t, (__bf16)hi) << 16);
+    typedef float f32x2_t __attribute__((ext_vector_type(2)));
+    typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2_t{lo, hi}, bf16x2_t));
 }
 __device__ __forceinline__ void buffer_store_out(__amdgpu_buffer_rsrc_t rsrc, uint32_t byte_offset,
                                                  float x, float y, float z, float w, bf16_t *) {

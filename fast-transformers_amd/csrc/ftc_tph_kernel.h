@@ -357,10 +357,10 @@ __global__ __launch_bounds__(768, 3) void scan_tph_kernel(uint32_t *__restrict__
             const u32x2 hi = __builtin_amdgcn_raw_buffer_load_b64(rs, bf ? kNoRow : off + 8u, 0, 0);
             return u32x4{lo.x, lo.y, hi.x, hi.y};
         };
-        auto widen = [&](const u32x4 r, bool bf) -> u32x4 {
-            if (!MIX) return r;
-            const u32x4 wide = widen_bf16_quad(r);
-            return u32x4{bf ? wide.x : r.x, bf ? wide.y : r.y, bf ? wide.z : r.z, bf ? wide.w : r.w};
+        // (bf16 quads are widened in place, once, when the look-ahead first touches them: one
+        // position later the cut finds fp32 bit patterns whatever the rows held)
+        auto widen = [&](u32x4 &r, bool bf) {
+            if (MIX && bf) r = widen_bf16_quad(r);
         };
         // Every request is made every time, whether its rows exist or not (a chunk walked for
         // its state alone needs no rows of a; positions past the end of the walk have no
@@ -377,17 +377,17 @@ __global__ __launch_bounds__(768, 3) void scan_tph_kernel(uint32_t *__restrict__
         };
         // the largest magnitudes of the rows of a position against the ceilings (rows that
         // were not asked for read as zeros); k: that position's slot
-        auto look_ahead = [&](const Raw &r, int k, int pos) {
-            raise_slot(slots, k, pos, ce, max_abs4(widen(r.a, a_bf), 0.f), max_abs4(widen(r.b, b_bf), 0.f),
-                       max_abs4(widen(r.v, v_bf), 0.f), lane);
+        auto look_ahead = [&](Raw &r, int k, int pos) {
+            widen(r.a, a_bf), widen(r.b, b_bf), widen(r.v, v_bf);
+            raise_slot(slots, k, pos, ce, max_abs4(r.a, 0.f), max_abs4(r.b, 0.f), max_abs4(r.v, 0.f), lane);
         };
         // A position of the walk goes to its LDS buffer through register set (position % PF).
         // The first n1 positions only feed the state: no piece of a.
         auto cut = [&](const Raw &r, int buf, bool own) {
             lds_char *const pc = unit_pc + buf * kBufBytes;
-            if (own) cut_quad_to_lds(widen(r.a, a_bf), ce.scale_a(), pc, kTileA, a_waddr);
-            cut_quad_to_lds(widen(r.b, b_bf), ce.scale_b(), pc + kOffB, kTileA, b_waddr);
-            cut_quad_to_lds(widen(r.v, v_bf), ce.scale_v(), pc + kOffV, kTileV, v_waddr);
+            if (own) cut_quad_to_lds(r.a, ce.scale_a(), pc, kTileA, a_waddr);
+            cut_quad_to_lds(r.b, ce.scale_b(), pc + kOffB, kTileA, b_waddr);
+            cut_quad_to_lds(r.v, ce.scale_v(), pc + kOffV, kTileV, v_waddr);
             if (!own) asm volatile("" ::"v"(r.a));
         };
 #pragma unroll
