@@ -274,8 +274,9 @@ def test_full_config3_size_properties(cp):
 
 def test_full_config5_size_properties(cp):
     """Config 5 at full size: bf16 Q, K, V, N=4, H=32, L=16384, E=32, M=128 (128 chains of 512
-    chunks, two-level state exchange, three backward launches).  Properties over all chains
-    plus two chains against the CPU checker on the same rounded inputs (2e-2 bar)."""
+    chunks; two-level state exchange in the forward and in two of the three backward launches,
+    the third, dV, on the chain-parallel kernel that walks each chain whole).  Properties over
+    all chains plus two chains against the CPU checker on the same rounded inputs (2e-2 bar)."""
     N, H, L, E, M = 4, 32, 16384, 32, 128
     Q, K, V, G = oracle.make_inputs(N, H, L, E, M, seed=5)
     Qb, Kb, Vb = (t.bfloat16().cuda() for t in (Q, K, V))
