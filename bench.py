@@ -44,10 +44,10 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 matrix, published
 # carries it only while the sources are unchanged, otherwise null.
 MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {
     # workload: (bytes, kernel source hash at the time of the measurement)
-    "cfg2": (139760441, "59c5d990cc74a069"),
-    "cfg3": (3144253172, "59c5d990cc74a069"),
-    "cfg5": (4976228341, "59c5d990cc74a069"),
-    "wide": (1877429610, "59c5d990cc74a069"),
+    "cfg2": (139416036, "330038701fbc7773"),
+    "cfg3": (2621805912, "330038701fbc7773"),
+    "cfg5": (4975946637, "330038701fbc7773"),
+    "wide": (1876787734, "330038701fbc7773"),
 }
 
 WORKLOADS = {

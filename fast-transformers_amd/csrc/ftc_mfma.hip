@@ -127,21 +127,33 @@ int tp_exchange_segments(int64_t units, int64_t L, bool wide, int *nseg) {
     // Up to 64 chunks the cut chains without an exchange are as fast (cfg2: 30 us either way)
     // and need no workspace.
     const bool force = tuning().tpx_segs >= 2;  // tuning aid: also where the rules below say no
-    if (!force && (units < 1 || (units > 128 && !wide) || total_chunks <= 64)) return 0;
-    // (wide states: also with more workgroups than CUs, where chains are too long to walk whole)
+    if (!force && (units < 1 || total_chunks <= 64)) return 0;
+    // (more workgroups than CUs: only where chains are too long to walk whole)
     if (!force && units > 128 && total_chunks <= 256) return 0;
     int64_t want = 256 / units;
-    if (wide && units * want != 256) {
-        // Workgroups that do not fill whole rounds of 256: the number of segments with the
-        // shortest estimated time -- rounds x (a segment walked twice, the first time at 0.4
-        // of the cost, plus about six chunks' time for the exchange and the start).
+    // the number of segments with the shortest estimated time, rounds x (a segment walked
+    // twice + the exchange and the start, in chunks' time)
+    auto shortest = [&](double twice, double fixed) {
         double best = 1e30;
         for (int64_t n = std::max<int64_t>(2, (total_chunks + 255) / 256); n <= 64; n++) {
             const int64_t c = ((total_chunks + n - 1) / n + kTpAhead - 1) / kTpAhead * kTpAhead;
             const int64_t rounds = (units * ((total_chunks + c - 1) / c) + 255) / 256;
-            const double t = (double)rounds * (1.4 * (double)c + 6.0);
+            const double t = (double)rounds * (twice * (double)c + fixed);
             if (t < best - 1e-9) best = t, want = n;
         }
+    };
+    if (wide) {
+        // workgroups that do not fill whole rounds of 256 (the first walk at 0.4 of the cost)
+        if (units * want != 256) shortest(1.4, 6.0);
+    } else if (want < 2 || (total_chunks + want - 1) / want > 256) {
+        // 64 x 64 with no single round of segments of at most 256 chunks: a few rounds still
+        // beat the kernels that split L while those have no more than a wavefront or two per
+        // SIMD to run (backward, ms, this way with the segments chosen here / split L:
+        // N*H = 16, L=65536: 0.71 / 0.79; 32, L=32768: 0.72 / 0.82; 64, L=16384: 0.80 / 0.91;
+        // 128, L=16384: 1.36 / 1.56; but 256, L=16384: 2.70 / 2.60.  Ten segments at N*H = 16
+        // against 8: 0.83, 11: 0.82, 16: 0.79 -- the last round wants to be full).
+        if (!force && units > 384) return 0;
+        shortest(1.0, 40.0);
     }
     want = std::min<int64_t>(want, total_chunks / 8);
     if (tuning().tpx_segs >= 0) want = std::max(1, tuning().tpx_segs);  // tuning aid

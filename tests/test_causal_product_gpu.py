@@ -845,6 +845,9 @@ TPX_SHAPES = [
     # wider states; the last one has more workgroups than the GPU has CUs (a workgroup only
     # ever waits for workgroups that started before it)
     (1, 8, 5000, 128, 128), (2, 4, 9000, 100, 68), (1, 130, 8200, 36, 36),
+    # 64 x 64 on chains too long to walk whole: the backward's 129 chains x scans in three
+    # segments each, two rounds of workgroups
+    (1, 43, 8300, 64, 64),
 ]
 
 

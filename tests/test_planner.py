@@ -40,9 +40,21 @@ def test_long_chains_exchange_their_segment_sums():
     need = int(field(fwd[0], r"workspace (\d+) bytes"))
     lib = _native.load()
     assert 0 < need <= lib.ftc_causal_dot_product_workspace_bytes(1, 16, 65536, 64, 64, 0)
-    # three scans of 16 chains would need segments of 412 chunks: the kernels that split L
+    # three scans of 16 chains: one round of workgroups would need segments of 412 chunks, so
+    # just under two rounds of shorter ones
     bwd = lines((1, 16, 65536, 64), (1, 16, 65536, 64), backward=True)
-    assert bwd[0].startswith("scan_dma_kernel: 3 scans")
+    assert bwd[0].startswith("scan_tph_kernel (exchange): 3 scans")
+    assert "10 segments of 6656 rows" in bwd[0] and "480 workgroups" in bwd[0]
+    need = int(field(bwd[0], r"workspace (\d+) bytes"))
+    assert 0 < need <= lib.ftc_causal_dot_backward_workspace_bytes(1, 16, 65536, 64, 64, 0)
+    # more workgroups than CUs: three full rounds for 64 chains, and the kernels that split L
+    # from 385 scans on, or where the chains can be walked whole
+    bwd = lines((4, 16, 16384, 64), (4, 16, 16384, 64), backward=True)
+    assert bwd[0].startswith("scan_tph_kernel (exchange): 3 scans")
+    assert "4 segments of 4096 rows" in bwd[0] and "768 workgroups" in bwd[0]
+    assert lines((3, 64, 16384, 64), (3, 64, 16384, 64), backward=True)[0].startswith("scan_dma_kernel")
+    assert lines((3, 64, 16384, 64), (3, 64, 16384, 64))[0].startswith("scan_tph_kernel (exchange):")
+    assert lines((8, 16, 8192, 64), (8, 16, 8192, 64), backward=True)[0].startswith("scan_tph_kernel:")
     # config 4's operator shape
     op = lines((10, 8, 4096, 64), (10, 8, 4096, 64))
     assert op[0].startswith("scan_tph_kernel (exchange):") and "3 segments of 1408 rows" in op[0]
