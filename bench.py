@@ -44,10 +44,10 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 matrix, published
 # carries it only while the sources are unchanged, otherwise null.
 MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {
     # workload: (bytes, kernel source hash at the time of the measurement)
-    "cfg2": (139416036, "330038701fbc7773"),
-    "cfg3": (2621805912, "330038701fbc7773"),
-    "cfg5": (4975946637, "330038701fbc7773"),
-    "wide": (1876787734, "330038701fbc7773"),
+    "cfg2": (139285323, "6082aeb65eab84bd"),
+    "cfg3": (2597256738, "6082aeb65eab84bd"),
+    "cfg5": (4976213514, "6082aeb65eab84bd"),
+    "wide": (1876867599, "6082aeb65eab84bd"),
 }
 
 WORKLOADS = {

@@ -120,7 +120,7 @@ int tp_segment_starts(int64_t chunks, int nseg, int32_t *start) {
 // chain is cut into as many equal segments as fill the GPU (one workgroup each); a workgroup
 // walks its own chunks twice, first for their state alone.  Returns the number of chunks per
 // segment (0: not this way) and the number of segments in *nseg.
-int tp_exchange_segments(int64_t units, int64_t L, bool wide, int *nseg) {
+int tp_exchange_segments(int64_t units, int64_t L, bool wide, int *nseg, bool keep_two = false) {
     const int64_t total_chunks = (L + kChunk - 1) / kChunk;
     *nseg = 0;
     if (tuning().tpx == 0) return 0;  // tuning aid
@@ -155,6 +155,12 @@ int tp_exchange_segments(int64_t units, int64_t L, bool wide, int *nseg) {
         if (!force && units > 384) return 0;
         shortest(1.0, 40.0);
     }
+    // Two segments of up to 64 chunks lose to chains cut in two without an exchange, whose
+    // first workgroup walks its part once (forward, 96 chains, L=4096: 117 against 100 us; 128
+    // chains: 145 against 128; backward of 32 chains: 110 against 95); with three segments the
+    // exchange wins again (backward of 24 chains: 83 against 86; forward of 64: 73 against 88).
+    // (`keep_two`: the caller compares with other kernels, not with cut chains)
+    if (!force && !wide && !keep_two && want == 2 && total_chunks <= 128) return 0;
     want = std::min<int64_t>(want, total_chunks / 8);
     if (tuning().tpx_segs >= 0) want = std::max(1, tuning().tpx_segs);  // tuning aid
     if (want < 2) return 0;
@@ -205,7 +211,7 @@ void tp_plan_compute(int64_t D, int64_t F, int64_t chains, int nscans, int64_t L
     // than two rounds of workgroups, as for 64 x 64.
     if (narrow && units > 512) return;
     if (!forced && D <= 64 && F <= 64 && units > 512 && L <= 2 * kChunk) return;
-    if (!narrow) *seg_chunks = tp_exchange_segments(units, L, wide, nseg);
+    if (!narrow) *seg_chunks = tp_exchange_segments(units, L, wide, nseg, lone_mixed);
     if (lone_mixed && units < 256 && *seg_chunks > 0) {
         *nseg = *seg_chunks = 0;
         return;

@@ -55,6 +55,10 @@ def test_long_chains_exchange_their_segment_sums():
     assert lines((3, 64, 16384, 64), (3, 64, 16384, 64), backward=True)[0].startswith("scan_dma_kernel")
     assert lines((3, 64, 16384, 64), (3, 64, 16384, 64))[0].startswith("scan_tph_kernel (exchange):")
     assert lines((8, 16, 8192, 64), (8, 16, 8192, 64), backward=True)[0].startswith("scan_tph_kernel:")
+    # two segments of up to 64 chunks: chains cut in two without an exchange instead
+    assert lines((1, 96, 4096, 64), (1, 96, 4096, 64))[0].startswith("scan_tph_kernel: 1 scan")
+    assert "cuts at chunks 0,92,128" in lines((1, 32, 4096, 64), (1, 32, 4096, 64), backward=True)[0]
+    assert lines((1, 96, 8192, 64), (1, 96, 8192, 64))[0].startswith("scan_tph_kernel (exchange):")
     # config 4's operator shape
     op = lines((10, 8, 4096, 64), (10, 8, 4096, 64))
     assert op[0].startswith("scan_tph_kernel (exchange):") and "3 segments of 1408 rows" in op[0]
