@@ -44,10 +44,10 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 matrix, published
 # carries it only while the sources are unchanged, otherwise null.
 MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {
     # workload: (bytes, kernel source hash at the time of the measurement)
-    "cfg2": (139285323, "6082aeb65eab84bd"),
-    "cfg3": (2597256738, "6082aeb65eab84bd"),
-    "cfg5": (4976213514, "6082aeb65eab84bd"),
-    "wide": (1876867599, "6082aeb65eab84bd"),
+    "cfg2": (139777467, "7455525e0f640423"),
+    "cfg3": (2610822417, "7455525e0f640423"),
+    "cfg5": (4976327361, "7455525e0f640423"),
+    "wide": (1877422781, "7455525e0f640423"),
 }
 
 WORKLOADS = {

@@ -46,7 +46,8 @@ bool mfma_scan_supported_widths(int64_t D, int64_t F) {
 // other than 64 x 64, for which the kernels that split L are half as fast as for 64 x 64;
 // `others`: one of those kernels takes this shape (else the choice is the VALU kernel).
 // Returns the number of segments per chain (0: another kernel takes the launch).
-int tp_kernel_segments(int64_t units, int64_t L, bool wide, bool others, bool long_chains = false) {
+int tp_kernel_segments(int64_t units, int64_t L, bool wide, bool others, bool long_chains = false,
+                       bool cut_long = false) {
     // a chain is walked by one workgroup from end to end: beyond 256 chunks the split of L
     // of the other kernels is faster, and its segment sums also keep the rounding of a long
     // running state in check (`long_chains`: the caller knows better, see tp_plan_compute)
@@ -65,7 +66,9 @@ int tp_kernel_segments(int64_t units, int64_t L, bool wide, bool others, bool lo
     // state alone are few.
     if (nseg > 1 && total_chunks > 128) {
         if (!wide) return 0;
-        nseg = 1;
+        // (`cut_long`: shapes that never exchange keep their cuts: 32 x 128, 64 chains, L=8192,
+        // forward: 190 us in two segments against 219 whole and 206 on the kernels that split L)
+        if (!cut_long) nseg = 1;
     }
     // (wide states: the other kernels run them as column slices that each repeat the chunk
     // product, and lose at any number of rounds; on a quarter of the CUs they still win, N=1,
@@ -210,6 +213,23 @@ void tp_plan_compute(int64_t D, int64_t F, int64_t chains, int nscans, int64_t L
     // against 0.60 ms, 20 x 20 0.63 against 0.46 on padded copies), and 32-wide shapes on more
     // than two rounds of workgroups, as for 64 x 64.
     if (narrow && units > 512) return;
+    // ... and 32-wide shapes on few workgroups: a workgroup of this kernel walks its chunks at
+    // 1.1 to 1.7 us each whatever else the GPU does, the kernels that split L spread them over
+    // all CUs (forward, us, this kernel / those: 32 x 128, 32 chains, L=4096: 83 / 62; 16 chains:
+    // 78 / 54; 64 chains, 128 workgroups: 94 / 106.  128 x 32, 32 chains, L=4096: 152 / 69; 64
+    // chains: 170 / 103; 128 chains: 227 / 204, L=2048: 107 / 101; 256 chains: 317 / 383).  Short
+    // chains stay (32 x 128, 32 chains, L=1024: 29 / 39; 128 x 32, 64 chains, L=512: 32 / 36),
+    // and 64 x 32 on the fp16-piece kernel needs 128 workgroups like 32 x 64 (128 chains,
+    // L=2048: 51 / 57, L=8192: 210 / 229; 64 chains, L=1024: 28 / 32, L=2048: 47 / 41).
+    if (narrow && tuning().tp < 0) {
+        const int64_t total_chunks = (L + kChunk - 1) / kChunk;
+        // a single scan on the bf16-piece kernel with half of its consumers without columns
+        const bool lone_slab = F <= 32 && D > 64 && nscans == 1;
+        int64_t least = 64, brief = lone_slab ? 16 : 32;
+        // (the kernels that split L run 96 columns as slices: 32 x 96, 16 chains, L=2048: 44 / 73)
+        if (D <= 32 && F == 96) least = 32, brief = 64;
+        if (units < (lone_slab ? 256 : 128) && !(units >= least && total_chunks <= brief)) return;
+    }
     if (!forced && D <= 64 && F <= 64 && units > 512 && L <= 2 * kChunk) return;
     if (!narrow) *seg_chunks = tp_exchange_segments(units, L, wide, nseg, lone_mixed);
     if (lone_mixed && units < 256 && *seg_chunks > 0) {
@@ -223,7 +243,7 @@ void tp_plan_compute(int64_t D, int64_t F, int64_t chains, int nscans, int64_t L
     // that either kernel writes once, loses: 0.656 against 0.495).  bf16 results make the
     // rounding of a long running fp32 state a non-issue.
     const bool long_chains = mixed == kMixedGradValues && D <= 32 && units == 256;
-    if (*seg_chunks == 0) *nseg = tp_kernel_segments(units, L, wide, others, long_chains);
+    if (*seg_chunks == 0) *nseg = tp_kernel_segments(units, L, wide, others, long_chains, narrow);
 }
 
 // workspace of the exchange: control block, then two state slots (own sum, group total) of

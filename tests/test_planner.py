@@ -199,6 +199,18 @@ def test_wide_states_on_the_chain_parallel_kernel():
     assert lines((512, 16, 64, 20), (512, 16, 64, 20))[0].startswith("pad_rows_kernel")
     assert lines((512, 16, 64, 32), (512, 16, 64, 128))[0].startswith("scan_dma_kernel")
     assert lines((512, 16, 64, 100), (512, 16, 64, 100))[0].startswith("scan_tp_kernel")
+    # 32-wide shapes on few workgroups: the kernels that split L unless the chains are short
+    assert lines((1, 32, 4096, 32), (1, 32, 4096, 128))[0].startswith("scan_dma_kernel")
+    assert lines((1, 32, 1024, 32), (1, 32, 1024, 128))[0].startswith("scan_tph_kernel:")
+    assert lines((1, 64, 4096, 32), (1, 64, 4096, 128))[0].startswith("scan_tph_kernel:")
+    cut = lines((1, 64, 8192, 32), (1, 64, 8192, 128))[0]
+    assert cut.startswith("scan_tph_kernel:") and "2 segments" in cut
+    assert lines((1, 128, 4096, 128), (1, 128, 4096, 32))[0].startswith("scan_mfma_kernel")
+    assert lines((1, 256, 4096, 128), (1, 256, 4096, 32))[0].startswith("scan_tp_kernel:")
+    assert lines((1, 64, 512, 128), (1, 64, 512, 32))[0].startswith("scan_tp_kernel:")
+    assert lines((1, 128, 4096, 64), (1, 128, 4096, 32))[0].startswith("scan_tph_kernel:")
+    assert lines((1, 64, 2048, 64), (1, 64, 2048, 32))[0].startswith("scan_dma_kernel")
+    assert lines((1, 16, 2048, 32), (1, 16, 2048, 96))[0].startswith("scan_tph_kernel:")
     # bf16 rows and widths that are not multiples of 4 go the other ways
     assert lines((8, 16, 4096, 128), (8, 16, 4096, 128), dtype=_native.FTC_BF16)[0] \
         .startswith("scan_mfma_kernel")
