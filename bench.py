@@ -44,10 +44,10 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 matrix, published
 # carries it only while the sources are unchanged, otherwise null.
 MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {
     # workload: (bytes, kernel source hash at the time of the measurement)
-    "cfg2": (139777467, "7455525e0f640423"),
-    "cfg3": (2610822417, "7455525e0f640423"),
-    "cfg5": (4976327361, "7455525e0f640423"),
-    "wide": (1877422781, "7455525e0f640423"),
+    "cfg2": (139800927, "7b32ad770c490eba"),
+    "cfg3": (2610818754, "7b32ad770c490eba"),
+    "cfg5": (4975856449, "7b32ad770c490eba"),
+    "wide": (1877440146, "7b32ad770c490eba"),
 }
 
 WORKLOADS = {

@@ -47,7 +47,7 @@ bool mfma_scan_supported_widths(int64_t D, int64_t F) {
 // `others`: one of those kernels takes this shape (else the choice is the VALU kernel).
 // Returns the number of segments per chain (0: another kernel takes the launch).
 int tp_kernel_segments(int64_t units, int64_t L, bool wide, bool others, bool long_chains = false,
-                       bool cut_long = false) {
+                       bool cut_long = false, int64_t most_units = 512) {
     // a chain is walked by one workgroup from end to end: beyond 256 chunks the split of L
     // of the other kernels is faster, and its segment sums also keep the rounding of a long
     // running state in check (`long_chains`: the caller knows better, see tp_plan_compute)
@@ -77,7 +77,7 @@ int tp_kernel_segments(int64_t units, int64_t L, bool wide, bool others, bool lo
     // Beyond two rounds of workgroups the other kernels win again (1024 chains of 512
     // positions: 128 / 315 us against 135 / 348): there every chain has its own wavefront,
     // all resident at once, and nothing is split either.
-    return units * nseg >= 128 && units <= 512 ? nseg : 0;
+    return units * nseg >= 128 && units <= most_units ? nseg : 0;
 }
 
 // Where to cut a chain of `chunks` chunks into (at most) `nseg` segments for the
@@ -128,9 +128,18 @@ int tp_exchange_segments(int64_t units, int64_t L, bool wide, int *nseg, bool ke
     *nseg = 0;
     if (tuning().tpx == 0) return 0;  // tuning aid
     // Up to 64 chunks the cut chains without an exchange are as fast (cfg2: 30 us either way)
-    // and need no workspace.
+    // and need no workspace -- unless the chains are so few that five or more segments of each
+    // fit one round of workgroups: those win from 24 chunks on, also against the kernels that
+    // split L (64 x 64 forward, us, this way / before: 16 chains, L=2048: 28 / 44, L=1024:
+    // 21 / 28; 8 chains, L=2048: 23 / 31; 32 chains, L=2048: 34 / 42; backward of 8 chains,
+    // L=2048: 31 / 38, of 4: 26 / 37; 128 x 128 forward, 16 chains, L=2048: 50 / 81), in
+    // segments of down to four chunks.
     const bool force = tuning().tpx_segs >= 2;  // tuning aid: also where the rules below say no
-    if (!force && (units < 1 || total_chunks <= 64)) return 0;
+    const bool brief = total_chunks <= 64;
+    // (not for one or two workgroups' worth of chains, 22 against 21 us, and from 33 on only
+    // from 48 chunks: backward of 16 chains, L=1024: 34 against 26 cut in five without an exchange)
+    if (!force && (units < 1 || total_chunks < 24)) return 0;
+    if (!force && brief && (units < 3 || units > 51 || (units > 32 && total_chunks < 48))) return 0;
     // (more workgroups than CUs: only where chains are too long to walk whole)
     if (!force && units > 128 && total_chunks <= 256) return 0;
     int64_t want = 256 / units;
@@ -164,7 +173,7 @@ int tp_exchange_segments(int64_t units, int64_t L, bool wide, int *nseg, bool ke
     // exchange wins again (backward of 24 chains: 83 against 86; forward of 64: 73 against 88).
     // (`keep_two`: the caller compares with other kernels, not with cut chains)
     if (!force && !wide && !keep_two && want == 2 && total_chunks <= 128) return 0;
-    want = std::min<int64_t>(want, total_chunks / 8);
+    want = std::min<int64_t>(want, total_chunks / (brief ? 4 : 8));
     if (tuning().tpx_segs >= 0) want = std::max(1, tuning().tpx_segs);  // tuning aid
     if (want < 2) return 0;
     const int64_t seg_chunks = ((total_chunks + want - 1) / want + kTpAhead - 1) / kTpAhead * kTpAhead;
@@ -201,6 +210,8 @@ void tp_plan_compute(int64_t D, int64_t F, int64_t chains, int nscans, int64_t L
     // here for up to 128 chains (L=1000, N*H = 80: 50 against 101 us).
     const bool lone_mixed = mixed && nscans == 1 && others;
     if (lone_mixed && units < 112) return;
+    // (N*H = 128, L=1024: 35 against 38 us; L=2048: 61 against 54)
+    if (lone_mixed && units < 192 && L > 48 * kChunk) return;
     // Shapes of the other kernels with 32 rows or columns (a workgroup here has half of its
     // matrix work or half of its consumers to spare for them): measured at N=8, H=16, L=4096,
     // forward + backward, 32 x 128 0.62 against 0.80 ms and 128 x 32 0.76 against 0.78 on whole
@@ -236,6 +247,14 @@ void tp_plan_compute(int64_t D, int64_t F, int64_t chains, int nscans, int64_t L
         *nseg = *seg_chunks = 0;
         return;
     }
+    // ... and so do the three scans of a backward call over bf16 rows where the exchange would
+    // have two segments per chain or more than one round of workgroups (32 chains, L=8192: 232
+    // against 201 us, L=16384: 448 against 364; 16 chains, five segments each: 109 against 168
+    // and 194 against 227)
+    if (mixed == kMixedRows && nscans == 3 && *seg_chunks > 0 && units * 3 > 256) {
+        *nseg = *seg_chunks = 0;
+        return;
+    }
     // The dV scan of a bf16 backward with a state of at most 32 rows and a workgroup for every
     // CU is walked whole however long the chain: what the kernels that split L read twice there
     // is the fp32 gradient, the widest operand by far (N=4, H=32, L=16384, 32 x 128: 0.485
@@ -243,7 +262,13 @@ void tp_plan_compute(int64_t D, int64_t F, int64_t chains, int nscans, int64_t L
     // that either kernel writes once, loses: 0.656 against 0.495).  bf16 results make the
     // rounding of a long running fp32 state a non-issue.
     const bool long_chains = mixed == kMixedGradValues && D <= 32 && units == 256;
-    if (*seg_chunks == 0) *nseg = tp_kernel_segments(units, L, wide, others, long_chains, narrow);
+    // The three scans of a backward call over bf16 rows stay here for up to six rounds of
+    // workgroups: the kernels that split L, good at many fp32 chains, multiply bf16 rows as they
+    // are but re-read them in a first pass (backward, us, this kernel / those: 256 chains, L=1024:
+    // 116 / 172; 512 chains, L=2048: 471 / 593; 768 chains, L=512: 227 / 196, L=2048: 701 / 732).
+    const int64_t most_units = mixed == kMixedRows && nscans == 3 ? 1536 : 512;
+    if (*seg_chunks == 0)
+        *nseg = tp_kernel_segments(units, L, wide, others, long_chains, narrow, most_units);
 }
 
 // workspace of the exchange: control block, then two state slots (own sum, group total) of

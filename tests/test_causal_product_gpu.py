@@ -848,6 +848,8 @@ TPX_SHAPES = [
     # 64 x 64 on chains too long to walk whole: the backward's 129 chains x scans in three
     # segments each, two rounds of workgroups
     (1, 43, 8300, 64, 64),
+    # few short chains: many segments of four chunks each (the last one ragged)
+    (1, 8, 1024, 64, 64), (2, 2, 2000, 128, 128), (1, 3, 1000, 100, 100), (1, 5, 800, 64, 64),
 ]
 
 

@@ -192,8 +192,18 @@ def test_wide_states_on_the_chain_parallel_kernel():
     assert "8 segments of 2560 rows" in rounds[0] and "768 workgroups" in rounds[0]
     # few chains: shapes that the kernels which split L also take go to those below half
     # the CUs, the others go to the chain-parallel kernel at any size
-    assert lines((1, 8, 2048, 128), (1, 8, 2048, 128))[0].startswith("scan_mfma_kernel")
-    assert lines((1, 4, 1000, 100), (1, 4, 1000, 100))[0].startswith("scan_tp_kernel: 1 scan")
+    assert lines((1, 8, 512, 128), (1, 8, 512, 128))[0].startswith("scan_mfma_kernel")
+    # ... unless five or more segments of every chain fit one round of workgroups: an exchange
+    # from 24 chunks on, in segments of down to four chunks
+    few = lines((1, 8, 2048, 128), (1, 8, 2048, 128))[0]
+    assert few.startswith("scan_tp_kernel (exchange):") and "16 segments of 128 rows" in few
+    few = lines((1, 16, 2048, 64), (1, 16, 2048, 64))[0]
+    assert few.startswith("scan_tph_kernel (exchange):") and "16 segments of 128 rows" in few
+    assert lines((1, 16, 1024, 64), (1, 16, 1024, 64), backward=True)[0].startswith("scan_tph_kernel: 3 scans")
+    assert lines((1, 16, 2048, 64), (1, 16, 2048, 64), backward=True)[0].startswith("scan_tph_kernel (exchange)")
+    assert lines((1, 1, 2048, 64), (1, 1, 2048, 64))[0].startswith("scan_dma_kernel")
+    assert lines((1, 4, 500, 100), (1, 4, 500, 100))[0].startswith("scan_tp_kernel: 1 scan")
+    assert lines((1, 4, 1000, 100), (1, 4, 1000, 100))[0].startswith("scan_tp_kernel (exchange): 1 scan")
     # thousands of chains of one or two chunks with a small state, 32-wide shapes on more
     # than two rounds of workgroups: the other routes
     assert lines((512, 16, 64, 20), (512, 16, 64, 20))[0].startswith("pad_rows_kernel")
