@@ -44,10 +44,10 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 matrix, published
 # carries it only while the sources are unchanged, otherwise null.
 MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {
     # workload: (bytes, kernel source hash at the time of the measurement)
-    "cfg2": (139800927, "7b32ad770c490eba"),
-    "cfg3": (2610818754, "7b32ad770c490eba"),
-    "cfg5": (4975856449, "7b32ad770c490eba"),
-    "wide": (1877440146, "7b32ad770c490eba"),
+    "cfg2": (139422559, "e921a76a903a9b53"),
+    "cfg3": (2607757800, "e921a76a903a9b53"),
+    "cfg5": (4976484087, "e921a76a903a9b53"),
+    "wide": (1876772031, "e921a76a903a9b53"),
 }
 
 WORKLOADS = {

@@ -132,8 +132,7 @@ int tp_exchange_segments(int64_t units, int64_t L, bool wide, int *nseg, bool ke
     // fit one round of workgroups: those win from 24 chunks on, also against the kernels that
     // split L (64 x 64 forward, us, this way / before: 16 chains, L=2048: 28 / 44, L=1024:
     // 21 / 28; 8 chains, L=2048: 23 / 31; 32 chains, L=2048: 34 / 42; backward of 8 chains,
-    // L=2048: 31 / 38, of 4: 26 / 37; 128 x 128 forward, 16 chains, L=2048: 50 / 81), in
-    // segments of down to four chunks.
+    // L=2048: 31 / 38, of 4: 26 / 37; 128 x 128 forward, 16 chains, L=2048: 50 / 81).
     const bool force = tuning().tpx_segs >= 2;  // tuning aid: also where the rules below say no
     const bool brief = total_chunks <= 64;
     // (not for one or two workgroups' worth of chains, 22 against 21 us, and from 33 on only
@@ -173,7 +172,8 @@ int tp_exchange_segments(int64_t units, int64_t L, bool wide, int *nseg, bool ke
     // exchange wins again (backward of 24 chains: 83 against 86; forward of 64: 73 against 88).
     // (`keep_two`: the caller compares with other kernels, not with cut chains)
     if (!force && !wide && !keep_two && want == 2 && total_chunks <= 128) return 0;
-    want = std::min<int64_t>(want, total_chunks / (brief ? 4 : 8));
+    // segments of at least four chunks (one or two chains, L=4096: 32 segments 21.5 us, 16: 25.1)
+    want = std::min<int64_t>(want, total_chunks / 4);
     if (tuning().tpx_segs >= 0) want = std::max(1, tuning().tpx_segs);  // tuning aid
     if (want < 2) return 0;
     const int64_t seg_chunks = ((total_chunks + want - 1) / want + kTpAhead - 1) / kTpAhead * kTpAhead;
@@ -219,6 +219,11 @@ void tp_plan_compute(int64_t D, int64_t F, int64_t chains, int nscans, int64_t L
     // 128 x 32 1.73 against 1.58 and 32 x 128 1.70 against 1.59: those stay where they were.
     const bool narrow = others && (D <= 32 || F <= 32);
     if (narrow && D <= 32 && F <= 32) return;
+    // A single scan over bf16 rows in blocks of 64 output columns reads a and b once per block:
+    // beyond two rounds of workgroups, or one for a state of 32 rows, the kernels that split L
+    // win (64 x 128, 512 chains, L=512: 92 against 58 us, L=2048: 309 against 272; 256 chains:
+    // 149 against 175.  32 x 128, 256 chains, L=1024: 75 against 58; 128 chains: 40 against 40)
+    if (lone_mixed && units > (narrow ? 256 : 512)) return;
     // ... and so do thousands of chains of one or two chunks with a state of at most 64 x 64,
     // where a workgroup's start costs more than its chunks (8192 chains, L=64: 32 x 128 1.17
     // against 0.60 ms, 20 x 20 0.63 against 0.46 on padded copies), and 32-wide shapes on more
