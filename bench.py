@@ -44,10 +44,10 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 matrix, published
 # carries it only while the sources are unchanged, otherwise null.
 MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {
     # workload: (bytes, kernel source hash at the time of the measurement)
-    "cfg2": (139422559, "e921a76a903a9b53"),
-    "cfg3": (2607757800, "e921a76a903a9b53"),
-    "cfg5": (4976484087, "e921a76a903a9b53"),
-    "wide": (1876772031, "e921a76a903a9b53"),
+    "cfg2": (139722614, "45bdc7f1c11114e9"),
+    "cfg3": (2611959995, "45bdc7f1c11114e9"),
+    "cfg5": (4975972352, "45bdc7f1c11114e9"),
+    "wide": (1877440570, "45bdc7f1c11114e9"),
 }
 
 WORKLOADS = {

@@ -128,7 +128,7 @@ int tp_exchange_segments(int64_t units, int64_t L, bool wide, int *nseg, bool ke
     *nseg = 0;
     if (tuning().tpx == 0) return 0;  // tuning aid
     // Up to 64 chunks the cut chains without an exchange are as fast (cfg2: 30 us either way)
-    // and need no workspace -- unless the chains are so few that five or more segments of each
+    // and need no workspace -- unless the chains are so few that four or more segments of each
     // fit one round of workgroups: those win from 24 chunks on, also against the kernels that
     // split L (64 x 64 forward, us, this way / before: 16 chains, L=2048: 28 / 44, L=1024:
     // 21 / 28; 8 chains, L=2048: 23 / 31; 32 chains, L=2048: 34 / 42; backward of 8 chains,
@@ -138,7 +138,7 @@ int tp_exchange_segments(int64_t units, int64_t L, bool wide, int *nseg, bool ke
     // (not for one or two workgroups' worth of chains, 22 against 21 us, and from 33 on only
     // from 48 chunks: backward of 16 chains, L=1024: 34 against 26 cut in five without an exchange)
     if (!force && (units < 1 || total_chunks < 24)) return 0;
-    if (!force && brief && (units < 3 || units > 51 || (units > 32 && total_chunks < 48))) return 0;
+    if (!force && brief && (units < 3 || units > 64 || (units > 32 && total_chunks < 48))) return 0;
     // (more workgroups than CUs: only where chains are too long to walk whole)
     if (!force && units > 128 && total_chunks <= 256) return 0;
     int64_t want = 256 / units;

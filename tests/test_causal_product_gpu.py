@@ -801,7 +801,7 @@ TP_SHAPES = [
     # N, H, L, E, M: enough chains for one workgroup per chain (and scan), or few enough that
     # a chain is cut into segments whose workgroups rebuild their starting state
     (16, 8, 1, 64, 64), (16, 8, 31, 64, 64), (20, 8, 33, 64, 64), (3, 16, 1000, 64, 64),
-    (40, 4, 97, 64, 64), (2, 32, 2048, 64, 64), (9, 7, 640, 64, 64),
+    (40, 4, 97, 64, 64), (2, 36, 2048, 64, 64), (9, 7, 640, 64, 64),
     # states of more than 64 rows (walked in two blocks) or columns (a workgroup per block of
     # 64), widths that leave the last block partly empty
     (10, 8, 1000, 128, 128), (8, 8, 333, 96, 96), (16, 4, 97, 100, 100), (4, 4, 640, 48, 80),

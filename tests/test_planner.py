@@ -193,7 +193,7 @@ def test_wide_states_on_the_chain_parallel_kernel():
     # few chains: shapes that the kernels which split L also take go to those below half
     # the CUs, the others go to the chain-parallel kernel at any size
     assert lines((1, 8, 512, 128), (1, 8, 512, 128))[0].startswith("scan_mfma_kernel")
-    # ... unless five or more segments of every chain fit one round of workgroups: an exchange
+    # ... unless four or more segments of every chain fit one round of workgroups: an exchange
     # from 24 chunks on, in segments of down to four chunks
     few = lines((1, 8, 2048, 128), (1, 8, 2048, 128))[0]
     assert few.startswith("scan_tp_kernel (exchange):") and "16 segments of 128 rows" in few
