@@ -587,8 +587,10 @@ def test_random_shapes_and_layouts_against_cpu_checker(cp):
 
 
 STATE_SHAPES = {
-    # (N, H, L, E, M, seed, dtype): LDS-fed kernel with several segments per chain
+    # (N, H, L, E, M, seed, dtype): few short chains, exchanged sums of many short segments
     "e64_m64": (2, 4, 1000, 64, 64, 51, torch.float32),
+    # LDS-fed kernel with several segments per chain
+    "dma_e64_m64": (2, 4, 600, 64, 64, 65, torch.float32),
     # one segment per chain (no exchange)
     "many_chains": (40, 32, 64, 64, 64, 52, torch.float32),
     # long chains: workgroups of the chain-parallel kernel exchange segment sums
