@@ -209,9 +209,13 @@ void tp_plan_compute(int64_t D, int64_t F, int64_t chains, int nscans, int64_t L
     // N*H = 192, L=4096: 160 against 140).  The three scans of a backward call are faster
     // here for up to 128 chains (L=1000, N*H = 80: 50 against 101 us).
     const bool lone_mixed = mixed && nscans == 1 && others;
-    if (lone_mixed && units < 112) return;
+    // ... except on so few chains that sixteen or more segments of each fit one round of
+    // workgroups (forward, 16 chains, L=2048: 30 against 41 us; 8 chains: 24 against 27; 4 chains,
+    // L=4096: 25 against 29; but 20 chains, L=2048: 32 against 29, 6 chains, L=1000: 22 against 20)
+    const bool few_mixed = lone_mixed && units <= 16 && L >= 32 * kChunk;
+    if (lone_mixed && units < 112 && !few_mixed) return;
     // (N*H = 128, L=1024: 35 against 38 us; L=2048: 61 against 54)
-    if (lone_mixed && units < 192 && L > 48 * kChunk) return;
+    if (lone_mixed && units < 192 && L > 48 * kChunk && !few_mixed) return;
     // Shapes of the other kernels with 32 rows or columns (a workgroup here has half of its
     // matrix work or half of its consumers to spare for them): measured at N=8, H=16, L=4096,
     // forward + backward, 32 x 128 0.62 against 0.80 ms and 128 x 32 0.76 against 0.78 on whole
@@ -248,7 +252,7 @@ void tp_plan_compute(int64_t D, int64_t F, int64_t chains, int nscans, int64_t L
     }
     if (!forced && D <= 64 && F <= 64 && units > 512 && L <= 2 * kChunk) return;
     if (!narrow) *seg_chunks = tp_exchange_segments(units, L, wide, nseg, lone_mixed);
-    if (lone_mixed && units < 256 && *seg_chunks > 0) {
+    if (lone_mixed && units < 256 && *seg_chunks > 0 && !few_mixed) {
         *nseg = *seg_chunks = 0;
         return;
     }
@@ -272,6 +276,7 @@ void tp_plan_compute(int64_t D, int64_t F, int64_t chains, int nscans, int64_t L
     // are but re-read them in a first pass (backward, us, this kernel / those: 256 chains, L=1024:
     // 116 / 172; 512 chains, L=2048: 471 / 593; 768 chains, L=512: 227 / 196, L=2048: 701 / 732).
     const int64_t most_units = mixed == kMixedRows && nscans == 3 ? 1536 : 512;
+    if (few_mixed && *seg_chunks == 0) return;
     if (*seg_chunks == 0)
         *nseg = tp_kernel_segments(units, L, wide, others, long_chains, narrow, most_units);
 }

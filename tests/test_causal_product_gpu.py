@@ -480,6 +480,8 @@ BF16_SHAPES = {
     "e64_m96": (2, 4, 1200, 64, 96, 23),
     "e96_m64": (2, 4, 1200, 96, 64, 24),
     "e96_m96": (1, 3, 500, 96, 96, 25),
+    # few chains: the fp16-piece kernel with exchanged sums of short segments, both directions
+    "few_e64_m64": (1, 8, 2048, 64, 64, 26),
 }
 
 

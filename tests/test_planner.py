@@ -85,6 +85,8 @@ def test_what_the_chain_parallel_kernel_leaves_to_the_others():
     # kernels would only take as padded copies, go to the chain-parallel kernel
     bf16 = dict(dtype=_native.FTC_BF16)
     assert lines((4, 8, 1000, 64), (4, 8, 1000, 64), **bf16)[0].startswith("scan_mfma_kernel")
+    assert lines((1, 8, 2048, 64), (1, 8, 2048, 64), **bf16)[0].startswith("scan_tph_kernel (exchange):")
+    assert lines((1, 20, 2048, 64), (1, 20, 2048, 64), **bf16)[0].startswith("scan_mfma_kernel")
     assert lines((10, 8, 1000, 64), (10, 8, 1000, 64), **bf16)[0].startswith("scan_mfma_kernel")
     assert lines((14, 8, 1000, 64), (14, 8, 1000, 64), **bf16)[0].startswith("scan_tph_kernel:")
     assert lines((16, 8, 1000, 64), (16, 8, 1000, 64), **bf16)[0].startswith("scan_tph_kernel:")
