@@ -44,10 +44,10 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 matrix, published
 # carries it only while the sources are unchanged, otherwise null.
 MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {
     # workload: (bytes, kernel source hash at the time of the measurement)
-    "cfg2": (139774862, "8830527fc556410e"),
-    "cfg3": (2611491745, "8830527fc556410e"),
-    "cfg5": (4974833416, "8830527fc556410e"),
-    "wide": (1877409003, "8830527fc556410e"),
+    "cfg2": (139753653, "6ecec02e31a7a6c1"),
+    "cfg3": (2610720461, "6ecec02e31a7a6c1"),
+    "cfg5": (4976761914, "6ecec02e31a7a6c1"),
+    "wide": (1877410734, "6ecec02e31a7a6c1"),
 }
 
 WORKLOADS = {

@@ -212,7 +212,8 @@ void tp_plan_compute(int64_t D, int64_t F, int64_t chains, int nscans, int64_t L
     // ... except on so few chains that sixteen or more segments of each fit one round of
     // workgroups (forward, 16 chains, L=2048: 30 against 41 us; 8 chains: 24 against 27; 4 chains,
     // L=4096: 25 against 29; but 20 chains, L=2048: 32 against 29, 6 chains, L=1000: 22 against 20)
-    const bool few_mixed = lone_mixed && units <= 16 && L >= 32 * kChunk;
+    // (and not beyond 256 chunks: 8 chains, L=32768: 84 against 75)
+    const bool few_mixed = lone_mixed && units <= 16 && L >= 32 * kChunk && L <= 256 * kChunk;
     if (lone_mixed && units < 112 && !few_mixed) return;
     // (N*H = 128, L=1024: 35 against 38 us; L=2048: 61 against 54)
     if (lone_mixed && units < 192 && L > 48 * kChunk && !few_mixed) return;
@@ -308,7 +309,19 @@ MfmaPlan make_plan_compute(int64_t N, int64_t H, int64_t L, int64_t D, int64_t F
         const int64_t waves = chains * nseg;
         if (waves * nscans * flags_per_unit > kMaxWaves || nseg > 4096) continue;  // <= 64 groups of 64 steps
         const double rounds = (double)((waves * nscans + slots - 1) / slots);
-        const double per_wave = nseg > 1 ? c * 1.5 + 3.0 : (double)c;
+        // (the exchange: a step reads the sums of its group and the totals of the groups before
+        // it one after the other, about a chunk and a half's time each beyond the first four;
+        // bf16 forward, 32 chains, L=1024: segments of 1 / 2 / 4 / 8 chunks 34 / 23 / 23 / 29 us)
+        double reads = (double)(nseg - 1);
+        if (nseg > 5) {
+            int64_t g = 1;
+            while (g * g < nseg) g++;
+            reads = (double)((g - 1) + ((nseg + g - 1) / g - 1));
+        }
+        // (states of up to 64 x 64 only: on wider ones a chunk takes longer and the reads weigh
+        // less -- 128 x 32, 8 chains, L=4096: segments of 4 chunks 51 us, of 8 chunks 69)
+        const double look_back = D <= 64 && F <= 64 ? 1.6 * std::max(0.0, reads - 4.0) : 0.0;
+        const double per_wave = nseg > 1 ? c * 1.5 + 3.0 + look_back : (double)c;
         const double cost = rounds * per_wave;
         if (cost < best_cost - 1e-9) {
             best_cost = cost;
