@@ -1,6 +1,7 @@
 // Host side of the MFMA scan (kernel: ftc_mfma_kernel.h): which scans qualify, how L is cut
 // into segments, workspace size, and the launch.
 #include <algorithm>
+#include <cstdint>
 #include <cstdlib>
 
 #include "ftc_wg_kernel.h"
@@ -74,9 +75,8 @@ int tp_kernel_segments(int64_t units, int64_t L, bool wide, bool others, bool lo
     // product, and lose at any number of rounds; on a quarter of the CUs they still win, N=1,
     // H=8, L=2048, 128 x 128 forward: 52 against 91 us.  The VALU kernel loses always.)
     if (wide) return !others || units * nseg >= 128 ? nseg : 0;
-    // Beyond two rounds of workgroups the other kernels win again (1024 chains of 512
-    // positions: 128 / 315 us against 135 / 348): there every chain has its own wavefront,
-    // all resident at once, and nothing is split either.
+    // Beyond `most_units` workgroups the other kernels win again (short chains: there every
+    // chain has its own wavefront, all resident at once, and nothing is split either).
     return units * nseg >= 128 && units <= most_units ? nseg : 0;
 }
 
@@ -276,7 +276,18 @@ void tp_plan_compute(int64_t D, int64_t F, int64_t chains, int nscans, int64_t L
     // workgroups: the kernels that split L, good at many fp32 chains, multiply bf16 rows as they
     // are but re-read them in a first pass (backward, us, this kernel / those: 256 chains, L=1024:
     // 116 / 172; 512 chains, L=2048: 471 / 593; 768 chains, L=512: 227 / 196, L=2048: 701 / 732).
-    const int64_t most_units = mixed == kMixedRows && nscans == 3 ? 1536 : 512;
+    // fp32 rows, 64 x 64: any number of chains of 16 chunks or more (the fp16-piece kernel walks
+    // them faster than the kernels that split L stream them: backward, 256 chains, L=4096: 528
+    // against 694 us; 768 chains, L=2048: 784 against 1013; forward, 1536 chains, L=1024: 309
+    // against 376), six rounds of workgroups from 8 chunks on (backward of 384 chains, L=256:
+    // 71 against 82; of 2048 chains: 327 against 295), two below that (256 chains, L=128: 31
+    // against 27)
+    const int64_t chunks = (L + kChunk - 1) / kChunk;
+    const int64_t most_units = mixed == kMixedRows && nscans == 3 ? 1536
+                               : mixed              ? 512
+                               : chunks >= 16       ? INT64_MAX
+                               : chunks >= 8        ? 1536
+                                                    : 512;
     if (few_mixed && *seg_chunks == 0) return;
     if (*seg_chunks == 0)
         *nseg = tp_kernel_segments(units, L, wide, others, long_chains, narrow, most_units);

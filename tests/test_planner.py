@@ -70,8 +70,12 @@ def test_what_the_chain_parallel_kernel_leaves_to_the_others():
     out = lines((1, 144, 8192, 64), (1, 144, 8192, 64), strides=(far, far, far))
     assert not out[0].startswith("scan_tp_kernel")
     # more chains than two rounds of workgroups
-    many = lines((64, 16, 512, 64), (64, 16, 512, 64))
+    many = lines((64, 16, 128, 64), (64, 16, 128, 64))
     assert many[0].startswith("scan_dma_kernel")
+    # ... which chains of 16 chunks or more fill without losing to them
+    assert lines((64, 16, 512, 64), (64, 16, 512, 64), backward=True)[0].startswith("scan_tph_kernel: 3 scans")
+    assert lines((64, 16, 256, 64), (64, 16, 256, 64), backward=True)[0].startswith("scan_dma_kernel")
+    assert lines((32, 16, 256, 64), (32, 16, 256, 64), backward=True)[0].startswith("scan_tph_kernel: 3 scans")
     # other state sizes and element types
     assert lines((10, 8, 1000, 32), (10, 8, 1000, 32))[0].startswith("scan_dma_kernel")
     # (32 rows or columns: the chain-parallel kernel on whole chains unless both are 32,
