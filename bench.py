@@ -44,10 +44,10 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 matrix, published
 # carries it only while the sources are unchanged, otherwise null.
 MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {
     # workload: (bytes, kernel source hash at the time of the measurement)
-    "cfg2": (139776419, "96bfb084f56e0089"),
-    "cfg3": (2614636155, "96bfb084f56e0089"),
-    "cfg5": (4974988794, "96bfb084f56e0089"),
-    "wide": (1877415417, "96bfb084f56e0089"),
+    "cfg2": (139687154, "1a1de38b75078b6b"),
+    "cfg3": (2610846806, "1a1de38b75078b6b"),
+    "cfg5": (4974030691, "1a1de38b75078b6b"),
+    "wide": (1877439609, "1a1de38b75078b6b"),
 }
 
 WORKLOADS = {

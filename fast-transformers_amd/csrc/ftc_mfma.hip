@@ -233,7 +233,9 @@ void tp_plan_compute(int64_t D, int64_t F, int64_t chains, int nscans, int64_t L
     // where a workgroup's start costs more than its chunks (8192 chains, L=64: 32 x 128 1.17
     // against 0.60 ms, 20 x 20 0.63 against 0.46 on padded copies), and 32-wide shapes on more
     // than two rounds of workgroups, as for 64 x 64.
-    if (narrow && units > 512) return;
+    // (four rounds for a state of 32 rows on chains of 32 chunks or more: 32 x 128 forward, 384
+    // chains, L=1024: 113 against 174 us; 512 chains, L=2048: 277 against 344; 1024 chains: 293 / 279)
+    if (narrow && units > (D <= 32 && L >= 32 * kChunk ? 1024 : 512) && tuning().tp < 0) return;
     // ... and 32-wide shapes on few workgroups: a workgroup of this kernel walks its chunks at
     // 1.1 to 1.7 us each whatever else the GPU does, the kernels that split L spread them over
     // all CUs (forward, us, this kernel / those: 32 x 128, 32 chains, L=4096: 83 / 62; 16 chains:
