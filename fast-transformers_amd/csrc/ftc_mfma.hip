@@ -66,7 +66,8 @@ int tp_kernel_segments(int64_t units, int64_t L, bool wide, bool others, bool lo
     // against 201 -- cut chains pay off while the chunks that a workgroup walks for its
     // state alone are few.
     if (nseg > 1 && total_chunks > 128) {
-        if (!wide) return 0;
+        if (!wide && !long_chains) return 0;
+        if (!wide) nseg = 1;
         // (`cut_long`: shapes that never exchange keep their cuts: 32 x 128, 64 chains, L=8192,
         // forward: 190 us in two segments against 219 whole and 206 on the kernels that split L)
         if (!cut_long) nseg = 1;
@@ -77,7 +78,7 @@ int tp_kernel_segments(int64_t units, int64_t L, bool wide, bool others, bool lo
     if (wide) return !others || units * nseg >= 128 ? nseg : 0;
     // Beyond `most_units` workgroups the other kernels win again (short chains: there every
     // chain has its own wavefront, all resident at once, and nothing is split either).
-    return units * nseg >= 128 && units <= most_units ? nseg : 0;
+    return units * nseg >= (long_chains ? 112 : 128) && units <= most_units ? nseg : 0;
 }
 
 // Where to cut a chain of `chunks` chunks into (at most) `nseg` segments for the
@@ -254,7 +255,15 @@ void tp_plan_compute(int64_t D, int64_t F, int64_t chains, int nscans, int64_t L
         if (units < (lone_slab ? 256 : 128) && !(units >= least && total_chunks <= brief)) return;
     }
     if (!forced && D <= 64 && F <= 64 && units > 512 && L <= 2 * kChunk) return;
-    if (!narrow) *seg_chunks = tp_exchange_segments(units, L, wide, nseg, lone_mixed);
+    // fp32 64 x 64 chains of 257 to 1024 chunks on 112 workgroups or more are walked whole: a
+    // running fp32 state of that length is what the reference keeps too (L=32768 against float64:
+    // scale errors 1.8e-6 forward and 3e-6 backward where the reference's own order has 1.1e-6 and
+    // 4e-6), and a workgroup per chain and scan reads every row once where an exchange reads it
+    // twice and the kernels that split L more often (us, whole / before: forward, 256 chains,
+    // L=16384: 883 / 1061; 128 chains: 485 / 537; backward of 64 chains: 559 / 704; of 256: 2082
+    // / 2626; of 256 at L=32768: 4134 / 5290; of 36 chains, 108 workgroups: 466 / 419).
+    const bool walk_long = !wide && !mixed && L > 256 * kChunk && L <= 1024 * kChunk && units >= 112;
+    if (!narrow && !walk_long) *seg_chunks = tp_exchange_segments(units, L, wide, nseg, lone_mixed);
     if (lone_mixed && units < 256 && *seg_chunks > 0 && !few_mixed) {
         *nseg = *seg_chunks = 0;
         return;
@@ -273,7 +282,7 @@ void tp_plan_compute(int64_t D, int64_t F, int64_t chains, int nscans, int64_t L
     // against 0.629 ms; the forward of the same shape, whose wide operand is the fp32 result
     // that either kernel writes once, loses: 0.656 against 0.495).  bf16 results make the
     // rounding of a long running fp32 state a non-issue.
-    const bool long_chains = mixed == kMixedGradValues && D <= 32 && units == 256;
+    const bool long_chains = walk_long || (mixed == kMixedGradValues && D <= 32 && units == 256);
     // The three scans of a backward call over bf16 rows stay here for up to six rounds of
     // workgroups: the kernels that split L, good at many fp32 chains, multiply bf16 rows as they
     // are but re-read them in a first pass (backward, us, this kernel / those: 256 chains, L=1024:

@@ -47,13 +47,19 @@ def test_long_chains_exchange_their_segment_sums():
     assert "10 segments of 6656 rows" in bwd[0] and "480 workgroups" in bwd[0]
     need = int(field(bwd[0], r"workspace (\d+) bytes"))
     assert 0 < need <= lib.ftc_causal_dot_backward_workspace_bytes(1, 16, 65536, 64, 64, 0)
-    # more workgroups than CUs: three full rounds for 64 chains, and the kernels that split L
-    # from 385 scans on, or where the chains can be walked whole
-    bwd = lines((4, 16, 16384, 64), (4, 16, 16384, 64), backward=True)
+    # more workgroups than CUs: three rounds for 32 chains of 2048 chunks
+    bwd = lines((2, 16, 65536, 64), (2, 16, 65536, 64), backward=True)
     assert bwd[0].startswith("scan_tph_kernel (exchange): 3 scans")
-    assert "4 segments of 4096 rows" in bwd[0] and "768 workgroups" in bwd[0]
-    assert lines((3, 64, 16384, 64), (3, 64, 16384, 64), backward=True)[0].startswith("scan_dma_kernel")
-    assert lines((3, 64, 16384, 64), (3, 64, 16384, 64))[0].startswith("scan_tph_kernel (exchange):")
+    assert "8 segments of 8192 rows" in bwd[0] and "768 workgroups" in bwd[0]
+    # chains of 257 to 1024 chunks on 112 workgroups or more are walked whole, in any number of
+    # rounds; on fewer they exchange
+    bwd = lines((4, 16, 16384, 64), (4, 16, 16384, 64), backward=True)
+    assert bwd[0].startswith("scan_tph_kernel: 3 scans") and "1 segment of 16384 rows" in bwd[0]
+    assert lines((4, 16, 16384, 64), (4, 16, 16384, 64))[0].startswith("scan_tph_kernel (exchange):")
+    assert lines((3, 64, 16384, 64), (3, 64, 16384, 64), backward=True)[0].startswith("scan_tph_kernel: 3 scans")
+    assert lines((3, 64, 16384, 64), (3, 64, 16384, 64))[0].startswith("scan_tph_kernel: 1 scan")
+    assert lines((1, 36, 16384, 64), (1, 36, 16384, 64), backward=True)[0].startswith("scan_tph_kernel (exchange)")
+    assert lines((4, 64, 40000, 64), (4, 64, 40000, 64), backward=True)[0].startswith("scan_dma_kernel")
     assert lines((8, 16, 8192, 64), (8, 16, 8192, 64), backward=True)[0].startswith("scan_tph_kernel:")
     # two segments of up to 64 chunks: chains cut in two without an exchange instead
     assert lines((1, 96, 4096, 64), (1, 96, 4096, 64))[0].startswith("scan_tph_kernel: 1 scan")
