@@ -44,10 +44,10 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 matrix, published
 # carries it only while the sources are unchanged, otherwise null.
 MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {
     # workload: (bytes, kernel source hash at the time of the measurement)
-    "cfg2": (139793830, "9495b84049b7336f"),
-    "cfg3": (2598847983, "9495b84049b7336f"),
-    "cfg5": (4976119843, "9495b84049b7336f"),
-    "wide": (1877347272, "9495b84049b7336f"),
+    "cfg2": (139768309, "5065af562d778f5f"),
+    "cfg3": (2612741944, "5065af562d778f5f"),
+    "cfg5": (4975477087, "5065af562d778f5f"),
+    "wide": (1877449133, "5065af562d778f5f"),
 }
 
 WORKLOADS = {

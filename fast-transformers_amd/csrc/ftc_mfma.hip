@@ -262,7 +262,12 @@ void tp_plan_compute(int64_t D, int64_t F, int64_t chains, int nscans, int64_t L
     // twice and the kernels that split L more often (us, whole / before: forward, 256 chains,
     // L=16384: 883 / 1061; 128 chains: 485 / 537; backward of 64 chains: 559 / 704; of 256: 2082
     // / 2626; of 256 at L=32768: 4134 / 5290; of 36 chains, 108 workgroups: 466 / 419).
-    const bool walk_long = !wide && !mixed && L > 256 * kChunk && L <= 1024 * kChunk && units >= 112;
+    // The same for the other states that the fp16-piece kernel takes, from 192 workgroups on, 128
+    // beyond 512 chunks (64 x 128 forward, 128 chains, L=16384: 662 against 1049 us; 64 chains,
+    // L=32768: 910 against 1083, L=16384: 458 against 452; 48 x 80, 64 chains, L=16384: 470 / 405).  Not for the bf16-piece kernel: 128 x 128 walked whole at L=12000 is outside the
+    // element-wise bound 2.8 times as often as the reference's own order, where twice is the bar.
+    const bool walk_long = !mixed && !narrow && D <= 64 && L > 256 * kChunk && L <= 1024 * kChunk &&
+                           units >= (!wide ? 112 : L > 512 * kChunk ? 128 : 192);
     if (!narrow && !walk_long) *seg_chunks = tp_exchange_segments(units, L, wide, nseg, lone_mixed);
     if (lone_mixed && units < 256 && *seg_chunks > 0 && !few_mixed) {
         *nseg = *seg_chunks = 0;

@@ -807,7 +807,7 @@ TP_SHAPES = [
     (16, 8, 1, 64, 64), (16, 8, 31, 64, 64), (20, 8, 33, 64, 64), (3, 16, 1000, 64, 64),
     (40, 4, 97, 64, 64), (2, 36, 2048, 64, 64), (9, 7, 640, 64, 64),
     # chains of 257 chunks walked whole
-    (1, 112, 8224, 64, 64),
+    (1, 112, 8224, 64, 64), (1, 200, 8200, 36, 36),
     # states of more than 64 rows (walked in two blocks) or columns (a workgroup per block of
     # 64), widths that leave the last block partly empty
     (10, 8, 1000, 128, 128), (8, 8, 333, 96, 96), (16, 4, 97, 100, 100), (4, 4, 640, 48, 80),
@@ -848,11 +848,11 @@ TPX_SHAPES = [
     # N, H, L, E, M: long chains on few CUs: segments that exchange their sums (one and two
     # levels of the sum, ragged last segment, a last segment shorter than the others)
     (2, 8, 4096, 64, 64), (1, 3, 9000, 64, 64), (3, 5, 2100, 64, 64), (1, 2, 40000, 64, 64),
-    # wider states; the last one has more workgroups than the GPU has CUs (a workgroup only
-    # ever waits for workgroups that started before it)
-    (1, 8, 5000, 128, 128), (2, 4, 9000, 100, 68), (1, 130, 8200, 36, 36),
+    # wider states
+    (1, 8, 5000, 128, 128), (2, 4, 9000, 100, 68), (1, 40, 8200, 36, 36),
     # 64 x 64 on chains too long to walk whole: the backward's 54 chains x scans in nine
-    # segments each, two rounds of workgroups
+    # segments each, two rounds of workgroups (a workgroup only ever waits for workgroups that
+    # started before it)
     (1, 18, 33000, 64, 64),
     # few short chains: many segments of four chunks each (the last one ragged)
     (1, 8, 1024, 64, 64), (2, 2, 2000, 128, 128), (1, 3, 1000, 100, 100), (1, 5, 800, 64, 64),
