@@ -482,6 +482,8 @@ BF16_SHAPES = {
     "e96_m96": (1, 3, 500, 96, 96, 25),
     # few chains: the fp16-piece kernel with exchanged sums of short segments, both directions
     "few_e64_m64": (1, 8, 2048, 64, 64, 26),
+    # the backward's chains of 257 chunks walked whole
+    "long_e64_m64": (1, 64, 8224, 64, 64, 27),
 }
 
 
