@@ -44,10 +44,10 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 matrix, published
 # carries it only while the sources are unchanged, otherwise null.
 MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {
     # workload: (bytes, kernel source hash at the time of the measurement)
-    "cfg2": (139434364, "f8438fc927fd73a2"),
-    "cfg3": (2603710332, "f8438fc927fd73a2"),
-    "cfg5": (4976680799, "f8438fc927fd73a2"),
-    "wide": (1877123745, "f8438fc927fd73a2"),
+    "cfg2": (139732675, "410dd97ab394ab6e"),
+    "cfg3": (2609627685, "410dd97ab394ab6e"),
+    "cfg5": (4975441313, "410dd97ab394ab6e"),
+    "wide": (1877418330, "410dd97ab394ab6e"),
 }
 
 WORKLOADS = {

@@ -266,11 +266,13 @@ void tp_plan_compute(int64_t D, int64_t F, int64_t chains, int nscans, int64_t L
     // beyond 512 chunks (64 x 128 forward, 128 chains, L=16384: 662 against 1049 us; 64 chains,
     // L=32768: 910 against 1083, L=16384: 458 against 452; 48 x 80, 64 chains, L=16384: 470 / 405).  Not for the bf16-piece kernel: 128 x 128 walked whole at L=12000 is outside the
     // element-wise bound 2.8 times as often as the reference's own order, where twice is the bar.
+    // (32-wide states included: 32 x 128 forward, 128 chains, L=16384: 553 against 756; 64 x 32
+    // backward, 256 chains, L=12000: 1404 against 1825)
     // ... and the three scans of a backward call over bf16 rows, whose results are rounded to
     // bf16 anyway, from 192 workgroups on (64 chains, L=16384: 634 against 783 us; 256 chains:
     // 1783 against 2430; 43 chains: 512 against 483)
     const bool mixed_backward = mixed == kMixedRows && nscans == 3;
-    const bool walk_long = (!mixed || mixed_backward) && !narrow && D <= 64 && L > 256 * kChunk &&
+    const bool walk_long = (!mixed || mixed_backward) && D <= 64 && L > 256 * kChunk &&
                            L <= 1024 * kChunk &&
                            units >= (mixed_backward ? 192 : !wide ? 112 : L > 512 * kChunk ? 128 : 192);
     if (!narrow && !walk_long) *seg_chunks = tp_exchange_segments(units, L, wide, nseg, lone_mixed);

@@ -809,7 +809,7 @@ TP_SHAPES = [
     (16, 8, 1, 64, 64), (16, 8, 31, 64, 64), (20, 8, 33, 64, 64), (3, 16, 1000, 64, 64),
     (40, 4, 97, 64, 64), (2, 36, 2048, 64, 64), (9, 7, 640, 64, 64),
     # chains of 257 chunks walked whole
-    (1, 112, 8224, 64, 64), (1, 200, 8200, 36, 36),
+    (1, 112, 8224, 64, 64), (1, 200, 8200, 36, 36), (1, 200, 8224, 32, 64),
     # states of more than 64 rows (walked in two blocks) or columns (a workgroup per block of
     # 64), widths that leave the last block partly empty
     (10, 8, 1000, 128, 128), (8, 8, 333, 96, 96), (16, 4, 97, 100, 100), (4, 4, 640, 48, 80),

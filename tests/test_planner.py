@@ -236,6 +236,8 @@ def test_wide_states_on_the_chain_parallel_kernel():
     assert lines((1, 128, 4096, 64), (1, 128, 4096, 32))[0].startswith("scan_tph_kernel:")
     assert lines((1, 64, 2048, 64), (1, 64, 2048, 32))[0].startswith("scan_dma_kernel")
     assert lines((1, 16, 2048, 32), (1, 16, 2048, 96))[0].startswith("scan_tph_kernel:")
+    # ... and long ones where whole chains fill three quarters of the CUs
+    assert lines((1, 128, 16384, 32), (1, 128, 16384, 128))[0].startswith("scan_tph_kernel: 1 scan")
     # bf16 rows and widths that are not multiples of 4 go the other ways
     assert lines((8, 16, 4096, 128), (8, 16, 4096, 128), dtype=_native.FTC_BF16)[0] \
         .startswith("scan_mfma_kernel")
