@@ -44,10 +44,10 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 matrix, published
 # carries it only while the sources are unchanged, otherwise null.
 MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {
     # workload: (bytes, kernel source hash at the time of the measurement)
-    "cfg2": (139732675, "410dd97ab394ab6e"),
-    "cfg3": (2609627685, "410dd97ab394ab6e"),
-    "cfg5": (4975441313, "410dd97ab394ab6e"),
-    "wide": (1877418330, "410dd97ab394ab6e"),
+    "cfg2": (139412242, "e5339226847dc061"),
+    "cfg3": (2611673914, "e5339226847dc061"),
+    "cfg5": (4973400091, "e5339226847dc061"),
+    "wide": (1877411258, "e5339226847dc061"),
 }
 
 WORKLOADS = {

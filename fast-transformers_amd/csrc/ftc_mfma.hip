@@ -145,6 +145,8 @@ int tp_exchange_segments(int64_t units, int64_t L, bool wide, int *nseg, bool ke
     int64_t want = 256 / units;
     // the number of segments with the shortest estimated time, rounds x (a segment walked
     // twice + the exchange and the start, in chunks' time)
+    // (wide states: twelve chunks' time for those -- with six, 128 x 128 backward of 16 chains,
+    // L=4096, went into three rounds of 16-chunk segments, 202 us, where two segments take 185)
     auto shortest = [&](double twice, double fixed) {
         double best = 1e30;
         for (int64_t n = std::max<int64_t>(2, (total_chunks + 255) / 256); n <= 64; n++) {
@@ -156,7 +158,7 @@ int tp_exchange_segments(int64_t units, int64_t L, bool wide, int *nseg, bool ke
     };
     if (wide) {
         // workgroups that do not fill whole rounds of 256 (the first walk at 0.4 of the cost)
-        if (units * want != 256) shortest(1.4, 6.0);
+        if (units * want != 256) shortest(1.4, 12.0);
     } else if (want < 2 || (total_chunks + want - 1) / want > 256) {
         // 64 x 64 with no single round of segments of at most 256 chunks: a few rounds still
         // beat the kernels that split L while those have no more than a wavefront or two per
@@ -171,8 +173,10 @@ int tp_exchange_segments(int64_t units, int64_t L, bool wide, int *nseg, bool ke
     // first workgroup walks its part once (forward, 96 chains, L=4096: 117 against 100 us; 128
     // chains: 145 against 128; backward of 32 chains: 110 against 95); with three segments the
     // exchange wins again (backward of 24 chains: 83 against 86; forward of 64: 73 against 88).
+    // Wider states the same (64 x 128 forward, 64 chains, L=4096: 116 against 104; 128 x 128
+    // backward of 16 chains: 204 against 186).
     // (`keep_two`: the caller compares with other kernels, not with cut chains)
-    if (!force && !wide && !keep_two && want == 2 && total_chunks <= 128) return 0;
+    if (!force && !keep_two && want == 2 && total_chunks <= 128) return 0;
     // segments of at least four chunks (one or two chains, L=4096: 32 segments 21.5 us, 16: 25.1)
     want = std::min<int64_t>(want, total_chunks / 4);
     if (tuning().tpx_segs >= 0) want = std::max(1, tuning().tpx_segs);  // tuning aid
@@ -210,14 +214,9 @@ void tp_plan_compute(int64_t D, int64_t F, int64_t chains, int nscans, int64_t L
     // N*H = 192, L=4096: 160 against 140).  The three scans of a backward call are faster
     // here for up to 128 chains (L=1000, N*H = 80: 50 against 101 us).
     const bool lone_mixed = mixed && nscans == 1 && others;
-    // ... except on so few chains that sixteen or more segments of each fit one round of
-    // workgroups (forward, 16 chains, L=2048: 30 against 41 us; 8 chains: 24 against 27; 4 chains,
-    // L=4096: 25 against 29; but 20 chains, L=2048: 32 against 29, 6 chains, L=1000: 22 against 20)
-    // (and not beyond 256 chunks: 8 chains, L=32768: 84 against 75)
-    const bool few_mixed = lone_mixed && units <= 16 && L >= 32 * kChunk && L <= 256 * kChunk;
-    if (lone_mixed && units < 112 && !few_mixed) return;
+    if (lone_mixed && units < 112) return;
     // (N*H = 128, L=1024: 35 against 38 us; L=2048: 61 against 54)
-    if (lone_mixed && units < 192 && L > 48 * kChunk && !few_mixed) return;
+    if (lone_mixed && units < 192 && L > 48 * kChunk) return;
     // Shapes of the other kernels with 32 rows or columns (a workgroup here has half of its
     // matrix work or half of its consumers to spare for them): measured at N=8, H=16, L=4096,
     // forward + backward, 32 x 128 0.62 against 0.80 ms and 128 x 32 0.76 against 0.78 on whole
@@ -276,7 +275,7 @@ void tp_plan_compute(int64_t D, int64_t F, int64_t chains, int nscans, int64_t L
                            L <= 1024 * kChunk &&
                            units >= (mixed_backward ? 192 : !wide ? 112 : L > 512 * kChunk ? 128 : 192);
     if (!narrow && !walk_long) *seg_chunks = tp_exchange_segments(units, L, wide, nseg, lone_mixed);
-    if (lone_mixed && units < 256 && *seg_chunks > 0 && !few_mixed) {
+    if (lone_mixed && units < 256 && *seg_chunks > 0) {
         *nseg = *seg_chunks = 0;
         return;
     }
@@ -302,16 +301,16 @@ void tp_plan_compute(int64_t D, int64_t F, int64_t chains, int nscans, int64_t L
     // fp32 rows, 64 x 64: any number of chains of 16 chunks or more (the fp16-piece kernel walks
     // them faster than the kernels that split L stream them: backward, 256 chains, L=4096: 528
     // against 694 us; 768 chains, L=2048: 784 against 1013; forward, 1536 chains, L=1024: 309
-    // against 376), six rounds of workgroups from 8 chunks on (backward of 384 chains, L=256:
-    // 71 against 82; of 2048 chains: 327 against 295), two below that (256 chains, L=128: 31
-    // against 27)
+    // against 376); from 8 chunks on three rounds of workgroups for a single scan and nine for
+    // the three of a backward call (L=256: backward of 384 chains 71 against 82, of 768 chains
+    // 136 against 146, of 2048 chains 327 against 295; forward of 768 chains 50 against 50, of
+    // 1024 chains 65 against 56), two below that (256 chains, L=128: 31 against 27)
     const int64_t chunks = (L + kChunk - 1) / kChunk;
     const int64_t most_units = mixed == kMixedRows && nscans == 3 ? 1536
                                : mixed              ? 512
                                : chunks >= 16       ? INT64_MAX
-                               : chunks >= 8        ? 1536
+                               : chunks >= 8        ? (nscans == 3 ? 2304 : 768)
                                                     : 512;
-    if (few_mixed && *seg_chunks == 0) return;
     if (*seg_chunks == 0)
         *nseg = tp_kernel_segments(units, L, wide, others, long_chains, narrow, most_units);
 }

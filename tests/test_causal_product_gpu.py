@@ -480,7 +480,7 @@ BF16_SHAPES = {
     "e64_m96": (2, 4, 1200, 64, 96, 23),
     "e96_m64": (2, 4, 1200, 96, 64, 24),
     "e96_m96": (1, 3, 500, 96, 96, 25),
-    # few chains: the fp16-piece kernel with exchanged sums of short segments, both directions
+    # few chains: the backward on the fp16-piece kernel with exchanged sums of short segments
     "few_e64_m64": (1, 8, 2048, 64, 64, 26),
     # the backward's chains of 257 chunks walked whole
     "long_e64_m64": (1, 64, 8224, 64, 64, 27),
