@@ -44,10 +44,10 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 matrix, published
 # carries it only while the sources are unchanged, otherwise null.
 MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {
     # workload: (bytes, kernel source hash at the time of the measurement)
-    "cfg2": (139412242, "e5339226847dc061"),
-    "cfg3": (2611673914, "e5339226847dc061"),
-    "cfg5": (4973400091, "e5339226847dc061"),
-    "wide": (1877411258, "e5339226847dc061"),
+    "cfg2": (139695660, "58af0cd3d23348b6"),
+    "cfg3": (2610208921, "58af0cd3d23348b6"),
+    "cfg5": (4976938155, "58af0cd3d23348b6"),
+    "wide": (1877438021, "58af0cd3d23348b6"),
 }
 
 WORKLOADS = {

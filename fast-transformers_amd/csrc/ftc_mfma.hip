@@ -48,7 +48,7 @@ bool mfma_scan_supported_widths(int64_t D, int64_t F) {
 // `others`: one of those kernels takes this shape (else the choice is the VALU kernel).
 // Returns the number of segments per chain (0: another kernel takes the launch).
 int tp_kernel_segments(int64_t units, int64_t L, bool wide, bool others, bool long_chains = false,
-                       bool cut_long = false, int64_t most_units = 512) {
+                       bool cut_long = false, int64_t most_units = 512, int64_t brief_chunks = 0) {
     // a chain is walked by one workgroup from end to end: beyond 256 chunks the split of L
     // of the other kernels is faster, and its segment sums also keep the rounding of a long
     // running state in check (`long_chains`: the caller knows better, see tp_plan_compute)
@@ -75,10 +75,12 @@ int tp_kernel_segments(int64_t units, int64_t L, bool wide, bool others, bool lo
     // (wide states: the other kernels run them as column slices that each repeat the chunk
     // product, and lose at any number of rounds; on a quarter of the CUs they still win, N=1,
     // H=8, L=2048, 128 x 128 forward: 52 against 91 us.  The VALU kernel loses always.)
-    if (wide) return !others || units * nseg >= 128 ? nseg : 0;
+    // (chains of up to `brief_chunks` chunks at any number, see tp_plan_compute)
+    const bool brief = total_chunks <= brief_chunks;
+    if (wide) return !others || brief || units * nseg >= 128 ? nseg : 0;
     // Beyond `most_units` workgroups the other kernels win again (short chains: there every
     // chain has its own wavefront, all resident at once, and nothing is split either).
-    return units * nseg >= (long_chains ? 112 : 128) && units <= most_units ? nseg : 0;
+    return (brief || units * nseg >= (long_chains ? 112 : 128)) && units <= most_units ? nseg : 0;
 }
 
 // Where to cut a chain of `chunks` chunks into (at most) `nseg` segments for the
@@ -223,6 +225,13 @@ void tp_plan_compute(int64_t D, int64_t F, int64_t chains, int nscans, int64_t L
     // chains, but 32 x 32 0.34 against 0.28, and with an exchange (N=4, H=16, L=16384)
     // 128 x 32 1.73 against 1.58 and 32 x 128 1.70 against 1.59: those stay where they were.
     const bool narrow = others && (D <= 32 || F <= 32);
+    // Chains too short for an exchange (fewer than 24 chunks) run here on any number of
+    // workgroups: the kernels that split L pay more for their exchange than a workgroup for
+    // walking the chain (64 x 64 forward, 8 chains, L=640: 19 against 27 us; 128 x 128 backward, 4
+    // chains, L=512: 29 against 62).  A single scan on the bf16-piece kernel, and its scans with
+    // half of the consumers idle, only up to 8 chunks (128 x 128 forward, 2 chains, L=256: 16
+    // against 17, L=512: 22 against 17; 128 x 32 forward, 8 chains, L=512: 27 against 20).
+    const int64_t brief_chunks = D <= 64 || (F > 32 && nscans >= 2) ? 23 : 8;
     if (narrow && D <= 32 && F <= 32) return;
     // A single scan over bf16 rows in blocks of 64 output columns reads a and b once per block:
     // beyond two rounds of workgroups, or one for a state of 32 rows, the kernels that split L
@@ -251,7 +260,9 @@ void tp_plan_compute(int64_t D, int64_t F, int64_t chains, int nscans, int64_t L
         int64_t least = 64, brief = lone_slab ? 16 : 32;
         // (the kernels that split L run 96 columns as slices: 32 x 96, 16 chains, L=2048: 44 / 73)
         if (D <= 32 && F == 96) least = 32, brief = 64;
-        if (units < (lone_slab ? 256 : 128) && !(units >= least && total_chunks <= brief)) return;
+        if (total_chunks > brief_chunks && units < (lone_slab ? 256 : 128) &&
+            !(units >= least && total_chunks <= brief))
+            return;
     }
     if (!forced && D <= 64 && F <= 64 && units > 512 && L <= 2 * kChunk) return;
     // fp32 64 x 64 chains of 257 to 1024 chunks on 112 workgroups or more are walked whole: a
@@ -312,7 +323,7 @@ void tp_plan_compute(int64_t D, int64_t F, int64_t chains, int nscans, int64_t L
                                : chunks >= 8        ? (nscans == 3 ? 2304 : 768)
                                                     : 512;
     if (*seg_chunks == 0)
-        *nseg = tp_kernel_segments(units, L, wide, others, long_chains, narrow, most_units);
+        *nseg = tp_kernel_segments(units, L, wide, others, long_chains, narrow, most_units, brief_chunks);
 }
 
 // workspace of the exchange: control block, then two state slots (own sum, group total) of

@@ -2,7 +2,7 @@
 
     python -m fast_transformers_amd.plan_check [--widths 64x64,32x128] [--dtype f32|bf16]
                                                [--chains 4,16,64,256,1024] [--lengths 256,...]
-                                               [--margin 0.07] [--quick]
+                                               [--margin 0.07] [--min-rows R] [--max-rows R] [--quick]
 
 Which kernel runs a launch is decided on the host from the sizes alone (csrc/ftc_mfma.hip), by
 rules whose thresholds were measured.  This tool measures them again: for every shape of the
@@ -38,6 +38,7 @@ def parse_args(argv=None):
     ap.add_argument("--lengths", default="256,1024,4096,16384,65536", help="values of L")
     ap.add_argument("--margin", type=float, default=0.07)
     ap.add_argument("--max-rows", type=int, default=1 << 21, help="skip shapes with more chains * L")
+    ap.add_argument("--min-rows", type=int, default=1 << 14, help="skip shapes with fewer chains * L")
     ap.add_argument("--quick", action="store_true", help="64x64 only, three chain counts")
     a = ap.parse_args(argv)
     if a.quick:
@@ -52,7 +53,7 @@ def shapes(a):
     for E, M in a.widths:
         for chains in a.chains:
             for L in a.lengths:
-                if 1 << 14 <= chains * L <= a.max_rows:
+                if a.min_rows <= chains * L <= a.max_rows:
                     yield E, M, chains, L
 
 

@@ -88,7 +88,10 @@ def test_what_the_chain_parallel_kernel_leaves_to_the_others():
     # the kernels that split L where it would need an exchange)
     assert lines((10, 8, 1000, 32), (10, 8, 1000, 128))[0].startswith("scan_tph_kernel:")
     assert lines((4, 16, 16384, 32), (4, 16, 16384, 128))[0].startswith("scan_dma_kernel")
-    assert lines((1, 3, 500, 128), (1, 3, 500, 128))[0].startswith("scan_mfma_kernel")  # few chains
+    # few chains too short for an exchange: cut or whole on the chain-parallel kernel all the same
+    assert lines((1, 3, 500, 128), (1, 3, 500, 128))[0].startswith("scan_mfma_kernel")
+    assert lines((1, 3, 500, 128), (1, 3, 500, 128), backward=True)[0].startswith("scan_tp_kernel: 3 scans")
+    assert lines((1, 8, 640, 64), (1, 8, 640, 64))[0].startswith("scan_tph_kernel: 1 scan")
     # bf16 rows: a single scan stays with the kernels that multiply such rows as they are
     # until the chain-parallel kernel has workgroups for about half of the CUs, and wherever
     # it would need an exchange; the three scans of a backward call, and widths that those
@@ -209,6 +212,9 @@ def test_wide_states_on_the_chain_parallel_kernel():
     # few chains: shapes that the kernels which split L also take go to those below half
     # the CUs, the others go to the chain-parallel kernel at any size
     assert lines((1, 8, 512, 128), (1, 8, 512, 128))[0].startswith("scan_mfma_kernel")
+    assert lines((1, 8, 256, 128), (1, 8, 256, 128))[0].startswith("scan_tp_kernel: 1 scan")
+    assert lines((1, 8, 512, 128), (1, 8, 512, 128), backward=True)[0].startswith("scan_tp_kernel: 3 scans")
+    assert lines((1, 40, 16384, 128), (1, 40, 16384, 32))[0].startswith("scan_mfma_kernel")
     # ... unless four or more segments of every chain fit one round of workgroups: an exchange
     # from 24 chunks on, in segments of down to four chunks
     few = lines((1, 8, 2048, 128), (1, 8, 2048, 128))[0]
